@@ -1,0 +1,311 @@
+"""ctypes binding of libae_hip.so (C ABI declared in include/ae_hip.h).
+
+This is the only place Python touches the native boundary.  It stands where the reference
+calls ``tl.compile(...)`` on a rendered template
+(attention_engine/core/template/tl_template/attn/attn_tl.py:523-528) or JIT-builds its CuTe
+extension (core/template/cute_template/flash_attn_interface.py:136-147).
+
+There is no CPU fallback: if the shared library is missing, or a launch is requested without
+a GPU, the calls raise.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import hashlib
+import os
+import os.path as osp
+import threading
+
+_PKG_ROOT = osp.dirname(osp.dirname(osp.dirname(osp.abspath(__file__))))
+CSRC_DIR = osp.join(_PKG_ROOT, "csrc")
+KERNEL_DIR = osp.join(CSRC_DIR, "kernels")
+INCLUDE_DIR = osp.join(osp.dirname(_PKG_ROOT), "include")
+LIB_PATH = osp.join(CSRC_DIR, "libae_hip.so")
+
+AE_MAX_ROWSCALES = 4
+AE_MAX_CUSTOM = 4
+
+# Options every kernel is compiled with.  Infinities stay meaningful (masks are additive
+# -inf), so no -ffast-math / -ffinite-math-only.  Packed-fp32 instruction selection is
+# switched off on purpose (scalar fp32 code only).
+COMPILE_OPTS = [
+    "-O3",
+    "-std=c++17",
+    "-fno-math-errno", "-fno-trapping-math", "-fno-signed-zeros", "-freciprocal-math",
+    "-ffp-contract=fast",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+class AEError(RuntimeError):
+    """A call into libae_hip.so returned a non-zero status."""
+
+
+class AttnParams(C.Structure):
+    """Mirror of ``ae_attn_params``."""
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("out", C.c_void_p),
+        ("rowscale_out", C.c_void_p * AE_MAX_ROWSCALES),
+        ("custom", C.c_void_p * AE_MAX_CUSTOM),
+        ("block_mask", C.c_void_p),
+        ("partial_o", C.c_void_p), ("partial_rs", C.c_void_p),
+        ("q2", C.c_void_p), ("k2", C.c_void_p),
+        ("q_stride_b", C.c_int64), ("q_stride_s", C.c_int64), ("q_stride_h", C.c_int64),
+        ("k_stride_b", C.c_int64), ("k_stride_s", C.c_int64), ("k_stride_h", C.c_int64),
+        ("v_stride_b", C.c_int64), ("v_stride_s", C.c_int64), ("v_stride_h", C.c_int64),
+        ("o_stride_b", C.c_int64), ("o_stride_s", C.c_int64), ("o_stride_h", C.c_int64),
+        ("q2_stride_b", C.c_int64), ("q2_stride_s", C.c_int64), ("q2_stride_h", C.c_int64),
+        ("k2_stride_b", C.c_int64), ("k2_stride_s", C.c_int64), ("k2_stride_h", C.c_int64),
+        ("batch", C.c_int32), ("heads_q", C.c_int32), ("heads_kv", C.c_int32),
+        ("seqlen_q", C.c_int32), ("seqlen_kv", C.c_int32),
+        ("mask_b", C.c_int32), ("mask_h", C.c_int32), ("mask_nq", C.c_int32), ("mask_nkv", C.c_int32),
+        ("mask_block_m", C.c_int32), ("mask_block_n", C.c_int32),
+        ("num_splits", C.c_int32), ("kv_per_split", C.c_int32),
+        ("reserved", C.c_int32 * 3),
+    ]
+
+
+class TileCfg(C.Structure):
+    """Mirror of ``ae_tile_cfg``."""
+    _fields_ = [
+        ("block_m", C.c_int32), ("block_n", C.c_int32), ("threads", C.c_int32),
+        ("lds_bytes", C.c_int32), ("head_dim", C.c_int32), ("head_dim_v", C.c_int32),
+        ("elem_bytes", C.c_int32), ("n_rowscales", C.c_int32), ("mask_mode", C.c_int32),
+        ("reserved", C.c_int32 * 3),
+    ]
+
+
+class DevInfo(C.Structure):
+    """Mirror of ``ae_devinfo``."""
+    _fields_ = [
+        ("name", C.c_char * 128), ("arch", C.c_char * 64),
+        ("compute_units", C.c_int32), ("clock_khz", C.c_int32), ("mem_clock_khz", C.c_int32),
+        ("mem_bus_bits", C.c_int32), ("lds_per_block", C.c_int32), ("l2_bytes", C.c_int32),
+        ("wavefront_size", C.c_int32), ("reserved", C.c_int32),
+        ("global_mem_bytes", C.c_uint64),
+    ]
+
+
+# every symbol include/ae_hip.h declares: name -> (restype, argtypes)
+_VP = C.c_void_p
+_SIGNATURES = {
+    "ae_abi_version": (C.c_int, []),
+    "ae_last_error": (C.c_char_p, []),
+    "ae_device_count": (C.c_int, []),
+    "ae_device_info": (C.c_int, [C.c_int, C.POINTER(DevInfo)]),
+    "ae_compile": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int,
+                             C.POINTER(C.c_char_p), C.POINTER(C.c_char_p), C.c_int, C.POINTER(_VP)]),
+    "ae_module_log": (C.c_char_p, [_VP]),
+    "ae_module_code": (C.c_int, [_VP, C.POINTER(_VP), C.POINTER(C.c_size_t)]),
+    "ae_module_save": (C.c_int, [_VP, C.c_char_p]),
+    "ae_module_load": (C.c_int, [C.c_char_p, C.POINTER(_VP)]),
+    "ae_module_free": (None, [_VP]),
+    "ae_module_get_kernel": (C.c_int, [_VP, C.c_char_p, C.POINTER(_VP)]),
+    "ae_launch": (C.c_int, [_VP, _VP, C.c_size_t, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32),
+                            C.c_uint32, _VP]),
+    "ae_prefill_fwd": (C.c_int, [_VP, C.POINTER(AttnParams), C.POINTER(TileCfg), _VP]),
+    "ae_decode_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
+                                C.POINTER(TileCfg), _VP]),
+    "ae_event_create": (C.c_int, [C.POINTER(_VP)]),
+    "ae_event_record": (C.c_int, [_VP, _VP]),
+    "ae_event_elapsed_ms": (C.c_int, [_VP, _VP, C.POINTER(C.c_float)]),
+    "ae_event_destroy": (None, [_VP]),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib = None
+_lib_lock = threading.Lock()
+
+
+def lib():
+    """Load libae_hip.so once; raise if it has not been built (no fallback)."""
+    global _lib
+    if _lib is None:
+        with _lib_lock:
+            if _lib is None:
+                if not osp.exists(LIB_PATH):
+                    raise AEError(
+                        f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; "
+                        "g.build()'` (or attentionengine_amd/csrc/build.py)")
+                handle = C.CDLL(LIB_PATH)
+                for name, (res, args) in _SIGNATURES.items():
+                    fn = getattr(handle, name)
+                    fn.restype = res
+                    fn.argtypes = args
+                _lib = handle
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise AEError(f"[ae status {rc}] " + lib().ae_last_error().decode("utf-8", "replace"))
+
+
+def device_count() -> int:
+    return lib().ae_device_count()
+
+
+def device_info(device: int = 0) -> dict:
+    info = DevInfo()
+    _check(lib().ae_device_info(device, C.byref(info)))
+    out = {f: getattr(info, f) for f, _ in DevInfo._fields_ if f != "reserved"}
+    out["name"] = info.name.decode()
+    out["arch"] = info.arch.decode()
+    return out
+
+
+def cache_dir() -> str:
+    """Directory of cached code objects (the reference caches rendered source under
+    attn_engine/cache/<md5>.py, attn_engine.py:369-375)."""
+    d = os.environ.get("AE_CACHE_DIR") or osp.join(_PKG_ROOT, "_cache")
+    try:
+        os.makedirs(d, exist_ok=True)
+        if not os.access(d, os.W_OK):
+            raise OSError
+    except OSError:
+        d = osp.join(osp.expanduser("~"), ".cache", "attentionengine_amd")
+        os.makedirs(d, exist_ok=True)
+    return d
+
+
+def _read(path):
+    with open(path, "r") as f:
+        return f.read()
+
+
+class Kernel:
+    """A kernel of a loaded module, bound to the device it was loaded on."""
+
+    def __init__(self, module: "Module", name: str):
+        self.module = module
+        self.name = name
+        h = _VP()
+        _check(lib().ae_module_get_kernel(module.handle, name.encode(), C.byref(h)))
+        self.handle = h
+
+    def launch(self, params: C.Structure, grid, block, lds_bytes: int, stream: int = 0):
+        g = (C.c_uint32 * 3)(*grid)
+        b = (C.c_uint32 * 3)(*block)
+        _check(lib().ae_launch(self.handle, C.byref(params), C.sizeof(params), g, b, lds_bytes,
+                               _VP(stream)))
+
+
+class Module:
+    """A compiled code object.  Compilation needs no GPU; ``kernel()`` does."""
+
+    def __init__(self, handle, source_key: str, from_cache: bool):
+        self.handle = handle
+        self.key = source_key
+        self.from_cache = from_cache
+        self._kernels = {}
+
+    @property
+    def log(self) -> str:
+        return lib().ae_module_log(self.handle).decode("utf-8", "replace")
+
+    def code(self) -> bytes:
+        data, size = _VP(), C.c_size_t()
+        _check(lib().ae_module_code(self.handle, C.byref(data), C.byref(size)))
+        return C.string_at(data, size.value)
+
+    def kernel(self, name: str) -> Kernel:
+        k = self._kernels.get(name)
+        if k is None:
+            k = self._kernels[name] = Kernel(self, name)
+        return k
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().ae_module_free(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+_modules = {}
+_modules_lock = threading.Lock()
+
+
+def compile_module(template: str, headers: dict, arch: str = None, use_cache: bool = True) -> Module:
+    """Compile kernel template ``template`` (a file name under csrc/kernels) with the generated
+    in-memory ``headers`` ({"ae_config.h": text, "ae_functors.h": text}).
+
+    The code object is cached on disk under a key that covers the template text, every header,
+    the architecture and the compiler options, and in memory for the life of the process.
+    """
+    arch = arch or os.environ.get("AE_HIP_ARCH", "gfx950")
+    src = _read(osp.join(KERNEL_DIR, template))
+    all_headers = {
+        "ae_hip.h": _read(osp.join(INCLUDE_DIR, "ae_hip.h")),
+        "ae_device.h": _read(osp.join(KERNEL_DIR, "ae_device.h")),
+    }
+    all_headers.update(headers)
+    hsh = hashlib.sha256()
+    for part in [template, src, arch, " ".join(COMPILE_OPTS)]:
+        hsh.update(part.encode())
+        hsh.update(b"\0")
+    for name in sorted(all_headers):
+        hsh.update(name.encode() + b"\0" + all_headers[name].encode() + b"\0")
+    key = hsh.hexdigest()[:32]
+    with _modules_lock:
+        m = _modules.get(key)
+        if m is not None:
+            return m
+        path = osp.join(cache_dir(), f"{osp.splitext(template)[0]}_{key}.hsaco")
+        handle = _VP()
+        if use_cache and osp.exists(path):
+            _check(lib().ae_module_load(path.encode(), C.byref(handle)))
+            m = Module(handle, key, True)
+        else:
+            names = list(all_headers)
+            n = len(names)
+            c_names = (C.c_char_p * n)(*[s.encode() for s in names])
+            c_srcs = (C.c_char_p * n)(*[all_headers[s].encode() for s in names])
+            c_opts = (C.c_char_p * len(COMPILE_OPTS))(*[o.encode() for o in COMPILE_OPTS])
+            _check(lib().ae_compile(src.encode(), template.encode(), arch.encode(), c_opts,
+                                    len(COMPILE_OPTS), c_names, c_srcs, n, C.byref(handle)))
+            m = Module(handle, key, False)
+            if use_cache:
+                try:
+                    _check(lib().ae_module_save(handle, path.encode()))
+                except AEError:
+                    pass  # an unwritable cache only costs a recompile next time
+        _modules[key] = m
+        return m
+
+
+class Event:
+    """HIP event recorded on the stream the kernels are launched on."""
+
+    def __init__(self):
+        h = _VP()
+        _check(lib().ae_event_create(C.byref(h)))
+        self.handle = h
+
+    def record(self, stream: int = 0):
+        _check(lib().ae_event_record(self.handle, _VP(stream)))
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        _check(lib().ae_event_elapsed_ms(self.handle, stop.handle, C.byref(ms)))
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().ae_event_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def prefill_fwd(kernel: Kernel, params: AttnParams, cfg: TileCfg, stream: int = 0):
+    _check(lib().ae_prefill_fwd(kernel.handle, C.byref(params), C.byref(cfg), _VP(stream)))
+
+
+def decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
+               combine_cfg: TileCfg, stream: int = 0):
+    _check(lib().ae_decode_fwd(split.handle, combine.handle if combine else None, C.byref(params),
+                               C.byref(cfg), C.byref(combine_cfg) if combine_cfg else None,
+                               _VP(stream)))

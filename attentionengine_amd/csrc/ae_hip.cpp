@@ -1,0 +1,399 @@
+// libae_hip.so: hipRTC compile + code-object cache + checked launches behind a C ABI.
+// Declarations and the reference interfaces they stand in for: include/ae_hip.h.
+//
+// Host-only translation unit (built with g++ or hipcc); links libamdhip64 + libhiprtc.
+
+#include "ae_hip.h"
+
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_last_error;
+std::mutex g_mutex;  // guards compilation and module load/unload
+
+int fail(int code, const char* fmt, ...) {
+  char buf[4096];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int fail_str(int code, const std::string& s) {
+  g_last_error = s;
+  return code;
+}
+
+#define AE_HIP_TRY(expr)                                                           \
+  do {                                                                             \
+    hipError_t e_ = (expr);                                                        \
+    if (e_ != hipSuccess)                                                          \
+      return fail(AE_ERR_HIP, "%s failed: %s (%d)", #expr, hipGetErrorString(e_),  \
+                  (int)e_);                                                        \
+  } while (0)
+
+}  // namespace
+
+struct ae_kernel {
+  hipFunction_t fn = nullptr;
+  int device = -1;
+  std::string name;
+};
+
+struct ae_module {
+  std::vector<char> code;
+  std::string log;
+  std::string name;
+  // one loaded hipModule_t per device, created on demand
+  std::map<int, hipModule_t> loaded;
+  std::map<std::pair<int, std::string>, ae_kernel*> kernels;
+};
+
+struct ae_event {
+  hipEvent_t ev = nullptr;
+};
+
+extern "C" {
+
+int ae_abi_version(void) { return AE_ABI_VERSION; }
+
+const char* ae_last_error(void) { return g_last_error.c_str(); }
+
+int ae_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+int ae_device_info(int device, ae_devinfo* out) {
+  if (!out) return fail(AE_ERR_INVALID_ARG, "ae_device_info: out is NULL");
+  hipDeviceProp_t pr;
+  AE_HIP_TRY(hipGetDeviceProperties(&pr, device));
+  memset(out, 0, sizeof *out);
+  snprintf(out->name, sizeof out->name, "%.127s", pr.name);
+  snprintf(out->arch, sizeof out->arch, "%.63s", pr.gcnArchName);
+  out->compute_units = pr.multiProcessorCount;
+  out->clock_khz = pr.clockRate;
+  out->mem_clock_khz = pr.memoryClockRate;
+  out->mem_bus_bits = pr.memoryBusWidth;
+  out->lds_per_block = (int32_t)pr.sharedMemPerBlock;
+  out->l2_bytes = pr.l2CacheSize;
+  out->wavefront_size = pr.warpSize;
+  out->global_mem_bytes = pr.totalGlobalMem;
+  return AE_OK;
+}
+
+int ae_compile(const char* src, const char* name, const char* arch,
+               const char* const* opts, int nopts,
+               const char* const* header_names, const char* const* headers, int nheaders,
+               ae_module** out) {
+  if (out) *out = nullptr;
+  if (!src || !out) return fail(AE_ERR_INVALID_ARG, "ae_compile: src/out is NULL");
+  if (nopts < 0 || nheaders < 0 || (nopts && !opts) ||
+      (nheaders && (!headers || !header_names)))
+    return fail(AE_ERR_INVALID_ARG, "ae_compile: bad option/header arrays");
+  std::lock_guard<std::mutex> lock(g_mutex);
+
+  hiprtcProgram prog = nullptr;
+  hiprtcResult r = hiprtcCreateProgram(&prog, src, name ? name : "ae_kernel.hip", nheaders,
+                                       const_cast<const char**>(headers),
+                                       const_cast<const char**>(header_names));
+  if (r != HIPRTC_SUCCESS)
+    return fail(AE_ERR_COMPILE, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+
+  std::vector<std::string> held;
+  held.push_back(std::string("--offload-arch=") + (arch && *arch ? arch : "gfx950"));
+  for (int i = 0; i < nopts; i++)
+    if (opts[i]) held.push_back(opts[i]);
+  std::vector<const char*> argv;
+  for (auto& s : held) argv.push_back(s.c_str());
+
+  r = hiprtcCompileProgram(prog, (int)argv.size(), argv.data());
+  std::string log;
+  size_t log_size = 0;
+  if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1) {
+    log.resize(log_size);
+    if (hiprtcGetProgramLog(prog, &log[0]) != HIPRTC_SUCCESS) log.clear();
+    while (!log.empty() && log.back() == '\0') log.pop_back();
+  }
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    return fail_str(AE_ERR_COMPILE, std::string("hipRTC compile failed (") +
+                                        hiprtcGetErrorString(r) + "):\n" + log);
+  }
+  size_t code_size = 0;
+  r = hiprtcGetCodeSize(prog, &code_size);
+  if (r != HIPRTC_SUCCESS || code_size == 0) {
+    hiprtcDestroyProgram(&prog);
+    return fail(AE_ERR_COMPILE, "hiprtcGetCodeSize: %s", hiprtcGetErrorString(r));
+  }
+  ae_module* m = new ae_module();
+  m->code.resize(code_size);
+  r = hiprtcGetCode(prog, m->code.data());
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS) {
+    delete m;
+    return fail(AE_ERR_COMPILE, "hiprtcGetCode: %s", hiprtcGetErrorString(r));
+  }
+  m->log = log;
+  m->name = name ? name : "";
+  *out = m;
+  return AE_OK;
+}
+
+const char* ae_module_log(const ae_module* m) { return m ? m->log.c_str() : ""; }
+
+int ae_module_code(const ae_module* m, const void** data, size_t* size) {
+  if (!m || !data || !size) return fail(AE_ERR_INVALID_ARG, "ae_module_code: NULL argument");
+  *data = m->code.data();
+  *size = m->code.size();
+  return AE_OK;
+}
+
+int ae_module_save(const ae_module* m, const char* path) {
+  if (!m || !path) return fail(AE_ERR_INVALID_ARG, "ae_module_save: NULL argument");
+  // write to a temporary name first so a concurrent reader never sees a torn file
+  std::string tmp = std::string(path) + ".tmp";
+  FILE* f = fopen(tmp.c_str(), "wb");
+  if (!f) return fail(AE_ERR_IO, "ae_module_save: cannot open %s", tmp.c_str());
+  size_t n = fwrite(m->code.data(), 1, m->code.size(), f);
+  int rc = fclose(f);
+  if (n != m->code.size() || rc != 0) {
+    remove(tmp.c_str());
+    return fail(AE_ERR_IO, "ae_module_save: short write to %s", tmp.c_str());
+  }
+  if (rename(tmp.c_str(), path) != 0) {
+    remove(tmp.c_str());
+    return fail(AE_ERR_IO, "ae_module_save: cannot rename to %s", path);
+  }
+  return AE_OK;
+}
+
+int ae_module_load(const char* path, ae_module** out) {
+  if (out) *out = nullptr;
+  if (!path || !out) return fail(AE_ERR_INVALID_ARG, "ae_module_load: NULL argument");
+  FILE* f = fopen(path, "rb");
+  if (!f) return fail(AE_ERR_IO, "ae_module_load: cannot open %s", path);
+  fseek(f, 0, SEEK_END);
+  long sz = ftell(f);
+  fseek(f, 0, SEEK_SET);
+  if (sz <= 0) {
+    fclose(f);
+    return fail(AE_ERR_IO, "ae_module_load: %s is empty", path);
+  }
+  ae_module* m = new ae_module();
+  m->code.resize((size_t)sz);
+  size_t n = fread(m->code.data(), 1, (size_t)sz, f);
+  fclose(f);
+  if (n != (size_t)sz) {
+    delete m;
+    return fail(AE_ERR_IO, "ae_module_load: short read from %s", path);
+  }
+  m->name = path;
+  *out = m;
+  return AE_OK;
+}
+
+void ae_module_free(ae_module* m) {
+  if (!m) return;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  for (auto& kv : m->kernels) delete kv.second;
+  for (auto& kv : m->loaded) {
+    if (kv.second) (void)hipModuleUnload(kv.second);
+  }
+  delete m;
+}
+
+int ae_module_get_kernel(ae_module* m, const char* kernel_name, ae_kernel** out) {
+  if (out) *out = nullptr;
+  if (!m || !kernel_name || !out)
+    return fail(AE_ERR_INVALID_ARG, "ae_module_get_kernel: NULL argument");
+  std::lock_guard<std::mutex> lock(g_mutex);
+  int dev = -1;
+  AE_HIP_TRY(hipGetDevice(&dev));
+  auto key = std::make_pair(dev, std::string(kernel_name));
+  auto it = m->kernels.find(key);
+  if (it != m->kernels.end()) {
+    *out = it->second;
+    return AE_OK;
+  }
+  hipModule_t mod = nullptr;
+  auto lit = m->loaded.find(dev);
+  if (lit == m->loaded.end()) {
+    AE_HIP_TRY(hipModuleLoadData(&mod, m->code.data()));
+    m->loaded[dev] = mod;
+  } else {
+    mod = lit->second;
+  }
+  hipFunction_t fn = nullptr;
+  hipError_t e = hipModuleGetFunction(&fn, mod, kernel_name);
+  if (e != hipSuccess || !fn)
+    return fail(AE_ERR_NOT_FOUND, "kernel '%s' not found in module '%s': %s", kernel_name,
+                m->name.c_str(), hipGetErrorString(e));
+  ae_kernel* k = new ae_kernel();
+  k->fn = fn;
+  k->device = dev;
+  k->name = kernel_name;
+  m->kernels[key] = k;
+  *out = k;
+  return AE_OK;
+}
+
+int ae_launch(ae_kernel* k, const void* params, size_t params_bytes, const uint32_t grid[3],
+              const uint32_t block[3], uint32_t lds_bytes, void* stream) {
+  if (!k || !k->fn || !grid || !block)
+    return fail(AE_ERR_INVALID_ARG, "ae_launch: NULL kernel/grid/block");
+  if (params_bytes && !params) return fail(AE_ERR_INVALID_ARG, "ae_launch: params is NULL");
+  for (int i = 0; i < 3; i++)
+    if (grid[i] == 0 || block[i] == 0)
+      return fail(AE_ERR_INVALID_ARG, "ae_launch: zero grid/block extent");
+  uint64_t threads = (uint64_t)block[0] * block[1] * block[2];
+  if (threads > 1024) return fail(AE_ERR_INVALID_ARG, "ae_launch: %llu threads per block",
+                                  (unsigned long long)threads);
+  if (lds_bytes > 160u * 1024u)
+    return fail(AE_ERR_INVALID_ARG, "ae_launch: %u bytes of LDS exceed 160 KiB", lds_bytes);
+  size_t size = params_bytes;
+  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(params),
+                    HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+  AE_HIP_TRY(hipModuleLaunchKernel(k->fn, grid[0], grid[1], grid[2], block[0], block[1],
+                                   block[2], lds_bytes, (hipStream_t)stream, nullptr,
+                                   params_bytes ? config : nullptr));
+  return AE_OK;
+}
+
+static int check_common(const char* who, const ae_attn_params* p, const ae_tile_cfg* cfg) {
+  if (!p || !cfg) return fail(AE_ERR_INVALID_ARG, "%s: params/cfg is NULL", who);
+  if (!p->q || !p->k || !p->v || !p->out)
+    return fail(AE_ERR_INVALID_ARG, "%s: q/k/v/out pointer is NULL", who);
+  if (p->batch <= 0 || p->heads_q <= 0 || p->heads_kv <= 0 || p->seqlen_q <= 0 ||
+      p->seqlen_kv <= 0)
+    return fail(AE_ERR_INVALID_ARG, "%s: non-positive extent (B=%d Hq=%d Hkv=%d Sq=%d Skv=%d)",
+                who, p->batch, p->heads_q, p->heads_kv, p->seqlen_q, p->seqlen_kv);
+  if (p->heads_q % p->heads_kv != 0)
+    return fail(AE_ERR_INVALID_ARG, "%s: Hq=%d is not a multiple of Hkv=%d", who, p->heads_q,
+                p->heads_kv);
+  if (cfg->block_m <= 0 || cfg->block_n <= 0 || cfg->threads <= 0 || cfg->threads % 64 != 0 ||
+      cfg->threads > 1024 || cfg->lds_bytes < 0 || cfg->lds_bytes > 160 * 1024)
+    return fail(AE_ERR_INVALID_ARG, "%s: bad tile configuration (bm=%d bn=%d threads=%d lds=%d)",
+                who, cfg->block_m, cfg->block_n, cfg->threads, cfg->lds_bytes);
+  if (cfg->n_rowscales < 0 || cfg->n_rowscales > AE_MAX_ROWSCALES)
+    return fail(AE_ERR_INVALID_ARG, "%s: n_rowscales=%d out of range", who, cfg->n_rowscales);
+  if (cfg->mask_mode == 2) {
+    if (!p->block_mask) return fail(AE_ERR_INVALID_ARG, "%s: block-mask kernel without a mask", who);
+    if (p->mask_block_m <= 0 || p->mask_block_n <= 0 || p->mask_nq <= 0 || p->mask_nkv <= 0)
+      return fail(AE_ERR_INVALID_ARG, "%s: bad block-mask geometry", who);
+    if ((p->mask_b != 1 && p->mask_b != p->batch) || (p->mask_h != 1 && p->mask_h != p->heads_q))
+      return fail(AE_ERR_INVALID_ARG, "%s: block-mask batch/head extent (%d,%d) must be 1 or (B,Hq)",
+                  who, p->mask_b, p->mask_h);
+    if ((int64_t)p->mask_nq * p->mask_block_m < p->seqlen_q ||
+        (int64_t)p->mask_nkv * p->mask_block_n < p->seqlen_kv)
+      return fail(AE_ERR_INVALID_ARG, "%s: block mask [%d x %d] of %dx%d blocks does not cover %d x %d",
+                  who, p->mask_nq, p->mask_nkv, p->mask_block_m, p->mask_block_n, p->seqlen_q,
+                  p->seqlen_kv);
+  }
+  return AE_OK;
+}
+
+int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream) {
+  if (!k) return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: kernel is NULL");
+  int rc = check_common("ae_prefill_fwd", p, cfg);
+  if (rc) return rc;
+  for (int i = 0; i < cfg->n_rowscales; i++)
+    if (!p->rowscale_out[i])
+      return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: rowscale_out[%d] is NULL", i);
+  if (cfg->mask_mode == 2 && (cfg->block_m % p->mask_block_m != 0 && p->mask_block_m % cfg->block_m != 0))
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: mask block rows %d incompatible with tile %d",
+                p->mask_block_m, cfg->block_m);
+  uint64_t q_tiles = ((uint64_t)p->seqlen_q + cfg->block_m - 1) / cfg->block_m;
+  uint64_t total = q_tiles * (uint64_t)p->heads_q * (uint64_t)p->batch;
+  if (total == 0 || total > 0x7fffffffull)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: grid of %llu workgroups",
+                (unsigned long long)total);
+  uint32_t grid[3] = {(uint32_t)total, 1, 1};
+  uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
+  return ae_launch(k, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+}
+
+int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                  const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
+  if (!split) return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split kernel is NULL");
+  int rc = check_common("ae_decode_fwd", p, cfg);
+  if (rc) return rc;
+  if (p->seqlen_q != 1)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: seqlen_q=%d (decode handles one query token)",
+                p->seqlen_q);
+  if (p->num_splits <= 0 || p->kv_per_split <= 0 ||
+      (int64_t)p->num_splits * p->kv_per_split < p->seqlen_kv)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: %d splits of %d do not cover Skv=%d",
+                p->num_splits, p->kv_per_split, p->seqlen_kv);
+  if (p->kv_per_split % cfg->block_n != 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: kv_per_split=%d is not a multiple of block_n=%d",
+                p->kv_per_split, cfg->block_n);
+  if (!p->partial_o || !p->partial_rs)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
+  if (!combine || !combine_cfg)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel is NULL");
+  int group = p->heads_q / p->heads_kv;
+  int head_tiles = (group + cfg->block_m - 1) / cfg->block_m;
+  uint32_t grid[3] = {(uint32_t)p->num_splits, (uint32_t)(head_tiles * p->heads_kv),
+                      (uint32_t)p->batch};
+  uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
+  rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+  if (rc) return rc;
+  if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: bad combine workgroup size %d",
+                combine_cfg->threads);
+  for (int i = 0; i < combine_cfg->n_rowscales; i++)
+    if (!p->rowscale_out[i])
+      return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: rowscale_out[%d] is NULL", i);
+  uint32_t cgrid[3] = {(uint32_t)p->heads_q, (uint32_t)p->batch, 1};
+  uint32_t cblock[3] = {(uint32_t)combine_cfg->threads, 1, 1};
+  return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
+}
+
+int ae_event_create(ae_event** out) {
+  if (!out) return fail(AE_ERR_INVALID_ARG, "ae_event_create: out is NULL");
+  *out = nullptr;
+  hipEvent_t ev = nullptr;
+  AE_HIP_TRY(hipEventCreate(&ev));
+  ae_event* e = new ae_event();
+  e->ev = ev;
+  *out = e;
+  return AE_OK;
+}
+
+int ae_event_record(ae_event* e, void* stream) {
+  if (!e) return fail(AE_ERR_INVALID_ARG, "ae_event_record: event is NULL");
+  AE_HIP_TRY(hipEventRecord(e->ev, (hipStream_t)stream));
+  return AE_OK;
+}
+
+int ae_event_elapsed_ms(ae_event* start, ae_event* stop, float* ms) {
+  if (!start || !stop || !ms) return fail(AE_ERR_INVALID_ARG, "ae_event_elapsed_ms: NULL argument");
+  AE_HIP_TRY(hipEventSynchronize(stop->ev));
+  AE_HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return AE_OK;
+}
+
+void ae_event_destroy(ae_event* e) {
+  if (!e) return;
+  if (e->ev) (void)hipEventDestroy(e->ev);
+  delete e;
+}
+
+}  // extern "C"

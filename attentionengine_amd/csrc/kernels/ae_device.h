@@ -1,0 +1,136 @@
+// Device-side helpers shared by the gfx950 attention kernel templates.
+//
+// Element types, MFMA wrappers, the register layouts of the 32x32x16 MFMA accumulator and
+// the row reductions / transcendentals the generated functors call. The transcendental
+// definitions follow the reference's code generator (core/codegen/tl_gen.py:89-117):
+// exp(x) = exp2(x * log2 e), log(x) = log2(x) * ln 2, tanh via a fast approximation.
+#ifndef AE_DEVICE_H
+#define AE_DEVICE_H
+
+// hipRTC predefines the HIP device environment; an offline hipcc build has to include it.
+#ifndef __HIPCC_RTC__
+#include <hip/hip_runtime.h>
+#endif
+#include "ae_hip.h"
+
+#if AE_DTYPE_BF16
+typedef __bf16 ae_elem;
+#else
+typedef _Float16 ae_elem;
+#endif
+typedef ae_elem ae_elem8 __attribute__((ext_vector_type(8)));
+typedef ae_elem ae_elem4 __attribute__((ext_vector_type(4)));
+typedef ae_elem ae_elem2 __attribute__((ext_vector_type(2)));
+typedef float ae_f32x16 __attribute__((ext_vector_type(16)));
+typedef float ae_f32x4 __attribute__((ext_vector_type(4)));
+typedef short ae_s16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int ae_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int ae_u32x2 __attribute__((ext_vector_type(2)));
+
+#define AE_DEV __device__ inline __attribute__((always_inline))
+#define AE_NEG_INF (-__builtin_inff())
+#define AE_LOG2E 1.4426950408889634f
+#define AE_LN2 0.6931471805599453f
+
+// D[m][n] += sum_k A[m][k] B[k][n], 32x32 output, 16-deep. Lane l supplies A[l%32][8*(l/32)+j]
+// and B[8*(l/32)+j][l%32], j=0..7, and owns D[8*(r/4) + 4*(l/32) + r%4][l%32], r=0..15.
+AE_DEV ae_f32x16 ae_mfma32(ae_elem8 a, ae_elem8 b, ae_f32x16 c) {
+#if AE_DTYPE_BF16
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// D[m][n], 16x16 output, 32-deep. Lane l supplies A[l%16][8*(l/16)+j], B[8*(l/16)+j][l%16]
+// and owns D[4*(l/16) + r][l%16], r=0..3.
+AE_DEV ae_f32x4 ae_mfma16(ae_elem8 a, ae_elem8 b, ae_f32x4 c) {
+#if AE_DTYPE_BF16
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// ---- transcendentals ------------------------------------------------------------------
+AE_DEV float ae_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+AE_DEV float ae_exp(float x) { return __builtin_amdgcn_exp2f(x * AE_LOG2E); }
+AE_DEV float ae_log2(float x) { return __builtin_amdgcn_logf(x); }
+AE_DEV float ae_log(float x) { return __builtin_amdgcn_logf(x) * AE_LN2; }
+AE_DEV float ae_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+// tanh(x) = 1 - 2 / (exp(2x) + 1); saturates cleanly at +-1 for large |x|.
+AE_DEV float ae_tanh(float x) {
+  float e = __builtin_amdgcn_exp2f(x * (2.0f * AE_LOG2E));
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+AE_DEV float ae_abs(float x) { return __builtin_fabsf(x); }
+AE_DEV float ae_max(float a, float b) { return __builtin_fmaxf(a, b); }
+
+// ---- lane-pair exchange -----------------------------------------------------------------
+// In the transposed score layout one query row lives in lanes l and l^32. permlane32_swap
+// with both operands equal returns (value of the low half, value of the high half) in
+// every lane of the pair.
+AE_DEV float ae_pair_max(float v) {
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_fmaxf(__builtin_bit_cast(float, (unsigned)r[0]),
+                         __builtin_bit_cast(float, (unsigned)r[1]));
+}
+AE_DEV float ae_pair_sum(float v) {
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
+// ---- row reductions over the lane's slice of a score row + its partner lane ------------
+// (ReduceMax / ReduceSum / ReduceAbsSum over dim=1 of the [block_M, block_N] tile,
+//  core/codegen/tl_gen.py:9-21.)
+template <int N>
+AE_DEV float ae_row_max(const float (&s)[N]) {
+  float m = s[0];
+#pragma unroll
+  for (int e = 1; e < N; e++) m = __builtin_fmaxf(m, s[e]);
+  return ae_pair_max(m);
+}
+template <int N>
+AE_DEV float ae_row_sum(const float (&s)[N]) {
+  // four independent chains keep the adds off one dependency path
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+  for (int e = 0; e + 3 < N; e += 4) {
+    a0 += s[e];
+    a1 += s[e + 1];
+    a2 += s[e + 2];
+    a3 += s[e + 3];
+  }
+#pragma unroll
+  for (int e = N & ~3; e < N; e++) a0 += s[e];
+  return ae_pair_sum((a0 + a1) + (a2 + a3));
+}
+template <int N>
+AE_DEV float ae_row_abssum(const float (&s)[N]) {
+  float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int e = 0; e + 1 < N; e += 2) {
+    a0 += __builtin_fabsf(s[e]);
+    a1 += __builtin_fabsf(s[e + 1]);
+  }
+#pragma unroll
+  for (int e = N & ~1; e < N; e++) a0 += __builtin_fabsf(s[e]);
+  return ae_pair_sum(a0 + a1);
+}
+
+// Per-row context handed to the functors.
+struct ae_ctx {
+  int b;        // batch index
+  int h;        // query head index
+  int q_idx;    // absolute query position of this lane's row
+  int kv_base;  // absolute kv position of element 0 of the lane's slice in the current tile
+};
+
+// kv offset (relative to ae_ctx::kv_base) of element e of a lane's slice of a score row:
+// the slice is NB accumulator blocks of 16; block nb covers kv 32*nb .. 32*nb+31 and
+// register r of the half-wave hf holds kv 8*(r/4) + 4*hf + r%4 (hf is folded into kv_base).
+AE_DEV constexpr int ae_kv_off(int e) { return (e >> 4) * 32 + ((e & 15) >> 2) * 8 + (e & 3); }
+
+#endif  // AE_DEVICE_H

@@ -1,0 +1,195 @@
+/*
+ * ae_hip.h -- C ABI of libae_hip.so, the native boundary of the MI355X (gfx950)
+ * attention-forward path.
+ *
+ * What it replaces in the reference (microsoft/AttentionEngine):
+ *   - the TileLang JIT boundary `tl.compile(prim_func, out_idx=[...])` that turns a
+ *     rendered kernel template into a callable
+ *     (attention_engine/core/template/tl_template/attn/attn_tl.py:523-528, 567-580;
+ *      attn_gqa_decode_tl.py:338-349; mla_decode_tl.py:326-335), and
+ *   - the pybind11 torch extensions of the CuTe backend, `fwd(...)`
+ *     (core/template/cute_template/flash_api.cpp:283-467, 694-697) and
+ *     `fwd_kvcache_mla(...)`
+ *     (core/template/cute_template_kvshared/flash_api.cpp:61-210, 212-216).
+ *
+ * Conventions
+ *   - plain C: pointers, sizes and PODs only; no torch, no C++ types, no exceptions.
+ *   - every function returns 0 on success and a non-zero ae_status otherwise; the text
+ *     of the last error of the calling thread is available from ae_last_error().
+ *     Nothing in the library calls exit()/abort().
+ *   - the caller owns every tensor and allocates all outputs and split-KV work
+ *     buffers before a launch; device pointers are passed inside ae_attn_params
+ *     together with their strides in ELEMENTS (the layout of Flash_fwd_params,
+ *     core/template/cute_template/flash.h:14-60, reduced to what the forward needs).
+ *   - launches are asynchronous on the caller's HIP stream (`void* stream` is a
+ *     hipStream_t; NULL is the default stream). The library never synchronises the
+ *     device except inside ae_event_elapsed_ms().
+ *   - compilation (ae_compile) needs no GPU: hipRTC cross-compiles for `arch`.
+ *     Loading a code object onto a device happens lazily in ae_module_get_kernel().
+ *   - ae_compile / ae_module_* are serialised by an internal mutex; launches take no
+ *     lock and may be issued from any thread whose current device matches the one the
+ *     kernel was loaded on.
+ */
+#ifndef AE_HIP_H
+#define AE_HIP_H
+
+/* hipRTC supplies the fixed-width integer types itself and has no libc headers. */
+#ifndef __HIPCC_RTC__
+#include <stddef.h>
+#include <stdint.h>
+#else
+using __hip_internal::int8_t;
+using __hip_internal::int32_t;
+using __hip_internal::int64_t;
+using __hip_internal::uint32_t;
+using __hip_internal::uint64_t;
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AE_ABI_VERSION 1
+
+typedef enum ae_status {
+  AE_OK = 0,
+  AE_ERR_INVALID_ARG = 1,   /* NULL pointer, bad size, shape/tile mismatch        */
+  AE_ERR_COMPILE = 2,       /* hipRTC rejected the source; see ae_module-less log  */
+  AE_ERR_HIP = 3,           /* a HIP runtime call failed (no device, load, launch) */
+  AE_ERR_IO = 4,            /* code-object cache file could not be read/written    */
+  AE_ERR_NOT_FOUND = 5      /* kernel symbol missing from the module               */
+} ae_status;
+
+typedef struct ae_module ae_module; /* a compiled code object (host memory)        */
+typedef struct ae_kernel ae_kernel; /* a function of a module loaded on one device  */
+
+/* Maximum counts baked into ae_attn_params. */
+#define AE_MAX_ROWSCALES 4
+#define AE_MAX_CUSTOM 4
+
+/*
+ * Kernel argument block shared by the prefill, split-KV decode and combine kernels.
+ * Passed BY VALUE as the single kernel parameter. Runtime tensors use the reference's
+ * layouts: q [B,Sq,Hq,D], k [B,Skv,Hkv,D], v [B,Skv,Hkv,DV], out [B,Sq,Hq,DV]
+ * (attention_engine/attn_engine/attn_engine.py:388-395; attn_tl.py:82-84), final
+ * rowscales fp32 [B,Hq,Sq] (core/lower/lower.py:385-392).
+ */
+typedef struct ae_attn_params {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* rowscale_out[AE_MAX_ROWSCALES]; /* final rowscales, fp32 [B,Hq,Sq]; may be NULL */
+  const void* custom[AE_MAX_CUSTOM];     /* CustomIO tensors in dict order                */
+  const int8_t* block_mask;              /* [mask_b,mask_h,mask_nq,mask_nkv] int8 or NULL */
+  float* partial_o;                      /* decode: fp32 [B,Hq,splits,DV]                 */
+  float* partial_rs;                     /* decode: fp32 [nrowscales,B,Hq,splits]         */
+  const void* q2;                        /* MLA: rope part of q  [B,Sq,Hq,D2] or NULL     */
+  const void* k2;                        /* MLA: rope part of k  [B,Skv,Hkv,D2] or NULL   */
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t q2_stride_b, q2_stride_s, q2_stride_h;
+  int64_t k2_stride_b, k2_stride_s, k2_stride_h;
+  int32_t batch, heads_q, heads_kv, seqlen_q, seqlen_kv;
+  int32_t mask_b, mask_h, mask_nq, mask_nkv; /* block-mask extents (mask_b/h may be 1)   */
+  int32_t mask_block_m, mask_block_n;        /* rows/cols one block-mask entry covers     */
+  int32_t num_splits;                        /* decode: KV splits per (batch, q-head)     */
+  int32_t kv_per_split;                      /* decode: KV positions per split            */
+  int32_t reserved[3];
+} ae_attn_params;
+
+/* Static facts of one compiled kernel instance, filled by the code generator. */
+typedef struct ae_tile_cfg {
+  int32_t block_m;     /* q rows per workgroup (prefill) / q-heads per workgroup (decode) */
+  int32_t block_n;     /* kv positions per inner tile                                     */
+  int32_t threads;     /* workgroup size, a multiple of 64                                */
+  int32_t lds_bytes;   /* dynamic LDS per workgroup                                       */
+  int32_t head_dim;    /* D (for MLA: latent + rope)                                      */
+  int32_t head_dim_v;  /* DV                                                              */
+  int32_t elem_bytes;  /* 2 for fp16/bf16                                                 */
+  int32_t n_rowscales; /* number of final rowscales the kernel writes                     */
+  int32_t mask_mode;   /* 0 none, 1 analytic causal, 2 block table                        */
+  int32_t reserved[3];
+} ae_tile_cfg;
+
+typedef struct ae_devinfo {
+  char name[128];
+  char arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
+  int32_t compute_units;
+  int32_t clock_khz;
+  int32_t mem_clock_khz;
+  int32_t mem_bus_bits;
+  int32_t lds_per_block;
+  int32_t l2_bytes;
+  int32_t wavefront_size;
+  int32_t reserved;
+  uint64_t global_mem_bytes;
+} ae_devinfo;
+
+typedef struct ae_event ae_event; /* a hipEvent_t with timing enabled */
+
+/* ---- library ------------------------------------------------------------------ */
+int ae_abi_version(void);
+/* Text of the calling thread's most recent failure ("" if none). Never NULL. */
+const char* ae_last_error(void);
+/* Number of HIP devices visible (0 when there is none); never fails. */
+int ae_device_count(void);
+int ae_device_info(int device, ae_devinfo* out);
+
+/* ---- compile: replaces tl.compile / torch.utils.cpp_extension.load -------------- */
+/*
+ * Compile HIP source `src` for `arch` ("gfx950") with hipRTC. `headers`/`header_names`
+ * are in-memory include files (`#include "name"`), `opts` extra compiler options.
+ * On failure *out is NULL and ae_last_error() holds the compiler log.
+ */
+int ae_compile(const char* src, const char* name, const char* arch,
+               const char* const* opts, int nopts,
+               const char* const* header_names, const char* const* headers, int nheaders,
+               ae_module** out);
+/* hipRTC log of the compilation that produced the module (warnings; "" if none). */
+const char* ae_module_log(const ae_module* m);
+/* Borrowed view of the code object bytes. */
+int ae_module_code(const ae_module* m, const void** data, size_t* size);
+/* Code-object cache: write to / read from a file (the reference caches generated
+ * source under attn_engine/cache/<md5>.py, attn_engine.py:369-375). */
+int ae_module_save(const ae_module* m, const char* path);
+int ae_module_load(const char* path, ae_module** out);
+void ae_module_free(ae_module* m);
+
+/* ---- load + launch -------------------------------------------------------------- */
+/* Load the module on the current device (first call) and look up `kernel_name`.
+ * The returned handle is owned by the module and dies with it. */
+int ae_module_get_kernel(ae_module* m, const char* kernel_name, ae_kernel** out);
+/* Raw launch: `params` (params_bytes) is copied into the kernel argument buffer. */
+int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
+              const uint32_t grid[3], const uint32_t block[3],
+              uint32_t lds_bytes, void* stream);
+
+/*
+ * Typed launches. They validate the argument block against the tile configuration
+ * (NULL pointers, non-positive extents, head-group divisibility, block-mask extents,
+ * split-KV work buffers) and derive the grid; nothing is launched when a check fails.
+ *
+ * ae_prefill_fwd: one workgroup per (q-tile, q-head, batch) -- the grid of
+ *   attn_tl.py:86 -- flattened to 1-D so the kernel can order heavy causal tiles first.
+ * ae_decode_fwd:  split-KV pass, grid (num_splits, ceil(Hq/Hkv / block_m)*Hkv, B), followed by
+ *   the combine kernel, grid (Hq, B) (attn_gqa_decode_tl.py:150-151, 224-266).
+ *   `combine` may be NULL only when num_splits == 1 and the split kernel writes `out`.
+ */
+int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream);
+int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                  const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
+
+/* ---- timing on the launch stream ------------------------------------------------- */
+int ae_event_create(ae_event** out);
+int ae_event_record(ae_event* e, void* stream);
+/* Blocks until `stop` has completed, then returns the elapsed milliseconds. */
+int ae_event_elapsed_ms(ae_event* start, ae_event* stop, float* ms);
+void ae_event_destroy(ae_event* e);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AE_HIP_H */
