@@ -1,0 +1,156 @@
+"""Public API: ``OnlineFunc`` and ``AttentionEngine``.
+
+Drop-in for attention_engine/attn_engine/attn_engine.py: ``OnlineFunc`` (16-105) keeps its
+constructor and static-method protocol; ``AttentionEngine(qkv_meta, custom_fwd_inputs, score_mod,
+mask_mod, online_func, ...)`` (108-215) keeps its signature and shape dispatch (218-332) and
+returns a callable ``mod(q, k, v, *custom_inputs, block_mask=None) -> o`` (388-395).
+
+Behind the API everything is new: the traced functions are lowered to HIP functors, spliced into
+the hand-written gfx950 kernel templates under csrc/kernels, compiled with hipRTC through
+libae_hip.so and launched on torch's current stream.  There is a single backend; ``backend="tl"``
+and ``backend="cute"`` are both accepted and select the call convention only (for MLA the CuTe
+form ``mod(q, kv_cache) -> (out, lse)``, attn_engine.py:193-214).  Tuner arguments are accepted
+and ignored: tile shapes are fixed per head dimension.
+"""
+from __future__ import annotations
+
+import torch
+
+from core.transform.core import CustomIO, SymbolicArray, SymbolScalar, Var
+
+
+class OnlineFunc:
+    """User-defined online row-scale algorithm (see attn_script/Readme.md:45-65).
+
+    ``online_rowscales``: running per-row state, ``{name: SymbolScalar(name, Var(init))}``;
+    ``final_rowscales``: per-row results saved at the end (e.g. lse).
+    Subclasses override the static methods below; they are *traced*, not executed on data.
+    """
+
+    def __init__(self, online_rowscales: dict, final_rowscales: dict, external_fwd_tensors: CustomIO):
+        self.online_rowscales = online_rowscales
+        self.final_rowscales = final_rowscales
+        self.vars = {"scores": SymbolicArray(), "o_scale": None}
+        self.external_fwd_tensors = external_fwd_tensors
+        self.doosum_rowscales = SymbolicArray("doosum", Var("doosum"), shape_idx=["block_M"])
+
+    @staticmethod
+    def online_fwd(scores, online_rowscales, b, h, q_idx):
+        """One kv tile: returns (scores', online_rowscales', o_scale)."""
+        o_scale = SymbolScalar("o_scale", Var("o_scale"))
+        return scores, online_rowscales, o_scale
+
+    @staticmethod
+    def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+        """After the last tile: returns (o', final_rowscales)."""
+        return o, online_rowscales
+
+    @staticmethod
+    def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+        """Recompute rule for the backward pass (unused by this forward-only build)."""
+        return scores
+
+    @staticmethod
+    def backward(dp, scores, final_rowscales, b, h, q_idx, kv_idx):
+        """Backward rule (unused by this forward-only build)."""
+        return dp
+
+    @staticmethod
+    def combine(final_rowscales):
+        """Split-KV merge: returns o_scale[num_split, row] applied to the partial outputs."""
+        return SymbolScalar("o_scale", Var("o_scale"))
+
+
+class AttentionEngine:
+    def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
+                 mask_value="-inf", device=None, backend="tl",
+                 tune=False, tune_file="", tune_bwd=False, tune_file_bwd="",
+                 infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
+                 extern_block_mask=False, kv_shared=False):
+        if backend not in ("tl", "cute", "hip"):
+            raise ValueError(f"unknown backend {backend!r}")
+        if mask_value not in ("-inf", "0"):
+            raise ValueError(f"mask_value must be '-inf' or '0', got {mask_value!r}")
+        self.backend = backend
+        self.block_mask = None
+        self.final_rowscales = {}
+        if custom_fwd_inputs is None:
+            custom_fwd_inputs = CustomIO()
+        if online_func is None:
+            # the reference's CuTe scripts pass online_func=None for identity-style attention
+            online_func = _IdentityOnline()
+        self._op = self._select_lower_template(
+            qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
+            infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
+            infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
+            kv_shared=kv_shared)
+        # generated device source, under the attribute name scripts read
+        # (attn_script/reluattn.py:75-76)
+        self.tl_code = self._op.source
+        self.attention = self._op
+        if infer_mask or extern_block_mask:
+            self.block_mask = getattr(self._op, "block_mask", None)
+
+    # same dispatch order as attn_engine.py:218-332
+    def _select_lower_template(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
+                               mask_value, infer_mask, infer_mask_block_M, infer_mask_block_N,
+                               extern_block_mask, kv_shared):
+        dtype_map = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
+        q_meta, k_meta, v_meta = qkv_meta
+        dtype_map[q_meta.dtype]  # KeyError for unsupported dtypes, as in the reference (225-228, 304)
+        q_seqlen, kv_len = q_meta.shape[2], v_meta.shape[2]
+        head, head_kv = q_meta.shape[1], v_meta.shape[1]
+        for dim in (q_meta.shape[0], head, head_kv, q_seqlen, kv_len):
+            if isinstance(dim, str):
+                # dynamic extents are runtime parameters of the kernels; the meta value is a hint
+                continue
+        dynamic = any(isinstance(d, str) for m in qkv_meta for d in m.shape)
+
+        if kv_shared:
+            from core.lower.lower_decode import MLADecodeOp
+            return MLADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
+                               mask_value, cute_convention=(self.backend == "cute"))
+        if not dynamic and q_seqlen != kv_len and head > head_kv:
+            assert q_seqlen < kv_len
+            assert q_seqlen == 1
+            from core.lower.lower_decode import GQADecodeOp
+            return GQADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value)
+        if not dynamic and q_seqlen != kv_len and head == head_kv:
+            assert q_seqlen < kv_len
+            raise NotImplementedError(
+                "MHA decode with q_len > 1 (attn_script/mha_inference.py) is not built yet")
+        from core.lower.prefill_op import PrefillOp
+        return PrefillOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
+                         infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
+                         infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask)
+
+    def __call__(self, *args, **kargs):
+        if kargs.get("block_mask") is not None:
+            self.block_mask = kargs["block_mask"]
+        kargs.pop("block_mask", None)
+        if self.block_mask is not None:
+            o = self._op(*args, self.block_mask, **kargs)
+        else:
+            o = self._op(*args, **kargs)
+        self.final_rowscales = getattr(self._op, "final_rowscales", {})
+        return o
+
+    def forward_with_rowscales(self, *args, **kargs):
+        """``mod(...)`` plus the final rowscales of that call: (o, {name: fp32 [B, Hq, Sq]})."""
+        o = self(*args, **kargs)
+        return o, dict(self.final_rowscales)
+
+
+class _IdentityOnline(OnlineFunc):
+    """No row state, no rescale: out = sum_kv score_mod(s) * v."""
+
+    def __init__(self):
+        super().__init__({}, {}, CustomIO())
+
+    @staticmethod
+    def online_fwd(scores, online_rowscales, b, h, q_idx):
+        return scores, online_rowscales, SymbolScalar("o_scale", Var("1"))
+
+    @staticmethod
+    def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+        return o, {}

@@ -1,0 +1,286 @@
+"""Prefill lowering: traced user functions -> the two generated headers of the HIP template.
+
+Stands where the reference's ``lower_tl`` fills the jinja slots of its TileLang prefill template
+(attention_engine/core/lower/lower.py:617-783, with lower_score_mod 475-558, lower_online_func
+318-472, lower_custom_inputs 560-614).  Output here: ``ae_config.h`` (compile-time
+configuration) and ``ae_functors.h`` (ae_score_mod / ae_mask_mod / ae_online_fwd / ae_epilogue /
+ae_load_custom) for csrc/kernels/ae_prefill.hip, plus the tile configuration and mask plan the
+host needs at launch time.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from ..codegen.hip_gen import Emitter, init_literal, var_as_constant
+from ..transform.core import CustomIO, SymbolicArray, SymbolScalar
+from ..transform.graph import Var
+from .mask import MASK_HELPERS, LoweredMask, MaskPlan, lower_mask_mod, plan_mask
+
+DTYPE_NAMES = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
+
+# symbolic dimension name of a CustomIO tensor -> index expression inside the kernel
+_DIM_INDEX = {"batch": "ctx.b", "heads": "ctx.h", "seq_len": "ctx.q_idx"}
+_KV_DIM = "seq_len_kv"
+
+
+@dataclass
+class CustomInput:
+    name: str
+    shape: list          # as declared: ints or symbolic names
+    per_kv: bool         # indexed by kv position -> read inside the tile loop
+    torch_dtype: object  # dtype the kernel reads
+
+
+@dataclass
+class LoweredFunctors:
+    """Everything the functor header needs, independent of tile sizes."""
+    score_mod_body: str
+    online_fwd_body: str
+    online_fwd_return: str
+    epilogue_body: str
+    rowstate_fields: list
+    rowstate_init: list
+    final_rowscale_names: list
+    o_scale_one: bool
+    customs: list = field(default_factory=list)
+    mask: LoweredMask = None
+
+
+def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
+    """Leaf expressions for the CustomIO tensors + their descriptors.
+
+    A tensor whose shape has no kv dimension is loaded once per row into ``cust.<name>``
+    (fp32, like the reference's accum_dtype fragments, lower.py:580); one with a
+    ``seq_len_kv`` dimension is read per element from global memory in the input dtype
+    (lower.py:590-597)."""
+    leaves, descs, loads, fields = {}, [], [], []
+    for slot, (name, sym) in enumerate(custom_fwd_inputs.input_tensors.items()):
+        slot += slot_offset
+        dims = list(sym.shape_idx)
+        per_kv = _KV_DIM in dims
+        idx_terms, stride = [], "1"
+        # row-major index over the declared shape
+        extents = {"batch": "p.batch", "heads": "p.heads_q", "seq_len": "p.seqlen_q",
+                   _KV_DIM: "p.seqlen_kv"}
+        for d in reversed(dims):
+            if d in _DIM_INDEX:
+                idx_terms.append(f"(int64_t)({_DIM_INDEX[d]}) * ({stride})")
+                stride = f"{stride} * (int64_t){extents[d]}"
+            elif d == _KV_DIM:
+                idx_terms.append(f"(int64_t)(AE_KV) * ({stride})")
+                stride = f"{stride} * (int64_t){extents[d]}"
+            elif d == "1":
+                pass
+            else:
+                raise NotImplementedError(
+                    f"custom input {name!r}: dimension {d!r} (use 1, 'batch', 'heads', 'seq_len', 'seq_len_kv')")
+        index = " + ".join(idx_terms) if idx_terms else "0"
+        if per_kv:
+            raise NotImplementedError(
+                f"custom input {name!r} has a seq_len_kv dimension; per-element custom tensors "
+                "(e.g. the retention decay mask) are not lowered yet")
+        fields.append(f"float {name};")
+        loads.append(f"c.{name} = ((const float*)p.custom[{slot}])[{index}];")
+        leaves[id(sym)] = (f"cust.{name}", False)
+        tdtype = torch.float32
+        descs.append(CustomInput(name, dims, per_kv, tdtype))
+    return leaves, descs, loads, fields
+
+
+def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO, in_dtype,
+                   mask_value: str = "-inf") -> LoweredFunctors:
+    """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
+    custom_fwd_inputs = custom_fwd_inputs if custom_fwd_inputs is not None else CustomIO()
+    cust_leaves, customs, cust_loads, cust_fields = _custom_leaves(custom_fwd_inputs, in_dtype)
+
+    def index_leaves():
+        b = SymbolScalar("b", Var("b"), shape_idx=[])
+        h = SymbolScalar("h", Var("h"), shape_idx=[])
+        q_idx = SymbolScalar("q_idx", Var("q_idx"), shape_idx=["block_M"])
+        kv_idx = SymbolScalar("kv_idx", Var("kv_idx"), shape_idx=["block_N"])
+        leaves = {id(b): ("(float)ctx.b", False), id(h): ("(float)ctx.h", False),
+                  id(q_idx): ("(float)ctx.q_idx", False), id(kv_idx): ("kvf", True)}
+        return b, h, q_idx, kv_idx, leaves
+
+    # ---- score_mod ------------------------------------------------------------------------
+    b, h, q_idx, kv_idx, leaves = index_leaves()
+    scores = SymbolicArray("scores", Var("scores"), shape_idx=["block_M", "block_N"])
+    leaves[id(scores)] = ("s", True)
+    leaves.update(cust_leaves)
+    if score_mod is not None:
+        out = score_mod(scores, custom_fwd_inputs, b, h, q_idx, kv_idx)
+    else:
+        out = scores
+    em = Emitter(leaves, {}, ["block_N"], n="N", prefix="sm")
+    val = em.value(out)
+    body = []
+    if id(kv_idx) in em.done:
+        body += ["  float kvf[N];", "#pragma unroll",
+                 "  for (int e = 0; e < N; e++) kvf[e] = (float)(ctx.kv_base + ae_kv_off(e));"]
+    body.append(em.code())
+    if val[0] != "s":
+        src = f"{val[0]}[e]" if val[1] else val[0]
+        body += ["#pragma unroll", f"  for (int e = 0; e < N; e++) s[e] = {src};"]
+    score_mod_body = "\n".join(body)
+
+    # ---- online_fwd -----------------------------------------------------------------------
+    b, h, q_idx, _, leaves = index_leaves()
+    scores = SymbolicArray("scores", Var("scores"), shape_idx=["block_M", "block_N"])
+    leaves[id(scores)] = ("s", True)
+    leaves.update(cust_leaves)
+    rowscales = online_func.online_rowscales
+    fields, inits = [], []
+    for k, v in rowscales.items():
+        v.clear_codegen()
+        leaves[id(v)] = (f"st.{k}", False)
+        fields.append(k)
+        inits.append(init_literal(v.code.name))
+    new_scores, new_rowscales, o_scale = online_func.online_fwd(scores, rowscales, b, h, q_idx)
+    em = Emitter(leaves, {}, ["block_N"], n="N", prefix="of")
+    new_vals = {k: em.value(v) for k, v in new_rowscales.items()}
+    sval = em.value(new_scores)
+    o_scale_const = var_as_constant(o_scale) if isinstance(o_scale, SymbolScalar) else float(o_scale)
+    o_scale_one = o_scale_const is not None and float(o_scale_const) == 1.0
+    oval = em.value(o_scale) if isinstance(o_scale, SymbolScalar) else (repr(float(o_scale)) + "f", False)
+    if oval[1]:
+        raise NotImplementedError("o_scale must be one value per row")
+    body = [em.code()]
+    if sval[0] != "s":
+        src = f"{sval[0]}[e]" if sval[1] else sval[0]
+        body += ["#pragma unroll", f"  for (int e = 0; e < N; e++) s[e] = {src};"]
+    body.append(f"  const float ae_o_scale = {oval[0]};")
+    for k, (expr, is_arr) in new_vals.items():
+        if k not in rowscales:
+            raise NotImplementedError(f"online_fwd returned an undeclared rowscale {k!r}")
+        if is_arr:
+            raise NotImplementedError(f"rowscale {k!r} must be one value per row")
+        if expr != f"st.{k}":
+            body.append(f"  st.{k} = {expr};")
+    online_fwd_body = "\n".join(body)
+
+    # ---- epilogue -------------------------------------------------------------------------
+    b, h, q_idx, _, leaves = index_leaves()
+    acc = SymbolicArray("acc_o", Var("acc_o"), shape_idx=["block_M", "dimv"])
+    leaves[id(acc)] = ("o", True)
+    leaves.update(cust_leaves)
+    for k, v in rowscales.items():
+        v.clear_codegen()
+        leaves[id(v)] = (f"st.{k}", False)
+    o_new, final_rowscales = online_func.online_fwd_epilogue(acc, rowscales, b, h, q_idx)
+    em = Emitter(leaves, {}, ["dimv"], n="N", prefix="ep")
+    oval = em.value(o_new)
+    fvals = [(k, em.value(v)) for k, v in final_rowscales.items()]
+    body = [em.code()]
+    if oval[0] != "o":
+        src = f"{oval[0]}[e]" if oval[1] else oval[0]
+        body += ["#pragma unroll", f"  for (int e = 0; e < N; e++) o[e] = {src};"]
+    for i, (k, (expr, is_arr)) in enumerate(fvals):
+        if is_arr:
+            raise NotImplementedError(f"final rowscale {k!r} must be one value per row")
+        body.append(f"  frs[{i}] = {expr};")
+    epilogue_body = "\n".join(body)
+
+    lowered_mask = lower_mask_mod(mask_mod) if mask_mod is not None else None
+    lf = LoweredFunctors(score_mod_body, online_fwd_body, "ae_o_scale", epilogue_body, fields, inits,
+                         [k for k, _ in fvals], o_scale_one, customs, lowered_mask)
+    lf.custom_fields = cust_fields
+    lf.custom_loads = cust_loads
+    return lf
+
+
+def render_functors(lf: LoweredFunctors) -> str:
+    """Text of ae_functors.h."""
+    nrs = max(1, len(lf.final_rowscale_names))
+    fields = "\n".join(f"  float {f};" for f in lf.rowstate_fields) or "  int ae_unused;"
+    inits = "\n".join(f"  st.{f} = {v};" for f, v in zip(lf.rowstate_fields, lf.rowstate_init)) or "  st.ae_unused = 0;"
+    cfields = "\n".join("  " + f for f in lf.custom_fields) or "  int ae_unused;"
+    cloads = "\n".join("  " + ld for ld in lf.custom_loads) or "  c.ae_unused = 0;"
+    mask_body = lf.mask.body if lf.mask is not None else "  return true;"
+    return f"""// generated by core/lower/lower.py -- do not edit
+{MASK_HELPERS}
+struct ae_custom {{
+{cfields}
+}};
+AE_DEV void ae_load_custom(ae_custom& c, const ae_attn_params& p, const ae_ctx& ctx) {{
+{cloads}
+}}
+struct ae_rowstate {{
+{fields}
+}};
+AE_DEV void ae_rowstate_init(ae_rowstate& st) {{
+{inits}
+}}
+AE_DEV bool ae_mask_mod(int b, int h, int q_idx, int kv_idx) {{
+{mask_body}
+}}
+template <int N>
+AE_DEV void ae_score_mod(float (&s)[N], const ae_ctx& ctx, const ae_custom& cust) {{
+{lf.score_mod_body}
+}}
+template <int N>
+AE_DEV float ae_online_fwd(float (&s)[N], ae_rowstate& st, const ae_ctx& ctx, const ae_custom& cust) {{
+{lf.online_fwd_body}
+  return {lf.online_fwd_return};
+}}
+template <int N>
+AE_DEV void ae_epilogue(float (&o)[N], ae_rowstate& st, float (&frs)[{nrs}], const ae_ctx& ctx,
+                        const ae_custom& cust) {{
+{lf.epilogue_body}
+}}
+"""
+
+
+@dataclass
+class PrefillTiles:
+    """Tile configuration of the prefill template (fixed per head dim; chosen from rocprof
+    measurements rather than tuned at run time)."""
+    n_waves: int = 4
+    block_n: int = 64
+    waves_per_eu: int = 2
+    k_pad: int = 16
+    v_pad: int = 64
+
+    @property
+    def block_m(self):
+        return 32 * self.n_waves
+
+    def lds_bytes(self, d: int, dv: int) -> int:
+        return 2 * (self.block_n * (2 * d + self.k_pad) + self.block_n * (2 * dv + self.v_pad))
+
+
+def choose_prefill_tiles(d: int, dv: int) -> PrefillTiles:
+    t = PrefillTiles()
+    if max(d, dv) > 128:
+        # larger head dims: one wave per SIMD gets the whole register file
+        t.waves_per_eu = 1
+        t.block_n = 32
+    # V rows must land on distinct LDS bank groups for the transpose reads: pitch = 64 mod 256
+    t.v_pad = (64 - (2 * dv) % 256) % 256
+    if t.v_pad == 0:
+        t.v_pad = 256
+    return t
+
+
+def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, has_mask_mod: bool,
+                  n_rowscales: int, o_scale_one: bool, even_q: bool, even_kv: bool) -> str:
+    """Text of ae_config.h."""
+    return "\n".join([
+        "// generated by core/lower/lower.py -- do not edit",
+        f"#define AE_D {d}",
+        f"#define AE_DV {dv}",
+        f"#define AE_BN {tiles.block_n}",
+        f"#define AE_NWAVES {tiles.n_waves}",
+        f"#define AE_DTYPE_BF16 {1 if dtype == torch.bfloat16 else 0}",
+        f"#define AE_MASK_MODE {mask_mode}",
+        f"#define AE_HAS_MASK_MOD {1 if has_mask_mod else 0}",
+        f"#define AE_N_ROWSCALES {n_rowscales}",
+        f"#define AE_O_SCALE_ONE {1 if o_scale_one else 0}",
+        f"#define AE_EVEN_Q {1 if even_q else 0}",
+        f"#define AE_EVEN_KV {1 if even_kv else 0}",
+        f"#define AE_WAVES_PER_EU {tiles.waves_per_eu}",
+        f"#define AE_K_PAD {tiles.k_pad}",
+        f"#define AE_V_PAD {tiles.v_pad}",
+        "",
+    ])

@@ -1,0 +1,188 @@
+"""Prefill operator: owns the compiled kernel variants of one AttentionEngine and launches them.
+
+Host-side counterpart of the reference's generated ``_attention.forward`` + ``tl.compile`` result
+(attention_engine/core/template/tl_template/attn/attn_tl.py:523-528, 567-580; block-sparse:
+blockattn_tl.py:401-447): takes q/k/v ``[B,S,H,D]`` plus the CustomIO tensors (and, when a block
+mask is in play, that mask as the LAST positional argument), allocates ``o`` and the final
+rowscales, launches on torch's current stream, returns ``o``.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..runtime import hip_rt as rt
+from ..transform.core import _convert_mask_to_block_mask, is_causal_mask
+from . import lower as L
+from .mask import plan_mask
+
+
+def _dim(x, default):
+    return default if isinstance(x, str) else int(x)
+
+
+class PrefillOp:
+    def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
+                 infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
+                 extern_block_mask=False):
+        q_meta, k_meta, v_meta = qkv_meta
+        self.dtype = q_meta.dtype
+        self.D = int(q_meta.shape[3])
+        self.DV = int(v_meta.shape[3])
+        if int(k_meta.shape[3]) != self.D:
+            raise ValueError("q and k head dims differ")
+        if self.D % 16 or self.DV % 32:
+            raise NotImplementedError(f"head dims (D={self.D}, DV={self.DV}) must be multiples of 16 / 32")
+        self.mask_mod = mask_mod
+        self.elementwise_mask = mask_mod is not None and mask_value == "-inf"
+        self.extern_block_mask = bool(extern_block_mask)
+        self.mask_block = (int(infer_mask_block_M), int(infer_mask_block_N))
+        self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
+                                         self.dtype, mask_value)
+        self.functor_src = L.render_functors(self.functors)
+        self.tiles = L.choose_prefill_tiles(self.D, self.DV)
+        if self.extern_block_mask:
+            # a q tile must sit inside one block-mask row, a kv tile inside one column
+            while self.tiles.block_m > self.mask_block[0] and self.tiles.n_waves > 1:
+                self.tiles.n_waves //= 2
+            while self.tiles.block_n > self.mask_block[1] and self.tiles.block_n > 32:
+                self.tiles.block_n //= 2
+            if self.mask_block[0] % self.tiles.block_m or self.mask_block[1] % self.tiles.block_n:
+                raise NotImplementedError(f"block mask granularity {self.mask_block} does not fit the tiles")
+        self.n_rowscales = len(self.functors.final_rowscale_names)
+        if self.n_rowscales > rt.AE_MAX_ROWSCALES or len(self.functors.customs) > rt.AE_MAX_CUSTOM:
+            raise NotImplementedError("too many rowscales / custom inputs")
+        self.final_rowscales = {}
+        self.block_mask = None
+        self._variants = {}   # (mask_mode, even_q, even_kv) -> (module, cfg, config_src)
+        self._plans = {}      # (B|1, H|1, Sq, Skv) -> MaskPlan with device table
+        self.meta_shape = (_dim(q_meta.shape[0], 1), _dim(q_meta.shape[1], 1), _dim(q_meta.shape[2], 0),
+                           _dim(v_meta.shape[2], 0))
+        # compile for the declared shape now (hipRTC needs no GPU) so construction reports
+        # lowering/compile errors, like the reference's constructor does
+        B, H, Sq, Skv = self.meta_shape
+        self.source = self.functor_src
+        if Sq > 0:
+            plan = self._plan(B, H, Sq, Skv, device=None)
+            mode = 2 if self.extern_block_mask else plan.mode
+            _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0)
+            self.source = cfg_src + "\n" + self.functor_src
+            if infer_mask and mask_mod is not None and not self.extern_block_mask:
+                self.block_mask = self._reference_block_mask(B, H, Sq, Skv)
+
+    # ---- mask --------------------------------------------------------------------------
+    def _plan(self, B, H, Sq, Skv, device):
+        key = (B, H, Sq, Skv)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = plan_mask(self.mask_mod, self.functors.mask, B, H, Sq, Skv, self.tiles.block_m,
+                             self.tiles.block_n, elementwise=self.elementwise_mask)
+            self._plans[key] = plan
+        if device is not None and plan.table is not None and plan.table.device != device:
+            plan.table = plan.table.to(device)
+        return plan
+
+    def _reference_block_mask(self, B, H, Sq, Skv):
+        """The block mask the reference would keep on ``mod.block_mask`` (lower.py:721-738):
+        int8 [B,H,Sq/bm,Skv/bn] "any element visible", or None when it is exactly block-causal
+        (dense template)."""
+        bm, bn = self.mask_block
+        lm = self.functors.mask
+        mb, mh = (B if lm.uses_b else 1), (H if lm.uses_h else 1)
+        rows = []
+        kv = torch.arange(Skv).view(1, 1, 1, Skv)
+        for r0 in range(0, Sq, bm * 8):
+            r1 = min(Sq, r0 + bm * 8)
+            q = torch.arange(r0, r1).view(1, 1, -1, 1)
+            m = self.mask_mod(torch.arange(mb).view(mb, 1, 1, 1), torch.arange(mh).view(1, mh, 1, 1), q, kv)
+            if not isinstance(m, torch.Tensor):
+                m = torch.tensor(bool(m))
+            m = m.to(torch.bool).expand(mb, mh, r1 - r0, Skv)
+            rows.append(_convert_mask_to_block_mask(m, bm, bn)[0])
+        blocks = torch.cat(rows, dim=2).expand(B, H, -1, -1)
+        if Sq == Skv and bool(is_causal_mask(blocks, bm, bn)):
+            return None
+        return blocks.contiguous()
+
+    # ---- kernels -------------------------------------------------------------------------
+    def _variant(self, mask_mode, even_q, even_kv):
+        key = (mask_mode, even_q, even_kv)
+        v = self._variants.get(key)
+        if v is None:
+            has_mask_mod = self.elementwise_mask and mask_mode != 1
+            cfg_src = L.render_config(self.D, self.DV, self.dtype, self.tiles, mask_mode, has_mask_mod,
+                                      self.n_rowscales, self.functors.o_scale_one, even_q, even_kv)
+            module = rt.compile_module("ae_prefill.hip", {"ae_config.h": cfg_src,
+                                                          "ae_functors.h": self.functor_src})
+            cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
+                             threads=64 * self.tiles.n_waves,
+                             lds_bytes=self.tiles.lds_bytes(self.D, self.DV), head_dim=self.D,
+                             head_dim_v=self.DV, elem_bytes=2, n_rowscales=self.n_rowscales,
+                             mask_mode=mask_mode)
+            v = self._variants[key] = (module, cfg, cfg_src)
+        return v
+
+    # ---- launch ----------------------------------------------------------------------------
+    def __call__(self, q, k, v, *extra):
+        n_custom = len(self.functors.customs)
+        extern_mask = None
+        if len(extra) == n_custom + 1:
+            extern_mask = extra[-1]
+            extra = extra[:-1]
+        if len(extra) != n_custom:
+            raise TypeError(f"expected {n_custom} custom input tensor(s), got {len(extra)}")
+        for name, t in (("q", q), ("k", k), ("v", v)):
+            if not (isinstance(t, torch.Tensor) and t.is_cuda):
+                raise RuntimeError(f"{name} must be a tensor on the GPU (there is no CPU path)")
+            if t.dtype != self.dtype:
+                raise TypeError(f"{name} has dtype {t.dtype}, the engine was built for {self.dtype}")
+            if t.dim() != 4:
+                raise ValueError(f"{name} must be [batch, seq, heads, dim]")
+        B, Sq, Hq, D = q.shape
+        Bk, Skv, Hkv, Dk = k.shape
+        if (D, Dk, v.shape[3]) != (self.D, self.D, self.DV):
+            raise ValueError(f"head dims {(D, Dk, v.shape[3])} differ from the compiled {(self.D, self.D, self.DV)}")
+        if Bk != B or v.shape[0] != B or v.shape[1] != Skv or v.shape[2] != Hkv or Hq % Hkv:
+            raise ValueError("inconsistent q/k/v shapes")
+        q, k, v = (t if t.stride(3) == 1 else t.contiguous() for t in (q, k, v))
+        dev = q.device
+
+        if extern_mask is not None:
+            bm, bn = self.mask_block
+            table = extern_mask
+            if table.dim() != 4:
+                raise ValueError("block_mask must be [B|1, H|1, Sq/bm, Skv/bn]")
+            if table.dtype != torch.int8:
+                table = table.to(torch.int8)
+            table = table.to(dev).contiguous()
+            mode, mbm, mbn = 2, bm, bn
+        else:
+            plan = self._plan(B, Hq, Sq, Skv, dev)
+            mode, table, mbm, mbn = plan.mode, plan.table, plan.block_m, plan.block_n
+        module, cfg, _ = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0)
+        kern = module.kernel("ae_prefill_kernel")
+
+        out = torch.empty((B, Sq, Hq, self.DV), dtype=self.dtype, device=dev)
+        rowscales = [torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev) for _ in range(self.n_rowscales)]
+        p = rt.AttnParams()
+        p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+        for i, r in enumerate(rowscales):
+            p.rowscale_out[i] = r.data_ptr()
+        keep = []
+        for i, (desc, t) in enumerate(zip(self.functors.customs, extra)):
+            t = t.to(device=dev, dtype=desc.torch_dtype).contiguous()
+            keep.append(t)
+            p.custom[i] = t.data_ptr()
+        p.q_stride_b, p.q_stride_s, p.q_stride_h = q.stride(0), q.stride(1), q.stride(2)
+        p.k_stride_b, p.k_stride_s, p.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
+        p.v_stride_b, p.v_stride_s, p.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
+        p.o_stride_b, p.o_stride_s, p.o_stride_h = out.stride(0), out.stride(1), out.stride(2)
+        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = B, Hq, Hkv, Sq, Skv
+        if mode == 2:
+            p.block_mask = table.data_ptr()
+            p.mask_b, p.mask_h, p.mask_nq, p.mask_nkv = table.shape
+            p.mask_block_m, p.mask_block_n = mbm, mbn
+            keep.append(table)
+        rt.prefill_fwd(kern, p, cfg, torch.cuda.current_stream(dev).cuda_stream)
+        self.final_rowscales = dict(zip(self.functors.final_rowscale_names, rowscales))
+        self._keepalive = keep
+        return out

@@ -1,0 +1,216 @@
+"""GPU parity of the prefill path: HIP kernels (through AttentionEngine -> libae_hip.so) against
+the CPU oracle on the same seeded inputs.
+
+Tolerances are the ones the task states: out max-abs <= 2e-2, lse max-abs <= 1e-3 against an fp32
+oracle that consumes the fp16/bf16-rounded inputs; masks bit-exact.
+"""
+import math
+
+import pytest
+import torch
+
+import attn_cases as C
+from attn_engine import AttentionEngine
+from core import CustomIO, meta_tensor
+from oracle import attention_ref as R
+from oracle import masks as M
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 2e-2
+LSE_TOL = 1e-3
+
+
+def _engine(B, H, S, D, DV, dtype, score_mod, mask_mod, online, customs=None, Hkv=None, **kw):
+    Hkv = H if Hkv is None else Hkv
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+            meta_tensor(B, Hkv, S, DV, dtype=dtype))
+    return AttentionEngine(meta, customs if customs is not None else CustomIO({}), score_mod=score_mod,
+                           mask_mod=mask_mod, online_func=online, **kw)
+
+
+def _dense(mask_mod, B, H, Sq, Skv):
+    return torch.from_numpy(M.dense_mask_grid(mask_mod, B, H, Sq, Skv))
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S,D,dtype", [
+    (1, 4, 512, 64, torch.float16),      # BASELINE config 1 shape, fp16 cast of the same inputs
+    (2, 4, 1024, 128, torch.float16),
+    (1, 2, 384, 128, torch.bfloat16),
+    (1, 2, 200, 128, torch.float16),     # ragged: S not a multiple of any tile
+    (1, 1, 77, 64, torch.bfloat16),
+])
+def test_softmax_prefill(cuda_device, B, H, S, D, dtype, causal):
+    print(f"case softmax B{B} H{H} S{S} D{D} {dtype} causal={causal}", flush=True)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)),
+                  C.causal_mask if causal else None, C.OnlineSoftmax())
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    ref, lse = R.softmax_attention(q, k, v, causal=causal)
+    assert out.dtype == dtype and out.shape == ref.shape
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
+def test_softmax_headline_shape_properties(cuda_device):
+    """BASELINE config 2 at full size (B2 H32 S4096 D128 fp16, causal): too big for the CPU
+    oracle in a test, so it is checked through size-independent properties -- one (batch, head)
+    slice against the oracle, and for all rows: row 0 attends only to itself (out == v[0],
+    lse == q0.k0*scale), outputs finite, lse non-decreasing... is NOT a property; instead lse is
+    compared on the slice only."""
+    B, H, S, D = 2, 32, 4096, 128
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask,
+                  C.OnlineSoftmax())
+    out = mod(q.cuda(), k.cuda(), v.cuda()).cpu()
+    lse = mod.final_rowscales["lse"].cpu()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    # first row of every (b, h) sees only kv 0
+    assert (out[:, 0].float() - v[:, 0].float()).abs().max().item() <= 1e-3
+    s00 = (q[:, 0].float() * k[:, 0].float()).sum(-1) / math.sqrt(D)
+    assert (lse[:, :, 0] - s00).abs().max().item() <= LSE_TOL
+    for b, h in ((0, 0), (1, 31)):
+        ref, lref = R.softmax_attention(q[b:b + 1, :, h:h + 1], k[b:b + 1, :, h:h + 1],
+                                        v[b:b + 1, :, h:h + 1], causal=True)
+        assert (out[b:b + 1, :, h:h + 1].float() - ref).abs().max().item() <= OUT_TOL
+        assert (lse[b:b + 1, h:h + 1] - lref).abs().max().item() <= LSE_TOL
+
+
+@pytest.mark.parametrize("B,H,S,D,causal", [(1, 2, 512, 128, False), (2, 2, 320, 64, True)])
+def test_sigmoid_prefill(cuda_device, B, H, S, D, causal):
+    """BASELINE config 3 form: sigmoid(s/sqrt(D) + b), b = -ln(S), identity rowscales."""
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    bias = torch.tensor([-math.log(S)], dtype=torch.float32)
+    mod = _engine(B, H, S, D, D, dtype, C.make_sigmoid_score_mod(1 / math.sqrt(D)),
+                  C.causal_mask if causal else None, C.OnlineIdentity(),
+                  customs=CustomIO({"softmax_bias": (1,)}))
+    out = mod(q.cuda(), k.cuda(), v.cuda(), bias.cuda())
+    ref = R.sigmoid_attention(q, k, v, bias=bias.item(), causal=causal)
+    assert mod.final_rowscales == {}
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+
+
+def test_relu_prefill(cuda_device):
+    B, H, S, D = 2, 3, 256, 64
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_relu_score_mod(1 / math.sqrt(D)), None, C.OnlineIdentity())
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    ref = R.relu_attention(q, k, v)
+    # relu attention sums ~S/2 positive terms: compare relative to the output scale
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL * max(1.0, ref.abs().max().item())
+
+
+@pytest.mark.parametrize("name,mask_mod", [
+    ("plus_one", C.causal_plus_one_mask),
+    ("shifted", C.causal_shifted_mask),          # first 128 rows see nothing: out 0, lse -inf
+    ("window", C.make_sliding_window_mask(256)),
+    ("head_dep", C.head_dependent_mask),
+])
+def test_masked_softmax_prefill(cuda_device, name, mask_mod):
+    B, H, S, D = 2, 4, 512, 64
+    dtype = torch.bfloat16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod, C.OnlineSoftmax())
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    lse = mod.final_rowscales["lse"].cpu()
+    dense = _dense(mask_mod, B, H, S, S)
+    ref, lref = R.softmax_attention(q, k, v, mask=dense)
+    visible = dense.any(-1)                       # [B,H,S]
+    vis_rows = visible.permute(0, 2, 1)           # [B,S,H]
+    assert (out - ref)[vis_rows].abs().max().item() <= OUT_TOL
+    assert (lse - lref)[visible].abs().max().item() <= LSE_TOL
+    if (~visible).any():
+        # rows with no visible key: out = 0, lse = -inf
+        assert out[~vis_rows].abs().max().item() == 0.0
+        assert torch.isneginf(lse[~visible]).all()
+
+
+def test_mask_is_bit_exact(cuda_device):
+    """Probe the effective device mask.  The score_mod maps every finite score to exactly 1 and a
+    masked (-inf) score to exactly 0 (tanh saturates), rowscales are the identity and V holds
+    one-hot rows (kv -> column kv mod DV), so out[q, j] COUNTS the visible keys of residue class j:
+    small integers, compared exactly against the host evaluation of the mask_mod."""
+    B, H, S, D = 1, 2, 256, 64
+
+    def ones_score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+        return ((score * 0.001 + 50.0).tanh() + 1.0) * 0.5
+
+    dtype = torch.float16
+    for mask_mod in (C.causal_mask, C.make_sliding_window_mask(100), C.head_dependent_mask,
+                     C.causal_plus_one_mask):
+        q, k, _ = C.make_inputs(B, S, S, H, H, D, D, dtype)
+        v = torch.zeros(B, S, H, D, dtype=dtype)
+        v[:, torch.arange(S), :, torch.arange(S) % D] = 1.0
+        mod = _engine(B, H, S, D, D, dtype, ones_score_mod, mask_mod, C.OnlineIdentity())
+        out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+        dense = _dense(mask_mod, B, H, S, S).float()                  # [B,H,S,S]
+        onehot = torch.zeros(S, D)
+        onehot[torch.arange(S), torch.arange(S) % D] = 1.0
+        expect = torch.einsum("bhqk,kd->bqhd", dense, onehot)
+        assert torch.equal(out, expect), mask_mod.__name__
+
+
+def test_extern_block_mask(cuda_device):
+    """attn_script/blocksparseattn.py: user-supplied int8 block mask [B,H,S/128,S/128], no
+    mask_mod; reference = masked softmax with the expanded block mask (129-135)."""
+    B, H, S, D = 1, 4, 1024, 128
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(1)
+    nb = S // 128
+    blocks = (torch.rand(B, H, nb, nb, generator=g) < 0.4)
+    blocks |= torch.eye(nb, dtype=torch.bool)      # every row sees something
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), None, C.OnlineSoftmax(),
+                  infer_mask=True, extern_block_mask=True)
+    out = mod(q.cuda(), k.cuda(), v.cuda(), block_mask=blocks.to(torch.int8).cuda())
+    dense = blocks.repeat_interleave(128, 2).repeat_interleave(128, 3)
+    ref, lref = R.softmax_attention(q, k, v, mask=dense)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lref).abs().max().item() <= LSE_TOL
+
+
+def test_score_mod_with_indices(cuda_device):
+    """score_mod that reads q_idx, kv_idx and h (an ALiBi-style bias)."""
+    B, H, S, D = 1, 4, 256, 64
+    dtype = torch.float16
+    scale, slope = 1 / math.sqrt(D), 0.05
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_alibi_score_mod(scale, slope), C.causal_mask, C.OnlineSoftmax())
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    s = torch.einsum("bqhd,bkhd->bhqk", q.float(), k.float()) * scale
+    dist = (torch.arange(S).view(S, 1) - torch.arange(S).view(1, S)).abs().float()
+    s = s - dist * ((torch.arange(H).float() + 1) * slope).view(1, H, 1, 1)
+    s = s.masked_fill(~torch.ones(S, S, dtype=torch.bool).tril(), float("-inf"))
+    ref = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(s, -1), v.float())
+    assert (out - ref).abs().max().item() <= OUT_TOL
+
+
+def test_gqa_prefill(cuda_device):
+    """Hq > Hkv with Sq == Skv: q head h reads kv head h // groups (attn_gqa_tl.py:80,95)."""
+    B, H, G, S, D = 1, 8, 2, 256, 128
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, G, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask,
+                  C.OnlineSoftmax(), Hkv=G)
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    ref, lse = R.softmax_attention(q, k, v, causal=True)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
+def test_abs_norm_online_func(cuda_device):
+    """An OnlineFunc other than softmax: running abs-sum normalisation with a clamp."""
+    from oracle.online_interp import online_attention
+    B, H, S, D = 1, 2, 256, 64
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    sm = C.make_scale_score_mod(1 / math.sqrt(D))
+    mod = _engine(B, H, S, D, D, dtype, sm, None, C.OnlineAbsNorm())
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    ref, finals = online_attention(q, k, v, sm, None, C.OnlineAbsNorm(), block_n=64)
+    assert (mod.final_rowscales["r"].cpu() - finals["r"].float()).abs().max().item() <= 1e-3 * finals["r"].max().item()
+    assert (out - ref.float()).abs().max().item() <= OUT_TOL
