@@ -75,7 +75,10 @@ class Emitter:
     that make a value an array; ``n`` is the C++ expression of the array length.
     """
 
-    def __init__(self, leaves: dict, named_leaves: dict, array_axes, n: str = "N", prefix: str = "t"):
+    def __init__(self, leaves: dict, named_leaves: dict, array_axes, n: str = "N", prefix: str = "t",
+                 split_axis: bool = False):
+        # split_axis: the array axis is the split axis of OnlineFunc.combine, reduced by ColReduce*
+        self.split_axis = split_axis
         self.leaves = leaves
         self.named_leaves = named_leaves
         self.array_axes = set(str(a) for a in array_axes)
@@ -136,6 +139,8 @@ class Emitter:
         ins = [self.value(p) for p in sym.prev]
         out = self._tmp()
         if t in ROW_REDUCTIONS:
+            if self.split_axis:
+                raise NotImplementedError(f"{t} inside OnlineFunc.combine (use the column reductions)")
             src, is_arr = ins[0]
             if not is_arr:
                 raise NotImplementedError(f"{t} of a value that has no kv axis")
@@ -143,7 +148,15 @@ class Emitter:
             self.lines.append(f"const float {out} = {fn}<{self.n}>({src});")
             return (out, False)
         if t in COL_REDUCTIONS:
-            raise NotImplementedError(f"{t} is only meaningful inside OnlineFunc.combine")
+            if not self.split_axis:
+                raise NotImplementedError(f"{t} is only meaningful inside OnlineFunc.combine")
+            src, is_arr = ins[0]
+            if not is_arr:
+                raise NotImplementedError(f"{t} of a value that has no split axis")
+            fn = {"ColReduceSum": "ae_arr_sum", "ColReduceMax": "ae_arr_max",
+                  "ColReduceAbsSum": "ae_arr_abssum"}[t]
+            self.lines.append(f"const float {out} = {fn}<{self.n}>({src});")
+            return (out, False)
         if t == "MaxBwd":
             raise NotImplementedError("MaxBwd belongs to the backward pass")
         if t not in ELEMENTWISE_UNARY and t not in ELEMENTWISE_BINARY:

@@ -348,9 +348,17 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
   if (!combine || !combine_cfg)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel is NULL");
+  // one partial per wave: a workgroup of W waves produces W consecutive partials
+  int waves = cfg->threads / 64;
+  if (p->num_splits % waves != 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: num_splits=%d is not a multiple of %d waves",
+                p->num_splits, waves);
+  if (combine_cfg && combine_cfg->block_n != p->num_splits)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel built for %d splits, got %d",
+                combine_cfg->block_n, p->num_splits);
   int group = p->heads_q / p->heads_kv;
   int head_tiles = (group + cfg->block_m - 1) / cfg->block_m;
-  uint32_t grid[3] = {(uint32_t)p->num_splits, (uint32_t)(head_tiles * p->heads_kv),
+  uint32_t grid[3] = {(uint32_t)(p->num_splits / waves), (uint32_t)(head_tiles * p->heads_kv),
                       (uint32_t)p->batch};
   uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
   rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);

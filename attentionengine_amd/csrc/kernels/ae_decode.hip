@@ -1,0 +1,288 @@
+// Split-KV attention decode (one query token per sequence) for gfx950 / CDNA4, and the kernel
+// that merges the per-split partial results.
+//
+// Takes the place of the reference's TileLang GQA decode template
+// (attention_engine/core/template/tl_template/attn/attn_gqa_decode_tl.py: flash_attn_split 141-222,
+// combine 224-266).  Unlike that template, which hard-codes softmax (52-67), score_mod / online_func
+// / combine come from the traced user functions ("ae_config.h" / "ae_functors.h").
+//
+// The kernel is HBM-bound: every K and V element is read exactly once and used for all query
+// heads of its group, so the design goal is bytes in flight, not MFMA occupancy.
+//   * one WAVE owns an independent partial result ("split"): it walks its own 32-row kv tiles,
+//     keeps (acc_o, rowstate) in registers and writes fp32 partial (o, rowscales); waves never
+//     synchronise with each other, there is no workgroup barrier in the loop;
+//   * the query heads of one kv head (<= 16 per workgroup) are the N dimension of
+//     v_mfma_f32_16x16x32: S^T[kv,head] = K Q^T, O^T[dv,head] += V^T P^T, the same transposed
+//     scheme as the prefill kernel, so a lane owns one head's row state;
+//   * K rows go straight from HBM into the MFMA A-operand registers (no transpose needed: the
+//     contraction index d is contiguous in memory), prefetched one tile ahead;
+//   * V rows are loaded with coalesced 16-byte accesses into a wave-private LDS tile and read back
+//     with ds_read_b64_tr_b16, which delivers the kv-contiguous A operand of the PV product;
+//   * partials are fp32 [B,Hq,splits,DV] + fp32 rowscales [n,B,Hq,splits] (the CuTe backend's
+//     convention, cute_template_kvshared/flash_api.cpp:180-181); the combine kernel evaluates the
+//     user's combine() per (batch, head) and writes out [B,1,Hq,DV] and the merged rowscales.
+
+#define AE_LAYOUT 1
+#include "ae_hip.h"
+#include "ae_config.h"
+#include "ae_device.h"
+#include "ae_functors.h"
+
+#define AE_NT (AE_NWAVES * 64)
+#define AE_TILE 32                      // kv rows per wave tile
+#define AE_NS 8                         // score elements per lane per tile (2 blocks of 4)
+#define AE_NDB (AE_DV / 16)             // 16-wide dv blocks
+#define AE_NO (AE_NDB * 4)              // output elements per lane
+#define AE_NKS (AE_D / 32)              // 32-deep k-steps of QK^T
+#define AE_VSTR (AE_DV * 2 + AE_V_PAD)  // LDS row pitch of the V tile, bytes
+#define AE_V_WAVE_BYTES (AE_TILE * AE_VSTR)
+#define AE_VCPR (AE_DV / 8)             // 16-byte chunks per V row
+#define AE_V_LOADS ((AE_TILE * AE_VCPR) / 64)
+
+static_assert(AE_D % 32 == 0, "head dim must be a multiple of 32");
+static_assert(AE_DV % 16 == 0, "value head dim must be a multiple of 16");
+static_assert((AE_TILE * AE_VCPR) % 64 == 0, "V tile must split evenly over a wave");
+
+typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
+
+extern "C" __global__ __launch_bounds__(AE_NT)
+__attribute__((amdgpu_waves_per_eu(AE_WAVES_PER_EU, AE_WAVES_PER_EU)))
+void ae_decode_split_kernel(const ae_attn_params p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l16 = lane & 15;
+  const int g4 = lane >> 4;
+  ae_lds_byte* vs = (ae_lds_byte*)ae_smem + wave * AE_V_WAVE_BYTES;
+
+  // ---- which (batch, kv head, head tile, split) ------------------------------------------------
+  const int group = p.heads_q / p.heads_kv;
+  const int b = blockIdx.z;
+  const int hk = blockIdx.y % p.heads_kv;
+  const int ht = blockIdx.y / p.heads_kv;
+  const int split = blockIdx.x * AE_NWAVES + wave;       // index of this wave's partial
+  const int head_in_group = ht * 16 + l16;
+  const bool head_ok = head_in_group < group;
+  const int hq = hk * group + (head_ok ? head_in_group : 0);
+
+  // this workgroup covers kv [wg_base, wg_base + AE_NWAVES*kv_per_split); wave w takes the tiles
+  // w, w+NWAVES, ... of that range, so the workgroup streams one contiguous region of HBM
+  const int wg_base = blockIdx.x * AE_NWAVES * p.kv_per_split;
+  const int n_tiles = p.kv_per_split / AE_TILE;
+
+  // ---- Q fragments (B operand of S^T = K Q^T): n = head = l16, k = d = 32*ks + 8*g4 + j ---------
+  const ae_elem* qptr = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)hq * p.q_stride_h;
+  ae_elem8 qf[AE_NKS];
+#pragma unroll
+  for (int ks = 0; ks < AE_NKS; ks++) qf[ks] = *(const ae_elem8*)(qptr + ks * 32 + g4 * 8);
+
+  const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
+  const ae_elem* vbase = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
+
+  ae_elem8 kf[2][AE_NKS];       // K of the current tile, A-operand layout: m = kv = 16*rb + l16
+  ae_elem8 kf_next[2][AE_NKS];
+  ae_u32x4 vreg[AE_V_LOADS];
+
+  auto tile_kv0 = [&](int i) { return wg_base + (wave + i * AE_NWAVES) * AE_TILE; };
+  auto clamp_kv = [&](int kv) {
+#if AE_EVEN_KV
+    return kv;
+#else
+    return kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
+#endif
+  };
+  auto load_k = [&](int kv0, ae_elem8 (&dst)[2][AE_NKS]) {
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+      const ae_elem* row = kbase + (int64_t)clamp_kv(kv0 + rb * 16 + l16) * p.k_stride_s + g4 * 8;
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS; ks++) dst[rb][ks] = *(const ae_elem8*)(row + ks * 32);
+    }
+  };
+  auto load_v = [&](int kv0) {
+#pragma unroll
+    for (int i = 0; i < AE_V_LOADS; i++) {
+      int c = lane + i * 64;
+      int row = c / AE_VCPR, col = c % AE_VCPR;
+      vreg[i] = *(const ae_u32x4*)(vbase + (int64_t)clamp_kv(kv0 + row) * p.v_stride_s + col * 8);
+    }
+  };
+  auto store_v = [&]() {
+#pragma unroll
+    for (int i = 0; i < AE_V_LOADS; i++) {
+      int c = lane + i * 64;
+      int row = c / AE_VCPR, col = c % AE_VCPR;
+      *(__attribute__((address_space(3))) ae_u32x4*)(vs + row * AE_VSTR + col * 16) = vreg[i];
+    }
+  };
+
+  ae_ctx ctx;
+  ctx.b = b;
+  ctx.h = hq;
+  ctx.q_idx = 0;
+  ctx.kv_base = 0;
+  ae_custom cust;
+  ae_load_custom(cust, p, ctx);
+  ae_rowstate st;
+  ae_rowstate_init(st);
+  ae_f32x4 oacc[AE_NDB];
+#pragma unroll
+  for (int db = 0; db < AE_NDB; db++) oacc[db] = (ae_f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // tiles of this wave that start inside the sequence
+  int my_tiles = 0;
+  for (int i = 0; i < n_tiles; i++)
+    if (tile_kv0(i) < p.seqlen_kv) my_tiles = i + 1;
+
+  if (my_tiles > 0) {
+    load_k(tile_kv0(0), kf);
+    load_v(tile_kv0(0));
+  }
+  // transpose-read offset: lane i of a 16-lane group reads row (i/4), 4 columns from 4*(i%4)
+  const int v_rd_off = (4 * g4 + (l16 >> 2)) * AE_VSTR + (4 * (l16 & 3)) * 2;
+
+  for (int i = 0; i < my_tiles; i++) {
+    const int kv0 = tile_kv0(i);
+    store_v();                          // V(i): registers -> LDS (previous tile's reads are done)
+    const bool more = i + 1 < my_tiles;
+    if (more) {
+      load_k(tile_kv0(i + 1), kf_next);
+      load_v(tile_kv0(i + 1));
+    }
+
+    // ---- S^T = K Q^T: two 16-row kv blocks -------------------------------------------------------
+    ae_f32x4 sacc[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++) {
+      sacc[rb] = (ae_f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS; ks++) sacc[rb] = ae_mfma16(kf[rb][ks], qf[ks], sacc[rb]);
+    }
+    float s[AE_NS];
+#pragma unroll
+    for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) s[rb * 4 + r] = sacc[rb][r];
+
+    ctx.kv_base = kv0 + 4 * g4;
+#if !AE_EVEN_KV
+    if (kv0 + AE_TILE > p.seqlen_kv) {
+#pragma unroll
+      for (int e = 0; e < AE_NS; e++)
+        s[e] = (ctx.kv_base + ae_kv_off(e) < p.seqlen_kv) ? s[e] : AE_NEG_INF;
+    }
+#endif
+    ae_score_mod<AE_NS>(s, ctx, cust);
+    float o_scale = ae_online_fwd<AE_NS>(s, st, ctx, cust);
+#if !AE_EVEN_KV
+    if (kv0 + AE_TILE > p.seqlen_kv) {
+#pragma unroll
+      for (int e = 0; e < AE_NS; e++)
+        s[e] = (ctx.kv_base + ae_kv_off(e) < p.seqlen_kv) ? s[e] : 0.f;
+    }
+#endif
+    // P as B operand of O^T += V^T P^T: slot j<4 is kv 4*g4+j, slot j>=4 is kv 16+4*g4+(j-4)
+    ae_elem8 pf;
+#pragma unroll
+    for (int t = 0; t < 8; t++) pf[t] = (ae_elem)s[t];
+
+#if !AE_O_SCALE_ONE
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) oacc[db][r] *= o_scale;
+#else
+    (void)o_scale;
+#endif
+
+    // make this wave's LDS writes visible to its own transpose reads
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++) {
+      ae_lds_byte* a0 = vs + v_rd_off + db * 32;
+      ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) ae_s16x4*)a0);
+      ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (__attribute__((address_space(3))) ae_s16x4*)(a0 + 16 * AE_VSTR));
+      ae_elem8 vf = __builtin_bit_cast(
+          ae_elem8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      oacc[db] = ae_mfma16(vf, pf, oacc[db]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    if (more) {
+#pragma unroll
+      for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+        for (int ks = 0; ks < AE_NKS; ks++) kf[rb][ks] = kf_next[rb][ks];
+    }
+  }
+
+  // ---- per-split epilogue: normalise within the split, emit its final rowscales ------------------
+  float o[AE_NO];
+#pragma unroll
+  for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) o[db * 4 + r] = oacc[db][r];
+  float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+  frs[0] = 0.f;
+  if (my_tiles > 0) {
+    ae_epilogue<AE_NO>(o, st, frs, ctx, cust);
+  } else {
+    // this split saw no kv at all: contributes nothing to the merge
+#pragma unroll
+    for (int e = 0; e < AE_NO; e++) o[e] = 0.f;
+#pragma unroll
+    for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
+  }
+  if (head_ok) {
+    const int64_t row = ((int64_t)b * p.heads_q + hq) * p.num_splits + split;
+    float* po = p.partial_o + row * AE_DV;
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++) {
+      ae_f32x4 w = {o[db * 4 + 0], o[db * 4 + 1], o[db * 4 + 2], o[db * 4 + 3]};
+      *(ae_f32x4*)(po + db * 16 + g4 * 4) = w;
+    }
+    if (g4 == 0) {
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+        p.partial_rs[(int64_t)i * p.batch * p.heads_q * p.num_splits + row] = frs[i];
+    }
+  }
+}
+
+// Merge of the per-split partials: grid (Hq, B), one workgroup per output row.
+// out[b,0,h,:] = sum_k partial_o[b,h,k,:] * o_scale[k], o_scale = combine(final_rowscales[k])
+// (attn_gqa_decode_tl.py:224-266; generic form core/template/tl_template/attn/attn_decode_tl.py:184-189).
+extern "C" __global__ __launch_bounds__(AE_COMBINE_THREADS)
+void ae_decode_combine_kernel(const ae_attn_params p) {
+  const int h = blockIdx.x;
+  const int b = blockIdx.y;
+  const int64_t row = ((int64_t)b * p.heads_q + h) * AE_NSPLIT;
+  float rs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1][AE_NSPLIT];
+#pragma unroll
+  for (int i = 0; i < AE_N_ROWSCALES; i++)
+#pragma unroll
+    for (int k = 0; k < AE_NSPLIT; k++)
+      rs[i][k] = p.partial_rs[(int64_t)i * p.batch * p.heads_q * AE_NSPLIT + row + k];
+  float w[AE_NSPLIT];
+  float merged[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+  ae_combine(rs, w, merged);
+  ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;
+  for (int dv = threadIdx.x; dv < AE_DV; dv += AE_COMBINE_THREADS) {
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < AE_NSPLIT; k++) acc += p.partial_o[(row + k) * AE_DV + dv] * w[k];
+    optr[dv] = (ae_elem)acc;
+  }
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < AE_N_ROWSCALES; i++)
+      if (p.rowscale_out[i]) p.rowscale_out[i][(int64_t)b * p.heads_q + h] = merged[i];
+  }
+}

@@ -66,23 +66,43 @@ AE_DEV float ae_tanh(float x) {
 AE_DEV float ae_abs(float x) { return __builtin_fabsf(x); }
 AE_DEV float ae_max(float a, float b) { return __builtin_fmaxf(a, b); }
 
-// ---- lane-pair exchange -----------------------------------------------------------------
-// In the transposed score layout one query row lives in lanes l and l^32. permlane32_swap
-// with both operands equal returns (value of the low half, value of the high half) in
-// every lane of the pair.
-AE_DEV float ae_pair_max(float v) {
+// ---- exchange between the lanes that share one query row -----------------------------------
+// AE_LAYOUT 0 (prefill, 32x32x16 MFMA, S^T accumulators): a row lives in lanes l and l^32.
+//   permlane32_swap with both operands equal returns (value of the low half, value of the
+//   high half) in every lane of the pair.
+// AE_LAYOUT 1 (decode, 16x16x32 MFMA): a row (one query head) lives in lanes l, l^16, l^32, l^48.
+#ifndef AE_LAYOUT
+#define AE_LAYOUT 0
+#endif
+AE_DEV float ae_swap32_lo_hi(float v, float& hi) {
   unsigned u = __builtin_bit_cast(unsigned, v);
   auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __builtin_fmaxf(__builtin_bit_cast(float, (unsigned)r[0]),
-                         __builtin_bit_cast(float, (unsigned)r[1]));
+  hi = __builtin_bit_cast(float, (unsigned)r[1]);
+  return __builtin_bit_cast(float, (unsigned)r[0]);
 }
-AE_DEV float ae_pair_sum(float v) {
-  unsigned u = __builtin_bit_cast(unsigned, v);
-  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+AE_DEV float ae_xor16(float v) {
+  int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  int r = __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, v));
+  return __builtin_bit_cast(float, r);
+}
+AE_DEV float ae_group_max(float v) {
+#if AE_LAYOUT == 1
+  v = __builtin_fmaxf(v, ae_xor16(v));
+#endif
+  float hi;
+  float lo = ae_swap32_lo_hi(v, hi);
+  return __builtin_fmaxf(lo, hi);
+}
+AE_DEV float ae_group_sum(float v) {
+#if AE_LAYOUT == 1
+  v = v + ae_xor16(v);
+#endif
+  float hi;
+  float lo = ae_swap32_lo_hi(v, hi);
+  return lo + hi;
 }
 
-// ---- row reductions over the lane's slice of a score row + its partner lane ------------
+// ---- row reductions over the lane's slice of a score row + the lanes sharing the row --------
 // (ReduceMax / ReduceSum / ReduceAbsSum over dim=1 of the [block_M, block_N] tile,
 //  core/codegen/tl_gen.py:9-21.)
 template <int N>
@@ -90,7 +110,7 @@ AE_DEV float ae_row_max(const float (&s)[N]) {
   float m = s[0];
 #pragma unroll
   for (int e = 1; e < N; e++) m = __builtin_fmaxf(m, s[e]);
-  return ae_pair_max(m);
+  return ae_group_max(m);
 }
 template <int N>
 AE_DEV float ae_row_sum(const float (&s)[N]) {
@@ -105,7 +125,7 @@ AE_DEV float ae_row_sum(const float (&s)[N]) {
   }
 #pragma unroll
   for (int e = N & ~3; e < N; e++) a0 += s[e];
-  return ae_pair_sum((a0 + a1) + (a2 + a3));
+  return ae_group_sum((a0 + a1) + (a2 + a3));
 }
 template <int N>
 AE_DEV float ae_row_abssum(const float (&s)[N]) {
@@ -117,7 +137,30 @@ AE_DEV float ae_row_abssum(const float (&s)[N]) {
   }
 #pragma unroll
   for (int e = N & ~1; e < N; e++) a0 += __builtin_fabsf(s[e]);
-  return ae_pair_sum(a0 + a1);
+  return ae_group_sum(a0 + a1);
+}
+
+// ---- reductions over the split axis (ColReduce*, used by OnlineFunc.combine) -----------------
+template <int N>
+AE_DEV float ae_arr_max(const float (&s)[N]) {
+  float m = s[0];
+#pragma unroll
+  for (int e = 1; e < N; e++) m = __builtin_fmaxf(m, s[e]);
+  return m;
+}
+template <int N>
+AE_DEV float ae_arr_sum(const float (&s)[N]) {
+  float a = 0.f;
+#pragma unroll
+  for (int e = 0; e < N; e++) a += s[e];
+  return a;
+}
+template <int N>
+AE_DEV float ae_arr_abssum(const float (&s)[N]) {
+  float a = 0.f;
+#pragma unroll
+  for (int e = 0; e < N; e++) a += __builtin_fabsf(s[e]);
+  return a;
 }
 
 // Per-row context handed to the functors.
@@ -128,9 +171,15 @@ struct ae_ctx {
   int kv_base;  // absolute kv position of element 0 of the lane's slice in the current tile
 };
 
-// kv offset (relative to ae_ctx::kv_base) of element e of a lane's slice of a score row:
-// the slice is NB accumulator blocks of 16; block nb covers kv 32*nb .. 32*nb+31 and
-// register r of the half-wave hf holds kv 8*(r/4) + 4*hf + r%4 (hf is folded into kv_base).
+// kv offset (relative to ae_ctx::kv_base) of element e of a lane's slice of a score row.
+// AE_LAYOUT 0: the slice is NB accumulator blocks of 16; block nb covers kv 32*nb .. 32*nb+31 and
+//   register r of half-wave hf holds kv 8*(r/4) + 4*hf + r%4 (4*hf is folded into kv_base).
+// AE_LAYOUT 1: blocks of 4; block rb covers kv 16*rb .. 16*rb+15 and register r of lane group g
+//   holds kv 4*g + r (4*g is folded into kv_base).
+#if AE_LAYOUT == 1
+AE_DEV constexpr int ae_kv_off(int e) { return (e >> 2) * 16 + (e & 3); }
+#else
 AE_DEV constexpr int ae_kv_off(int e) { return (e >> 4) * 32 + ((e & 15) >> 2) * 8 + (e & 3); }
+#endif
 
 #endif  // AE_DEVICE_H

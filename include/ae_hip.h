@@ -174,9 +174,11 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
  *
  * ae_prefill_fwd: one workgroup per (q-tile, q-head, batch) -- the grid of
  *   attn_tl.py:86 -- flattened to 1-D so the kernel can order heavy causal tiles first.
- * ae_decode_fwd:  split-KV pass, grid (num_splits, ceil(Hq/Hkv / block_m)*Hkv, B), followed by
- *   the combine kernel, grid (Hq, B) (attn_gqa_decode_tl.py:150-151, 224-266).
- *   `combine` may be NULL only when num_splits == 1 and the split kernel writes `out`.
+ * ae_decode_fwd:  split-KV pass followed by the combine kernel, grid (Hq, B)
+ *   (attn_gqa_decode_tl.py:150-151, 224-266). Every WAVE of the split kernel produces one partial,
+ *   so its grid is (num_splits / (threads/64), ceil(Hq/Hkv / block_m)*Hkv, B); kv_per_split is the
+ *   share of one partial and must be a multiple of block_n; combine_cfg->block_n is the number of
+ *   splits the combine kernel was compiled for and must equal num_splits.
  */
 int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream);
 int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
