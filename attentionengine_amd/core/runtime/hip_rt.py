@@ -106,6 +106,8 @@ _SIGNATURES = {
     "ae_prefill_fwd": (C.c_int, [_VP, C.POINTER(AttnParams), C.POINTER(TileCfg), _VP]),
     "ae_decode_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
                                 C.POINTER(TileCfg), _VP]),
+    "ae_mla_decode_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
+                                    C.POINTER(TileCfg), _VP]),
     "ae_event_create": (C.c_int, [C.POINTER(_VP)]),
     "ae_event_record": (C.c_int, [_VP, _VP]),
     "ae_event_elapsed_ms": (C.c_int, [_VP, _VP, C.POINTER(C.c_float)]),
@@ -239,6 +241,7 @@ def compile_module(template: str, headers: dict, arch: str = None, use_cache: bo
     all_headers = {
         "ae_hip.h": _read(osp.join(INCLUDE_DIR, "ae_hip.h")),
         "ae_device.h": _read(osp.join(KERNEL_DIR, "ae_device.h")),
+        "ae_combine.h": _read(osp.join(KERNEL_DIR, "ae_combine.h")),
     }
     all_headers.update(headers)
     hsh = hashlib.sha256()
@@ -309,3 +312,9 @@ def decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
     _check(lib().ae_decode_fwd(split.handle, combine.handle if combine else None, C.byref(params),
                                C.byref(cfg), C.byref(combine_cfg) if combine_cfg else None,
                                _VP(stream)))
+
+
+def mla_decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
+                   combine_cfg: TileCfg, stream: int = 0):
+    _check(lib().ae_mla_decode_fwd(split.handle, combine.handle, C.byref(params), C.byref(cfg),
+                                   C.byref(combine_cfg), _VP(stream)))

@@ -374,6 +374,48 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
   return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
 }
 
+int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                      const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
+  if (!split || !combine || !combine_cfg)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: kernel/cfg is NULL");
+  int rc = check_common("ae_mla_decode_fwd", p, cfg);
+  if (rc) return rc;
+  if (!p->q2 || !p->k2)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: rope pointers q2/k2 are NULL");
+  if (p->seqlen_q != 1)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: seqlen_q=%d (decode handles one query token)",
+                p->seqlen_q);
+  if (p->num_splits <= 0 || p->kv_per_split <= 0 ||
+      (int64_t)p->num_splits * p->kv_per_split < p->seqlen_kv)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: %d splits of %d do not cover Skv=%d",
+                p->num_splits, p->kv_per_split, p->seqlen_kv);
+  if (combine_cfg->block_n != p->num_splits)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: combine kernel built for %d splits, got %d",
+                combine_cfg->block_n, p->num_splits);
+  if (!p->partial_o || !p->partial_rs)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: split-KV work buffers are NULL");
+  if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: bad combine workgroup size %d",
+                combine_cfg->threads);
+  for (int i = 0; i < combine_cfg->n_rowscales; i++)
+    if (!p->rowscale_out[i])
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: rowscale_out[%d] is NULL", i);
+  // 1-D grid: head tiles of one (batch, kv head, split) sit 8 ids apart (same XCD); the
+  // (batch, kv head, split) count is padded to a multiple of 8, surplus workgroups exit at once.
+  int group = p->heads_q / p->heads_kv;
+  int64_t n_ht = (group + cfg->block_m - 1) / cfg->block_m;
+  int64_t units = (int64_t)p->batch * p->heads_kv * p->num_splits;
+  int64_t total = ((units + 7) / 8) * 8 * n_ht;
+  if (total > 0x7fffffffll) return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: grid too large");
+  uint32_t grid[3] = {(uint32_t)total, 1, 1};
+  uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
+  rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+  if (rc) return rc;
+  uint32_t cgrid[3] = {(uint32_t)p->heads_q, (uint32_t)p->batch, 1};
+  uint32_t cblock[3] = {(uint32_t)combine_cfg->threads, 1, 1};
+  return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
+}
+
 int ae_event_create(ae_event** out) {
   if (!out) return fail(AE_ERR_INVALID_ARG, "ae_event_create: out is NULL");
   *out = nullptr;

@@ -1,0 +1,37 @@
+// Merge kernel of the split-KV decode paths (shared by ae_decode.hip and ae_mla_decode.hip).
+// Needs AE_DV, AE_NSPLIT, AE_N_ROWSCALES, AE_COMBINE_THREADS and the generated ae_combine().
+#ifndef AE_COMBINE_H
+#define AE_COMBINE_H
+
+// Merge of the per-split partials: grid (Hq, B), one workgroup per output row.
+// out[b,0,h,:] = sum_k partial_o[b,h,k,:] * o_scale[k], o_scale = combine(final_rowscales[k])
+// (attn_gqa_decode_tl.py:224-266; generic form core/template/tl_template/attn/attn_decode_tl.py:184-189).
+extern "C" __global__ __launch_bounds__(AE_COMBINE_THREADS)
+void ae_decode_combine_kernel(const ae_attn_params p) {
+  const int h = blockIdx.x;
+  const int b = blockIdx.y;
+  const int64_t row = ((int64_t)b * p.heads_q + h) * AE_NSPLIT;
+  float rs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1][AE_NSPLIT];
+#pragma unroll
+  for (int i = 0; i < AE_N_ROWSCALES; i++)
+#pragma unroll
+    for (int k = 0; k < AE_NSPLIT; k++)
+      rs[i][k] = p.partial_rs[(int64_t)i * p.batch * p.heads_q * AE_NSPLIT + row + k];
+  float w[AE_NSPLIT];
+  float merged[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+  ae_combine(rs, w, merged);
+  ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;
+  for (int dv = threadIdx.x; dv < AE_DV; dv += AE_COMBINE_THREADS) {
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < AE_NSPLIT; k++) acc += p.partial_o[(row + k) * AE_DV + dv] * w[k];
+    optr[dv] = (ae_elem)acc;
+  }
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < AE_N_ROWSCALES; i++)
+      if (p.rowscale_out[i]) p.rowscale_out[i][(int64_t)b * p.heads_q + h] = merged[i];
+  }
+}
+
+#endif  // AE_COMBINE_H

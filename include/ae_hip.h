@@ -184,6 +184,16 @@ int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg
 int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                   const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
 
+/*
+ * ae_mla_decode_fwd: shared-latent-KV (MLA) decode. K = [k | k2] (latent | rope), q = [q | q2],
+ *   V = the first head_dim_v columns of k. Stands where the reference calls its TileLang MLA
+ *   kernel (mla_decode_tl.py:326-335) or `fwd_kvcache_mla`
+ *   (cute_template_kvshared/flash_api.cpp:61-210). Every workgroup covers cfg->block_m query heads
+ *   of one (batch, kv head, split); 1-D grid ordered so workgroups sharing a KV range run on one XCD.
+ */
+int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                      const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
+
 /* ---- timing on the launch stream ------------------------------------------------- */
 int ae_event_create(ae_event** out);
 int ae_event_record(ae_event* e, void* stream);

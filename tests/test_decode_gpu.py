@@ -74,3 +74,58 @@ def test_gqa_decode_sigmoid(cuda_device):
     out = mod(q.cuda(), k.cuda(), v.cuda())
     ref = R.sigmoid_attention(q, k, v, bias=-6.0)
     assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+
+
+def _mla_inputs(B, H, G, S, DV, DPE, dtype, seed=0):
+    """q, q_pe, kv, k_pe generated on the CPU in that order."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, 1, H, DV, generator=g).to(dtype)
+    q_pe = torch.randn(B, 1, H, DPE, generator=g).to(dtype)
+    kv = torch.randn(B, S, G, DV, generator=g).to(dtype)
+    k_pe = torch.randn(B, S, G, DPE, generator=g).to(dtype)
+    return q, q_pe, kv, k_pe
+
+
+def _mla_engine(B, H, G, S, D, DV, dtype, scale, **kw):
+    meta = (meta_tensor(B, H, 1, D, dtype=dtype), meta_tensor(B, G, S, D, dtype=dtype),
+            meta_tensor(B, G, S, DV, dtype=dtype))
+    return AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(scale), mask_mod=None,
+                           online_func=C.OnlineSoftmax(), kv_shared=True, **kw)
+
+
+@pytest.mark.parametrize("B,H,G,S,dtype", [
+    (2, 128, 1, 512, torch.bfloat16),     # DeepSeek-V3 head layout (BASELINE config 5, short KV)
+    (1, 128, 1, 4096, torch.bfloat16),    # attn_script/mla_decode.py shape, one batch entry -> many splits
+    (3, 16, 1, 200, torch.float16),       # fewer heads than a workgroup covers, ragged KV
+    (2, 64, 2, 96, torch.bfloat16),       # two latent heads
+])
+def test_mla_decode_tl_convention(cuda_device, B, H, G, S, dtype):
+    D, DV = 576, 512
+    scale = 1 / math.sqrt(192)            # BASELINE config 5 scale
+    print(f"case mla B{B} H{H} G{G} S{S} {dtype}", flush=True)
+    q, q_pe, kv, k_pe = _mla_inputs(B, H, G, S, DV, D - DV, dtype)
+    mod = _mla_engine(B, H, G, S, D, DV, dtype, scale)
+    out = mod(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda())
+    ref, lse = R.mla_decode(q[:, 0], q_pe[:, 0], kv, k_pe, scale=scale)
+    assert out.shape == (B, 1, H, DV) and out.dtype == dtype
+    assert (out[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"][:, :, 0].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
+def test_mla_decode_cute_convention(cuda_device):
+    """mod(q [B,1,H,576], paged kv cache [B*S/64, 64, 1, 576]) -> (out, lse), as in
+    attn_script/mla_decode_cute.py:286-303; lse checked with the script's cos-diff bound (107-113)."""
+    B, H, G, S, D, DV = 2, 128, 1, 1024, 576, 512
+    dtype = torch.bfloat16
+    scale = 1 / math.sqrt(D)
+    q, q_pe, kv, k_pe = _mla_inputs(B, H, G, S, DV, D - DV, dtype, seed=3)
+    mod = _mla_engine(B, H, G, S, D, DV, dtype, scale, backend="cute")
+    q_full = torch.cat([q, q_pe], -1)
+    cache = torch.cat([kv, k_pe], -1).reshape(B * S // 64, 64, G, D).contiguous()
+    out, lse = mod(q_full.cuda(), cache.cuda())
+    ref, lref = R.mla_decode(q[:, 0], q_pe[:, 0], kv, k_pe, scale=scale)
+    assert (out[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL
+    x, y = lse[:, :, 0].double().cpu(), lref.double()
+    cos_diff = 1 - 2 * (x * y).sum().item() / max((x * x + y * y).sum().item(), 1e-12)
+    assert cos_diff < 1e-5
+    assert (x - y).abs().max().item() <= LSE_TOL
