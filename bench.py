@@ -1,0 +1,224 @@
+"""Benchmark of the fused attention forward path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
+
+A "step" is one forward pass of the hot path over one batch of synthetic input that is already
+resident in HBM.  The headline workload (default) is the configuration the metric is quoted on:
+causal softmax prefill, fp16, B=2 H=32 S=4096 D=DV=128 ("c2_causal").  Rank 0 prints ONE JSON line.
+Its `roofline` object prices the dominant kernel of the workload against MI355X's published peaks
+(dense fp16/bf16 MFMA 2.5 PFLOP/s, HBM 8 TB/s) using the ALGORITHMIC flops / bytes of one launch and
+the average launch duration measured with HIP events on the launch stream; `cpu_baseline` is the
+CPU oracle (a restatement of the reference's eager PyTorch path) timed on the host cores on a
+bounded sample of the same workload.  The remaining benchmark configurations are measured too and
+reported inside the same line under `other_configs` (disable with --no-extra).
+
+FLOP / byte conventions are the reference's: prefill 2*B*H*Sq*Skv*(D+DV), halved if causal
+(attention_engine/benchmark/bench_utils.py:1185-1186); GQA decode bytes = K+V streamed; MLA
+bytes = B*Skv*D*itemsize, flops = 2*B*H*Skv*(D+DV) (attn_script/mla_decode.py:129).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "attentionengine_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_MFMA_TFLOPS = 2500.0   # dense fp16 / bf16
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (engine key in __graft_entry__.benchmark_engines, kind)
+    "c2_causal": ("c2_softmax_causal", "prefill"),
+    "c2_full": ("c2_softmax_full", "prefill"),
+    "c3_sigmoid": ("c3_sigmoid", "prefill"),
+    "c4_gqa_decode": ("c4_gqa_decode", "gqa_decode"),
+    "c5_mla_decode": ("c5_mla_decode", "mla_decode"),
+}
+
+
+def _inputs(name, device):
+    """Synthetic N(0,1) inputs of the workload's shape, generated on the CPU with seed 0 in the
+    order q, k, v (MLA: q, q_pe, kv, k_pe), rounded to the compute dtype, copied to the GPU."""
+    import torch
+    g = torch.Generator().manual_seed(0)
+
+    def rn(*shape, dtype):
+        return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype).to(device)
+    f16, bf16 = torch.float16, torch.bfloat16
+    if name in ("c2_causal", "c2_full", "c3_sigmoid"):
+        B, H, S, D = 2, 32, 4096, 128
+        args = [rn(B, S, H, D, dtype=f16), rn(B, S, H, D, dtype=f16), rn(B, S, H, D, dtype=f16)]
+        if name == "c3_sigmoid":
+            args.append(torch.tensor([-math.log(S)], dtype=torch.float32, device=device))
+        flops = 4.0 * B * H * S * S * D * (0.5 if name == "c2_causal" else 1.0)
+        return args, {"flops": flops, "bytes": 4.0 * B * S * H * D * 2,
+                      "shape": {"B": B, "H": H, "S": S, "D": D, "DV": D}, "dtype": "fp16"}
+    if name == "c4_gqa_decode":
+        B, Hq, Hkv, Skv, D = 64, 32, 8, 8192, 128
+        args = [rn(B, 1, Hq, D, dtype=f16), rn(B, Skv, Hkv, D, dtype=f16), rn(B, Skv, Hkv, D, dtype=f16)]
+        return args, {"flops": 4.0 * B * Hq * Skv * D, "bytes": 2.0 * B * Skv * Hkv * D * 2,
+                      "shape": {"B": B, "Hq": Hq, "Hkv": Hkv, "Skv": Skv, "D": D, "DV": D}, "dtype": "fp16"}
+    if name == "c5_mla_decode":
+        B, H, Skv, D, DV = 128, 128, 4096, 576, 512
+        args = [rn(B, 1, H, DV, dtype=bf16), rn(B, 1, H, D - DV, dtype=bf16),
+                rn(B, Skv, 1, DV, dtype=bf16), rn(B, Skv, 1, D - DV, dtype=bf16)]
+        return args, {"flops": 2.0 * B * H * Skv * (D + DV), "bytes": 1.0 * B * Skv * D * 2,
+                      "shape": {"B": B, "Hq": H, "Hkv": 1, "Skv": Skv, "D": D, "DV": DV}, "dtype": "bf16"}
+    raise KeyError(name)
+
+
+def measure(name, steps, warmup):
+    """Time `steps` forward passes of workload `name`; returns a result dict."""
+    import torch
+    import __graft_entry__ as G
+    from core.runtime import hip_rt as rt
+    dev = torch.device("cuda:0")
+    key, kind = WORKLOADS[name]
+    mod = G.benchmark_engines({key})[key]
+    args, info = _inputs(name, dev)
+    for _ in range(max(1, warmup)):
+        mod(*args)
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    e0, e1 = rt.Event(), rt.Event()
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        mod(*args)
+    e1.record(stream)
+    ev_ms = e0.elapsed_ms(e1) / steps          # synchronises on e1
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    res = {"workload": name, "kind": kind, "ms_per_step": wall_ms, "kernel_ms": ev_ms, **info}
+    res["tflops"] = info["flops"] / (wall_ms * 1e-3) / 1e12
+    res["gbs"] = info["bytes"] / (wall_ms * 1e-3) / 1e9
+    if kind == "prefill":
+        ach = info["flops"] / (ev_ms * 1e-3) / 1e12
+        res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                           "frac": ach / PEAK_MFMA_TFLOPS, "traffic": None}
+    else:
+        ach = info["bytes"] / (ev_ms * 1e-3) / 1e9
+        res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                           "frac": ach / PEAK_HBM_GBS, "traffic": None}
+        if kind == "mla_decode":
+            res["mfma_frac"] = info["flops"] / (ev_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS
+    del args, mod
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(name):
+    """The CPU oracle on a bounded sample of the workload (one batch entry; heads in chunks so the
+    [heads, S, S] fp32 score tensor stays below ~1 GiB), fp32 compute on the rounded inputs."""
+    import torch
+    from oracle import attention_ref as R
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+    if name in ("c2_causal", "c2_full", "c3_sigmoid"):
+        H, S, D, chunk = 32, 4096, 128, 4
+        q = torch.randn(1, S, H, D, generator=g).half().float()
+        k = torch.randn(1, S, H, D, generator=g).half().float()
+        v = torch.randn(1, S, H, D, generator=g).half().float()
+        causal = name == "c2_causal"
+
+        def run():
+            for h0 in range(0, H, chunk):
+                sl = slice(h0, h0 + chunk)
+                if name == "c3_sigmoid":
+                    R.sigmoid_attention(q[:, :, sl], k[:, :, sl], v[:, :, sl], bias=-math.log(S))
+                else:
+                    R.softmax_attention(q[:, :, sl], k[:, :, sl], v[:, :, sl], causal=causal)
+        flops = 4.0 * H * S * S * D * (0.5 if causal else 1.0)
+        R.softmax_attention(q[:, :256, :1], k[:, :256, :1], v[:, :256, :1])   # warm the thread pool
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": f"oracle/attention_ref.py on 1 of 2 batch entries (32 heads, S=4096, D=128, "
+                          f"fp32), {dt:.2f} s, reference flop convention"}
+    if name == "c4_gqa_decode":
+        nb, Hq, Hkv, Skv, D = 8, 32, 8, 8192, 128
+        q = torch.randn(nb, 1, Hq, D, generator=g).half().float()
+        k = torch.randn(nb, Skv, Hkv, D, generator=g).half().float()
+        v = torch.randn(nb, Skv, Hkv, D, generator=g).half().float()
+        R.softmax_attention(q[:1], k[:1], v[:1])
+        t0 = time.perf_counter()
+        R.softmax_attention(q, k, v)
+        dt = time.perf_counter() - t0
+        by = 2.0 * nb * Skv * Hkv * D * 2
+        return {"value": by / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"oracle on 8 of 64 batch entries (fp32 compute, fp16-sized KV bytes), {dt:.2f} s"}
+    if name == "c5_mla_decode":
+        nb, H, Skv, D, DV = 8, 128, 4096, 576, 512
+        q = torch.randn(nb, H, DV, generator=g).bfloat16().float()
+        qpe = torch.randn(nb, H, D - DV, generator=g).bfloat16().float()
+        kv = torch.randn(nb, Skv, 1, DV, generator=g).bfloat16().float()
+        kpe = torch.randn(nb, Skv, 1, D - DV, generator=g).bfloat16().float()
+        R.mla_decode(q[:1], qpe[:1], kv[:1], kpe[:1])
+        t0 = time.perf_counter()
+        R.mla_decode(q, qpe, kv, kpe, scale=1 / math.sqrt(192))
+        dt = time.perf_counter() - t0
+        by = 1.0 * nb * Skv * D * 2
+        return {"value": by / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+                "sample": f"oracle on 8 of 128 batch entries (fp32 compute, bf16-sized KV bytes), {dt:.2f} s"}
+    raise KeyError(name)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2_causal", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the attention forward path on ONE GPU; "
+              "--gpus N with N > 1 is not supported (the path shards over batch/heads with no "
+              "exchange, so N GPUs are N independent copies of this measurement).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU fallback for the measured path.", file=sys.stderr)
+        sys.exit(3)
+    from core.runtime import hip_rt as rt
+    info = rt.device_info(0)
+
+    head = measure(a.workload, a.steps, a.warmup)
+    unit = head["roofline"]["unit"]
+    value = head["tflops"] if unit == "TFLOP/s" else head["gbs"]
+    line = {
+        "metric": "prefill TFLOP/s (causal S=4096 D=128 fp16) + decode GB/s; % of MI355X peak",
+        "value": value, "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": a.workload, **head["shape"]},
+        "roofline": head["roofline"],
+        "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
+                   "clock_khz": info["clock_khz"]},
+    }
+    if "mfma_frac" in head:
+        line["mfma_frac"] = head["mfma_frac"]
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(a.workload)
+    if not a.no_extra:
+        others = {}
+        for name in WORKLOADS:
+            if name == a.workload:
+                continue
+            r = measure(name, max(5, a.steps // 2), max(2, a.warmup // 2))
+            others[name] = {"ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
+                            "tflops": r["tflops"], "gbs": r["gbs"], "roofline": r["roofline"],
+                            **({"mfma_frac": r["mfma_frac"]} if "mfma_frac" in r else {})}
+        line["other_configs"] = others
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
