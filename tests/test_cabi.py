@@ -1,0 +1,123 @@
+"""The C-ABI library loads, exports every symbol include/ae_hip.h declares, compiles for gfx950
+without a GPU, caches code objects, and fails loudly (status + message, no exit) on bad input."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from core.runtime import hip_rt as rt
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ae_hip.h")
+
+KERNEL = r'''
+#include "ae_hip.h"
+extern "C" __global__ void ae_probe(const ae_attn_params p) {
+  if (threadIdx.x == 0) ((float*)p.out)[0] = (float)sizeof(ae_attn_params);
+}
+'''
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ae_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    names = _declared_functions()
+    assert "ae_compile" in names and "ae_prefill_fwd" in names and "ae_mla_decode_fwd" in names
+    lib = ctypes.CDLL(rt.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in ae_hip.h but not exported"
+    assert sorted(rt.EXPORTED_SYMBOLS) == names
+    assert rt.lib().ae_abi_version() == 1
+
+
+def test_struct_layout_matches_the_header():
+    """sizeof(ae_attn_params) as the device compiler sees it == the ctypes mirror."""
+    # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints
+    assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16
+    assert ctypes.sizeof(rt.TileCfg) == 4 * 12
+
+
+def _compile(src, opts=()):
+    lib = rt.lib()
+    handle = ctypes.c_void_p()
+    hdr = open(HEADER).read().encode()
+    names = (ctypes.c_char_p * 1)(b"ae_hip.h")
+    srcs = (ctypes.c_char_p * 1)(hdr)
+    copts = (ctypes.c_char_p * max(1, len(opts)))(*[o.encode() for o in opts]) if opts else None
+    rc = lib.ae_compile(src.encode(), b"probe.hip", b"gfx950", copts, len(opts), names, srcs, 1,
+                        ctypes.byref(handle))
+    return rc, handle
+
+
+def test_compile_save_load_roundtrip(tmp_path):
+    lib = rt.lib()
+    rc, h = _compile(KERNEL, ["-O3"])
+    assert rc == 0, lib.ae_last_error()
+    data, size = ctypes.c_void_p(), ctypes.c_size_t()
+    assert lib.ae_module_code(h, ctypes.byref(data), ctypes.byref(size)) == 0
+    code = ctypes.string_at(data, size.value)
+    assert code[:4] == b"\x7fELF" and size.value > 1000
+    path = str(tmp_path / "probe.hsaco").encode()
+    assert lib.ae_module_save(h, path) == 0
+    h2 = ctypes.c_void_p()
+    assert lib.ae_module_load(path, ctypes.byref(h2)) == 0
+    assert lib.ae_module_code(h2, ctypes.byref(data), ctypes.byref(size)) == 0
+    assert ctypes.string_at(data, size.value) == code
+    lib.ae_module_free(h)
+    lib.ae_module_free(h2)
+
+
+def test_compile_error_returns_status_and_log():
+    lib = rt.lib()
+    rc, h = _compile("extern \"C\" __global__ void k() { this is not C++; }")
+    assert rc == 2 and not h.value
+    msg = lib.ae_last_error().decode()
+    assert "hipRTC compile failed" in msg and "error" in msg
+
+
+def test_bad_arguments_fail_without_exiting(tmp_path):
+    lib = rt.lib()
+    assert lib.ae_compile(None, None, None, None, 0, None, None, 0, None) == 1
+    h = ctypes.c_void_p()
+    assert lib.ae_module_load(str(tmp_path / "missing.hsaco").encode(), ctypes.byref(h)) == 4
+    assert b"cannot open" in lib.ae_last_error()
+    p, cfg = rt.AttnParams(), rt.TileCfg()
+    assert lib.ae_prefill_fwd(None, ctypes.byref(p), ctypes.byref(cfg), None) == 1
+    assert lib.ae_device_info(0, None) == 1
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")
+def test_no_gpu_is_reported_not_hidden():
+    lib = rt.lib()
+    assert lib.ae_device_count() == 0
+    rc, h = _compile(KERNEL)
+    assert rc == 0
+    k = ctypes.c_void_p()
+    assert lib.ae_module_get_kernel(h, b"ae_probe", ctypes.byref(k)) == 3     # AE_ERR_HIP
+    assert b"failed" in lib.ae_last_error()
+    lib.ae_module_free(h)
+    with pytest.raises(rt.AEError):
+        rt.device_info(0)
+
+
+def test_code_object_cache_is_keyed_by_content(tmp_path, monkeypatch):
+    monkeypatch.setenv("AE_CACHE_DIR", str(tmp_path))
+    import __graft_entry__ as G
+    (template, headers) = G.representative_headers()[2]
+    rt._modules.clear()
+    m1 = rt.compile_module(template, headers)
+    assert not m1.from_cache and len(os.listdir(tmp_path)) == 1
+    rt._modules.clear()
+    m2 = rt.compile_module(template, headers)
+    assert m2.from_cache and m2.code() == m1.code()
+    headers2 = dict(headers)
+    headers2["ae_config.h"] = headers["ae_config.h"].replace("#define AE_NSPLIT 16", "#define AE_NSPLIT 8")
+    m3 = rt.compile_module(template, headers2)
+    assert not m3.from_cache and m3.key != m1.key
+    rt._modules.clear()

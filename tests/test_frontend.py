@@ -1,0 +1,204 @@
+"""CPU tests of the host side: symbolic tracer, mask utilities (product code vs the oracle's brute
+force), mask_mod lowering, functor emission + hipRTC compilation (no GPU needed), engine dispatch
+and error behaviour."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import attn_cases as C
+from attn_engine import AttentionEngine, OnlineFunc
+from core import CustomIO, SymbolicArray, SymbolScalar, Var, create_block_mask, create_mask, meta_tensor
+from core.lower import lower as L
+from core.lower.lower_decode import lower_combine
+from core.lower.mask import lower_mask_mod, plan_mask
+from core.transform.core import (SymbolicConst, create_block_idx, is_causal_mask, is_less_causal_mask)
+from oracle import masks as M
+
+
+# ---- tracer ---------------------------------------------------------------------------------------
+def test_tracer_builds_the_softmax_graph():
+    """Node sequence of OnlineSoftmax.online_fwd as traced from attn_script/mha.py:47-63."""
+    on = C.OnlineSoftmax()
+    scores = SymbolicArray("scores", Var("scores"), shape_idx=["block_M", "block_N"])
+    b = h = q = SymbolScalar("b", Var("b"))
+    s2, rows, o_scale = on.online_fwd(scores, on.online_rowscales, b, h, q)
+    assert s2.code.type == "Exp" and s2.prev[0].code.type == "Sub"
+    assert s2.shape_idx == ["block_M", "block_N"]
+    m_new = rows["m"]
+    assert m_new.code.type == "Max" and m_new.prev[1].code.type == "ReduceMax"
+    assert m_new.prev[1].shape_idx == ["block_M"] and m_new.prev[1].varname == "scores_max_0"
+    assert rows["r"].code.type == "Add" and rows["r"].prev[1].code.type == "ReduceSum"
+    assert o_scale.code.type == "Exp" and o_scale.prev[0].prev[1] is m_new
+    # naming rule <varname>[_<suffix>]_<use count>
+    assert m_new.varname == "m_0"
+
+
+def test_python_numbers_become_constants_on_either_side():
+    x = SymbolScalar("x", Var("x"))
+    y = (x * 2 + 1.5) / 3
+    assert y.code.type == "Div" and isinstance(y.prev[1], SymbolicConst) and y.prev[1].code.value == 3
+    z = 1 - x
+    assert z.code.type == "Sub" and z.prev[0].code.type == "Const" and z.prev[1] is x
+    with pytest.raises(TypeError):
+        x + "a"
+
+
+def test_customio_declares_symbolic_tensors():
+    io = CustomIO({"softmax_bias": (1,), "slopes": ("heads",)})
+    assert io.input_tensors["softmax_bias"].shape_idx == ["1"]
+    assert io.input_tensors["slopes"].shape_idx == ["heads"]
+
+
+# ---- masks (product) vs brute force (oracle) --------------------------------------------------------
+@pytest.mark.parametrize("mask_mod", [C.causal_mask, C.causal_plus_one_mask, C.causal_shifted_mask,
+                                      C.make_sliding_window_mask(100), C.head_dependent_mask])
+def test_create_mask_and_block_mask_match_brute_force(mask_mod):
+    B, H, S = 2, 4, 512
+    dense = create_mask(mask_mod, B, H, S, S, device="cpu")
+    ref = M.dense_mask_grid(mask_mod, B, H, S, S)
+    assert dense.dtype == torch.bool and np.array_equal(dense.numpy(), ref)
+    blocks = create_block_mask(mask_mod, B, H, S, S, "cpu", 128, 64)
+    assert blocks.dtype == torch.int8 and np.array_equal(blocks.numpy(), M.block_any(ref, 128, 64))
+    assert bool(is_causal_mask(blocks, 128, 64)) == bool(
+        np.array_equal(np.broadcast_to(M.block_causal_pattern(4, 8, 128, 64), blocks.shape), blocks.numpy().astype(bool)))
+    assert bool(is_less_causal_mask(blocks, 128, 64)) == M.no_block_above_diagonal(blocks.numpy(), 128, 64)
+    idx = create_block_idx(mask_mod, B, H, S, S, "cpu", 128, 64)
+    assert idx.shape == (int(blocks.sum()), 4)
+
+
+def test_block_mask_known_answers_of_the_reference_test_script():
+    """attention_engine/tests/test_blockmask.py:3-27 prints these; values hand-derived."""
+    for mask_mod, last, causal, less in [(C.causal_mask, [1, 3, 5, 7], True, True),
+                                         (C.causal_plus_one_mask, [2, 4, 6, 7], False, False),
+                                         (C.causal_shifted_mask, [-1, 1, 3, 5], False, True)]:
+        blocks = create_block_mask(mask_mod, 2, 4, 512, 512, "cpu", 128, 64)
+        for i, l in enumerate(last):
+            assert blocks[0, 0, i].tolist() == [1] * (l + 1) + [0] * (7 - l)
+        assert bool(is_causal_mask(blocks, 128, 64)) == causal
+        assert bool(is_less_causal_mask(blocks, 128, 64)) == less
+
+
+def test_ragged_block_mask_pads_with_invisible():
+    blocks = create_block_mask(C.causal_mask, 1, 1, 200, 200, "cpu", 128, 64)
+    assert blocks.shape == (1, 1, 2, 4)
+    assert blocks[0, 0].tolist() == [[1, 1, 0, 0], [1, 1, 1, 1]]
+
+
+def test_mask_plan_classes_match_oracle():
+    for mask_mod in (C.causal_plus_one_mask, C.make_sliding_window_mask(100), C.head_dependent_mask):
+        lm = lower_mask_mod(mask_mod)
+        plan = plan_mask(mask_mod, lm, 2, 4, 300, 300, 128, 64, chunk_rows=128)
+        assert plan.mode == 2
+        mb, mh = (2 if lm.uses_b else 1), (4 if lm.uses_h else 1)
+        ref = M.block_classes(M.dense_mask_grid(mask_mod, mb, mh, 300, 300), 128, 64)
+        assert np.array_equal(plan.table.numpy(), ref)
+    lm = lower_mask_mod(C.causal_mask)
+    assert plan_mask(C.causal_mask, lm, 2, 4, 300, 300, 128, 64).mode == 1
+    assert not lm.uses_b and not lm.uses_h
+    assert lower_mask_mod(C.head_dependent_mask).uses_h
+
+
+def test_mask_mod_lowering_text_and_unsupported_ops():
+    lm = lower_mask_mod(C.make_sliding_window_mask(256))
+    assert "n_ge" in lm.body and "(bool)(n_ge) & (bool)(n_lt)" in lm.body and "return (bool)" in lm.body
+
+    def bad(b, h, q_idx, kv_idx):
+        return torch.sin(q_idx) > kv_idx
+    with pytest.raises(NotImplementedError):
+        lower_mask_mod(bad)
+
+
+# ---- functor emission -----------------------------------------------------------------------------
+def test_emitted_softmax_functors():
+    lf = L.trace_functors(C.make_scale_score_mod(0.125), C.causal_mask, C.OnlineSoftmax(), CustomIO({}),
+                          torch.float16)
+    assert lf.rowstate_fields == ["m", "r"] and lf.rowstate_init == ["-1e38f", "0.0f"]
+    assert lf.final_rowscale_names == ["lse"] and not lf.o_scale_one
+    assert "ae_row_max<N>(s)" in lf.online_fwd_body and "ae_row_sum<N>" in lf.online_fwd_body
+    # exp(scores - m_new) is fused into one fma + exp2 per element
+    assert "ae_exp2(__builtin_fmaf(s[e], AE_LOG2E" in lf.online_fwd_body
+    assert "frs[0]" in lf.epilogue_body and "ae_log(st.r)" in lf.epilogue_body
+    src = L.render_functors(lf)
+    for name in ("ae_score_mod", "ae_online_fwd", "ae_epilogue", "ae_mask_mod", "ae_rowstate_init"):
+        assert name in src
+
+
+def test_emitted_identity_and_custom_scalar():
+    lf = L.trace_functors(C.make_sigmoid_score_mod(0.1), None, C.OnlineIdentity(),
+                          CustomIO({"softmax_bias": (1,)}), torch.float16)
+    assert lf.o_scale_one and lf.rowstate_fields == [] and lf.final_rowscale_names == []
+    assert lf.customs[0].name == "softmax_bias" and lf.customs[0].torch_dtype == torch.float32
+    assert "ae_tanh" in lf.score_mod_body and "cust.softmax_bias" in lf.score_mod_body
+
+
+def test_unsupported_graphs_raise():
+    class Bad(OnlineFunc):
+        def __init__(self):
+            super().__init__({"m": SymbolScalar("m", Var("banana"))}, {}, CustomIO())
+    with pytest.raises(NotImplementedError):
+        L.trace_functors(None, None, Bad(), CustomIO({}), torch.float16)
+    with pytest.raises(NotImplementedError):   # per-element custom tensors are not lowered yet
+        L.trace_functors(lambda s, c, b, h, q, kv: s * c.input_tensors["mask"], None, C.OnlineIdentity(),
+                         CustomIO({"mask": (1, "heads", "seq_len", "seq_len_kv")}), torch.float16)
+
+
+def test_combine_lowering_finds_the_merged_lse():
+    text = lower_combine(C.OnlineSoftmax(), ["lse"])
+    assert "ae_arr_max<AE_NSPLIT>(rs[0])" in text and "ae_arr_sum<AE_NSPLIT>" in text
+    assert "merged[0] = cb" in text and "nanf" not in text
+    text = lower_combine(C.OnlineIdentity(), [])
+    assert "w[e] = 1.0f" in text
+
+
+# ---- engine construction compiles through hipRTC without a GPU ---------------------------------------
+def _meta(B, Hq, Hkv, Sq, Skv, D, DV, dt):
+    return (meta_tensor(B, Hq, Sq, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt),
+            meta_tensor(B, Hkv, Skv, DV, dtype=dt))
+
+
+def test_engine_dispatch_and_compile_on_cpu():
+    from core.lower.lower_decode import GQADecodeOp, MLADecodeOp
+    from core.lower.prefill_op import PrefillOp
+    sm = C.make_scale_score_mod(0.1)
+    pre = AttentionEngine(_meta(1, 2, 2, 256, 256, 64, 64, torch.float16), CustomIO({}), sm, C.causal_mask,
+                          C.OnlineSoftmax())
+    assert isinstance(pre._op, PrefillOp) and "#define AE_MASK_MODE 1" in pre.tl_code
+    assert pre.block_mask is None     # exactly block-causal -> dense template in the reference
+    win = AttentionEngine(_meta(1, 2, 2, 512, 512, 64, 64, torch.bfloat16), CustomIO({}), sm,
+                          C.make_sliding_window_mask(128), C.OnlineSoftmax())
+    assert "#define AE_MASK_MODE 2" in win.tl_code and "#define AE_DTYPE_BF16 1" in win.tl_code
+    assert win.block_mask.shape == (1, 2, 4, 4) and win.block_mask.dtype == torch.int8
+    dec = AttentionEngine(_meta(2, 32, 8, 1, 1024, 128, 128, torch.float16), CustomIO({}), sm, None,
+                          C.OnlineSoftmax())
+    assert isinstance(dec._op, GQADecodeOp) and "ae_combine" in dec.tl_code
+    mla = AttentionEngine(_meta(2, 128, 1, 1, 512, 576, 512, torch.bfloat16), CustomIO({}), sm, None,
+                          C.OnlineSoftmax(), kv_shared=True)
+    assert isinstance(mla._op, MLADecodeOp)
+    gqa = AttentionEngine(_meta(1, 8, 2, 256, 256, 64, 64, torch.float16), CustomIO({}), sm, C.causal_mask,
+                          C.OnlineSoftmax())
+    assert isinstance(gqa._op, PrefillOp)
+    # tuner / backend arguments of the reference scripts are accepted
+    AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), sm, C.causal_mask,
+                    C.OnlineSoftmax(), tune=True, tune_file="x.json", tune_bwd=True, backend="cute")
+    # identity online function may be None (reference CuTe scripts)
+    AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), C.make_relu_score_mod(0.1),
+                    None, None)
+
+
+def test_engine_error_behaviour():
+    sm = C.make_scale_score_mod(0.1)
+    with pytest.raises(KeyError):       # unsupported dtype, as attn_engine.py:225-228 / 304
+        AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float32), CustomIO({}), sm, None, C.OnlineSoftmax())
+    with pytest.raises(AssertionError):  # decode asserts q_len == 1 (attn_engine.py:255)
+        AttentionEngine(_meta(1, 8, 2, 4, 1024, 64, 64, torch.float16), CustomIO({}), sm, None, C.OnlineSoftmax())
+    with pytest.raises(NotImplementedError):
+        AttentionEngine(_meta(1, 2, 2, 128, 1024, 64, 64, torch.float16), CustomIO({}), sm, None, C.OnlineSoftmax())
+    with pytest.raises(ValueError):
+        AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), sm, None,
+                        C.OnlineSoftmax(), backend="triton")
+    mod = AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), sm, None, C.OnlineSoftmax())
+    q = torch.zeros(1, 128, 2, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="no CPU path"):   # the product never falls back to the CPU
+        mod(q, q, q)
