@@ -39,9 +39,11 @@ class PrefillOp:
         self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
                                          self.dtype, mask_value)
         self.functor_src = L.render_functors(self.functors)
-        self.tiles = L.choose_prefill_tiles(self.D, self.DV)
+        self.tiles = L.choose_prefill_tiles(self.D, self.DV, 0 if isinstance(q_meta.shape[2], str) else int(q_meta.shape[2]))
         if self.extern_block_mask:
             # a q tile must sit inside one block-mask row, a kv tile inside one column
+            if self.tiles.block_m > self.mask_block[0] and self.tiles.row_blocks > 1:
+                self.tiles.row_blocks, self.tiles.waves_per_eu = 1, 2
             while self.tiles.block_m > self.mask_block[0] and self.tiles.n_waves > 1:
                 self.tiles.n_waves //= 2
             while self.tiles.block_n > self.mask_block[1] and self.tiles.block_n > 32:

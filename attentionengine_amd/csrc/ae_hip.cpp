@@ -319,8 +319,10 @@ int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg
   if (cfg->mask_mode == 2 && (cfg->block_m % p->mask_block_m != 0 && p->mask_block_m % cfg->block_m != 0))
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: mask block rows %d incompatible with tile %d",
                 p->mask_block_m, cfg->block_m);
+  // ids are 8*slot + xcd with slot = (batch*head / 8)*q_tiles + q_tile, see ae_prefill.hip
   uint64_t q_tiles = ((uint64_t)p->seqlen_q + cfg->block_m - 1) / cfg->block_m;
-  uint64_t total = q_tiles * (uint64_t)p->heads_q * (uint64_t)p->batch;
+  uint64_t bh = (uint64_t)p->heads_q * (uint64_t)p->batch;
+  uint64_t total = q_tiles * ((bh + 7) / 8) * 8;
   if (total == 0 || total > 0x7fffffffull)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: grid of %llu workgroups",
                 (unsigned long long)total);

@@ -8,14 +8,18 @@
 //
 // The user-defined parts arrive in "ae_config.h" / "ae_functors.h", generated from the traced
 // score_mod / mask_mod / OnlineFunc graphs:
-//   configuration  AE_D AE_DV AE_BN AE_NWAVES AE_DTYPE_BF16 AE_MASK_MODE AE_HAS_MASK_MOD
+//   configuration  AE_D AE_DV AE_BN AE_NWAVES AE_RB AE_DTYPE_BF16 AE_MASK_MODE AE_HAS_MASK_MOD
 //                  AE_N_ROWSCALES AE_O_SCALE_ONE AE_EVEN_Q AE_EVEN_KV AE_WAVES_PER_EU
 //                  AE_K_PAD AE_V_PAD
 //   functors       ae_rowstate, ae_rowstate_init, ae_mask_mod, ae_score_mod, ae_online_fwd,
 //                  ae_epilogue, ae_load_custom
 //
 // Mapping to the hardware
-//   * one workgroup = AE_NWAVES waves = AE_NWAVES*32 query rows of one (batch, head);
+//   * one workgroup = AE_NWAVES waves of one (batch, head); a wave owns AE_RB blocks of 32
+//     query rows.  Every K / V fragment read from LDS feeds one MFMA per row block, so AE_RB = 2
+//     halves the LDS (and HBM/L2) bytes moved per flop -- LDS read bandwidth (128 B/clk per CU,
+//     exactly what four SIMDs of 32x32x16 MFMAs consume with one row block) is what bounds the
+//     one-block variant;
 //   * scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16: in the
 //     accumulator layout every lane then owns ONE query row (column l%32) and 16 kv
 //     positions per 32x32 block, so row max / row sum are in-register reductions plus one
@@ -37,7 +41,11 @@
 #include "ae_device.h"
 #include "ae_functors.h"  // generated: the functor bodies
 
-#define AE_BM (AE_NWAVES * 32)
+#ifndef AE_RB
+#define AE_RB 1
+#endif
+#define AE_WROWS (AE_RB * 32)     // query rows per wave
+#define AE_BM (AE_NWAVES * AE_WROWS)
 #define AE_NT (AE_NWAVES * 64)
 #define AE_NB (AE_BN / 32)        // 32-wide kv blocks per tile
 #define AE_NS (AE_NB * 16)        // score elements per lane per tile
@@ -75,14 +83,20 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int hf = lane >> 5;
 
   // ---- which (q-tile, head, batch) -----------------------------------------------------
-  // (batch, head) varies fastest so that consecutive workgroups, which the dispatcher deals
-  // round-robin to the 8 XCDs, keep every q-tile of one (batch, head) on one XCD's L2.
+  // The dispatcher deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own
+  // L2.  All q-tiles of one (batch, head) read the same K/V, so they are given ids that land on
+  // ONE XCD back to back (id = 8*slot + xcd, slot = bh_local*n_qt + qt_i): the tiles run
+  // concurrently, walk the kv axis roughly in step and share K/V through that XCD's L2.
   // With a causal mask the tiles with the most kv work (last q-tiles) are issued first.
+  // The grid is padded to 8*ceil(n_bh/8)*n_qt ids; surplus workgroups exit immediately.
   const int n_qt = (p.seqlen_q + AE_BM - 1) / AE_BM;
   const int n_bh = p.batch * p.heads_q;
   const int wg = blockIdx.x;
-  const int bh = wg % n_bh;
-  const int qt_i = wg / n_bh;
+  const int xcd = wg & 7;
+  const int slot = wg >> 3;
+  const int qt_i = slot % n_qt;
+  const int bh = (slot / n_qt) * 8 + xcd;
+  if (bh >= n_bh) return;
 #if AE_MASK_MODE == 1
   const int qt = n_qt - 1 - qt_i;
 #else
@@ -92,22 +106,29 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int b = bh / p.heads_q;
   const int hk = h / (p.heads_q / p.heads_kv);
   const int q0 = qt * AE_BM;
-  const int q0w = q0 + wave * 32;
-  const int qrow = q0w + l32;
+  const int q0w = q0 + wave * AE_WROWS;       // first row of this wave
+  int qrow[AE_RB];                             // this lane's row in each row block
+  bool q_ok[AE_RB];
+#pragma unroll
+  for (int rb = 0; rb < AE_RB; rb++) {
+    qrow[rb] = q0w + rb * 32 + l32;
 #if AE_EVEN_Q
-  const bool q_ok = true;
-  const int qrow_c = qrow;
+    q_ok[rb] = true;
 #else
-  const bool q_ok = qrow < p.seqlen_q;
-  const int qrow_c = q_ok ? qrow : p.seqlen_q - 1;
+    q_ok[rb] = qrow[rb] < p.seqlen_q;
 #endif
+  }
 
   // ---- Q fragments: B operand of S^T = K Q^T, resident for the whole kernel -------------
-  const ae_elem* qptr = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b +
-                        (int64_t)qrow_c * p.q_stride_s + (int64_t)h * p.q_stride_h;
-  ae_elem8 qf[AE_D / 16];
+  ae_elem8 qf[AE_RB][AE_D / 16];
 #pragma unroll
-  for (int ks = 0; ks < AE_D / 16; ks++) qf[ks] = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
+  for (int rb = 0; rb < AE_RB; rb++) {
+    const int qr = q_ok[rb] ? qrow[rb] : p.seqlen_q - 1;
+    const ae_elem* qptr = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b +
+                          (int64_t)qr * p.q_stride_s + (int64_t)h * p.q_stride_h;
+#pragma unroll
+    for (int ks = 0; ks < AE_D / 16; ks++) qf[rb][ks] = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
+  }
 
   // ---- KV tile range ---------------------------------------------------------------------
   const int n_kvt = (p.seqlen_kv + AE_BN - 1) / AE_BN;
@@ -179,20 +200,23 @@ void ae_prefill_kernel(const ae_attn_params p) {
   };
 
   // ---- state ------------------------------------------------------------------------------
-  ae_ctx ctx;
-  ctx.b = b;
-  ctx.h = h;
-  ctx.q_idx = qrow;
-  ctx.kv_base = 0;
-  ae_custom cust;
-  ae_load_custom(cust, p, ctx);
-  ae_rowstate st;
-  ae_rowstate_init(st);
-  ae_f32x16 oacc[AE_NDB];
+  ae_ctx ctx[AE_RB];
+  ae_custom cust[AE_RB];
+  ae_rowstate st[AE_RB];
+  ae_f32x16 oacc[AE_RB][AE_NDB];
 #pragma unroll
-  for (int db = 0; db < AE_NDB; db++)
+  for (int rb = 0; rb < AE_RB; rb++) {
+    ctx[rb].b = b;
+    ctx[rb].h = h;
+    ctx[rb].q_idx = qrow[rb];
+    ctx[rb].kv_base = 0;
+    ae_load_custom(cust[rb], p, ctx[rb]);
+    ae_rowstate_init(st[rb]);
 #pragma unroll
-    for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
+    for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[rb][db][r] = 0.f;
+  }
 
   // lane-constant LDS offsets
   const int k_rd_off = l32 * AE_KSTR + hf * 16;                     // + nb*32*KSTR + ks*32
@@ -205,6 +229,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
     load_tile(j);
     store_tile(0);
   }
+  // Drain every outstanding load (Q fragments, first tile) before the loop: with loads still
+  // pending at the loop header the compiler's wait-count insertion makes the QK^T MFMAs of every
+  // iteration wait for that iteration's K/V prefetch, which serialises the pipeline.
+  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
   int stage = 0;
@@ -216,97 +244,105 @@ void ae_prefill_kernel(const ae_attn_params p) {
     ae_lds_byte* vs_ = ks_ + AE_K_BYTES;
     const int kv0 = j * AE_BN;
 
-    // ---- S^T = K Q^T ---------------------------------------------------------------------
-    ae_f32x16 sacc[AE_NB];
+    // ---- S^T = K Q^T: every K fragment feeds one MFMA per row block -------------------------
+    ae_f32x16 sacc[AE_RB][AE_NB];
 #pragma unroll
-    for (int nb = 0; nb < AE_NB; nb++)
+    for (int rb = 0; rb < AE_RB; rb++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) sacc[nb][r] = 0.f;
+      for (int nb = 0; nb < AE_NB; nb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[rb][nb][r] = 0.f;
 #pragma unroll
     for (int ks = 0; ks < AE_D / 16; ks++) {
 #pragma unroll
       for (int nb = 0; nb < AE_NB; nb++) {
         ae_elem8 kf = *(__attribute__((address_space(3))) ae_elem8*)(
             ks_ + k_rd_off + nb * 32 * AE_KSTR + ks * 32);
-        sacc[nb] = ae_mfma32(kf, qf[ks], sacc[nb]);
+#pragma unroll
+        for (int rb = 0; rb < AE_RB; rb++) sacc[rb][nb] = ae_mfma32(kf, qf[rb][ks], sacc[rb][nb]);
       }
     }
-    float s[AE_NS];
-#pragma unroll
-    for (int nb = 0; nb < AE_NB; nb++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) s[nb * 16 + r] = sacc[nb][r];
 
-    ctx.kv_base = kv0 + 4 * hf;
+    ae_elem8 pf[AE_RB][AE_BN / 16];
+#pragma unroll
+    for (int rb = 0; rb < AE_RB; rb++) {
+      float s[AE_NS];
+#pragma unroll
+      for (int nb = 0; nb < AE_NB; nb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[nb * 16 + r] = sacc[rb][nb][r];
+      ctx[rb].kv_base = kv0 + 4 * hf;
+      const int kvb = ctx[rb].kv_base;
 
-    // ---- mask (additive -inf before score_mod, attn_tl.py:124-137) ----------------------------
+      // ---- mask (additive -inf before score_mod, attn_tl.py:124-137) --------------------------
 #if AE_MASK_MODE == 1
-    if (kv0 + AE_BN - 1 > q0w) {  // tile crosses the diagonal of this wave's rows
+      if (kv0 + AE_BN - 1 > q0w + rb * 32) {  // tile crosses the diagonal of this row block
 #pragma unroll
-      for (int e = 0; e < AE_NS; e++)
-        s[e] = (qrow >= ctx.kv_base + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
-    }
+        for (int e = 0; e < AE_NS; e++) s[e] = (qrow[rb] >= kvb + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
+      }
 #elif AE_HAS_MASK_MOD
 #if AE_MASK_MODE == 2
-    if (AE_TILE_CLASS(j) != 2)
+      if (AE_TILE_CLASS(j) != 2)
 #endif
-    {
+      {
 #pragma unroll
-      for (int e = 0; e < AE_NS; e++)
-        s[e] = ae_mask_mod(b, h, qrow, ctx.kv_base + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
-    }
+        for (int e = 0; e < AE_NS; e++)
+          s[e] = ae_mask_mod(b, h, qrow[rb], kvb + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
+      }
 #endif
 #if !AE_EVEN_KV
-    if (kv0 + AE_BN > p.seqlen_kv) {
+      if (kv0 + AE_BN > p.seqlen_kv) {
 #pragma unroll
-      for (int e = 0; e < AE_NS; e++)
-        s[e] = (ctx.kv_base + ae_kv_off(e) < p.seqlen_kv) ? s[e] : AE_NEG_INF;
-    }
+        for (int e = 0; e < AE_NS; e++) s[e] = (kvb + ae_kv_off(e) < p.seqlen_kv) ? s[e] : AE_NEG_INF;
+      }
 #endif
 
-    // ---- user functors ------------------------------------------------------------------------
-    ae_score_mod<AE_NS>(s, ctx, cust);
-    float o_scale = ae_online_fwd<AE_NS>(s, st, ctx, cust);
+      // ---- user functors ----------------------------------------------------------------------
+      ae_score_mod<AE_NS>(s, ctx[rb], cust[rb]);
+      float o_scale = ae_online_fwd<AE_NS>(s, st[rb], ctx[rb], cust[rb]);
 
 #if !AE_EVEN_KV
-    if (kv0 + AE_BN > p.seqlen_kv) {
+      if (kv0 + AE_BN > p.seqlen_kv) {
 #pragma unroll
-      for (int e = 0; e < AE_NS; e++)
-        s[e] = (ctx.kv_base + ae_kv_off(e) < p.seqlen_kv) ? s[e] : 0.f;
-    }
+        for (int e = 0; e < AE_NS; e++) s[e] = (kvb + ae_kv_off(e) < p.seqlen_kv) ? s[e] : 0.f;
+      }
 #endif
 
-    // ---- P -> B-operand fragments -----------------------------------------------------------
-    ae_elem8 pf[AE_BN / 16];
+      // ---- P -> B-operand fragments -----------------------------------------------------------
 #pragma unroll
-    for (int kk = 0; kk < AE_BN / 16; kk++)
+      for (int kk = 0; kk < AE_BN / 16; kk++)
 #pragma unroll
-      for (int t = 0; t < 8; t++) pf[kk][t] = (ae_elem)s[kk * 8 + t];
+        for (int t = 0; t < 8; t++) pf[rb][kk][t] = (ae_elem)s[kk * 8 + t];
 
 #if !AE_O_SCALE_ONE
+      // skip the rescale when no row of this block changed its scale (wave-uniform branch)
+      if (__builtin_amdgcn_ballot_w64(o_scale != 1.0f) != 0) {
 #pragma unroll
-    for (int db = 0; db < AE_NDB; db++)
+        for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) oacc[db][r] *= o_scale;
+          for (int r = 0; r < 16; r++) oacc[rb][db][r] *= o_scale;
+      }
 #else
-    (void)o_scale;
+      (void)o_scale;
 #endif
+    }
 
-    // ---- O^T += V^T P^T ----------------------------------------------------------------------
+    // ---- O^T += V^T P^T: every V fragment feeds one MFMA per row block ------------------------
 #pragma unroll
     for (int kk = 0; kk < AE_BN / 16; kk++) {
-      // slots 0..3 of this k-step are kv rows rb+4*hf+0..3, slots 4..7 rows rb+8+4*hf+0..3
-      const int rb = (kk >> 1) * 32 + (kk & 1) * 16;
+      // slots 0..3 of this k-step are kv rows rb0+4*hf+0..3, slots 4..7 rows rb0+8+4*hf+0..3
+      const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
 #pragma unroll
       for (int db = 0; db < AE_NDB; db++) {
-        ae_lds_byte* a0 = vs_ + v_rd_off + rb * AE_VSTR + db * 64;
+        ae_lds_byte* a0 = vs_ + v_rd_off + rb0 * AE_VSTR + db * 64;
         ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) ae_s16x4*)a0);
         ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) ae_s16x4*)(a0 + 8 * AE_VSTR));
         ae_elem8 vf = __builtin_bit_cast(
             ae_elem8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-        oacc[db] = ae_mfma32(vf, pf[kk], oacc[db]);
+#pragma unroll
+        for (int rb = 0; rb < AE_RB; rb++) oacc[rb][db] = ae_mfma32(vf, pf[rb][kk], oacc[rb][db]);
       }
     }
 
@@ -317,37 +353,39 @@ void ae_prefill_kernel(const ae_attn_params p) {
   }
 
   // ---- epilogue -------------------------------------------------------------------------------
-  float o[AE_NO];
 #pragma unroll
-  for (int db = 0; db < AE_NDB; db++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) o[db * 16 + r] = oacc[db][r];
-  float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
-  frs[0] = 0.f;
-  if (any_tile) {
-    ae_epilogue<AE_NO>(o, st, frs, ctx, cust);
-  } else {
-    // no visible kv block for this q-tile: out = 0 (blockattn_tl.py:153-160), rowscales = -inf
-#pragma unroll
-    for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
-  }
-
-  if (q_ok) {
-    ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow * p.o_stride_s +
-                    (int64_t)h * p.o_stride_h;
+  for (int rb = 0; rb < AE_RB; rb++) {
+    float o[AE_NO];
 #pragma unroll
     for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        ae_elem4 w;
+      for (int r = 0; r < 16; r++) o[db * 16 + r] = oacc[rb][db][r];
+    float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+    frs[0] = 0.f;
+    if (any_tile) {
+      ae_epilogue<AE_NO>(o, st[rb], frs, ctx[rb], cust[rb]);
+    } else {
+      // no visible kv block for this q-tile: out = 0 (blockattn_tl.py:153-160), rowscales = -inf
 #pragma unroll
-        for (int t = 0; t < 4; t++) w[t] = (ae_elem)o[db * 16 + rg * 4 + t];
-        *(ae_elem4*)(optr + db * 32 + rg * 8 + hf * 4) = w;
+      for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
+    }
+    if (q_ok[rb]) {
+      ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow[rb] * p.o_stride_s +
+                      (int64_t)h * p.o_stride_h;
+#pragma unroll
+      for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int t = 0; t < 4; t++) w[t] = (ae_elem)o[db * 16 + rg * 4 + t];
+          *(ae_elem4*)(optr + db * 32 + rg * 8 + hf * 4) = w;
+        }
+      if (hf == 0) {
+#pragma unroll
+        for (int i = 0; i < AE_N_ROWSCALES; i++)
+          p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[rb]] = frs[i];
       }
-    if (hf == 0) {
-#pragma unroll
-      for (int i = 0; i < AE_N_ROWSCALES; i++)
-        p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow] = frs[i];
     }
   }
 }

@@ -173,7 +173,8 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
  * split-KV work buffers) and derive the grid; nothing is launched when a check fails.
  *
  * ae_prefill_fwd: one workgroup per (q-tile, q-head, batch) -- the grid of
- *   attn_tl.py:86 -- flattened to 1-D so the kernel can order heavy causal tiles first.
+ *   attn_tl.py:86 -- flattened to 1-D (padded to a multiple of 8 (batch, head) pairs) so the
+ *   kernel can keep the q-tiles of one (batch, head) on one XCD and issue heavy causal tiles first.
  * ae_decode_fwd:  split-KV pass followed by the combine kernel, grid (Hq, B)
  *   (attn_gqa_decode_tl.py:150-151, 224-266). Every WAVE of the split kernel produces one partial,
  *   so its grid is (num_splits / (threads/64), ceil(Hq/Hkv / block_m)*Hkv, B); kv_per_split is the
