@@ -234,29 +234,32 @@ AE_DEV void ae_epilogue(float (&o)[N], ae_rowstate& st, float (&frs)[{nrs}], con
 
 @dataclass
 class PrefillTiles:
-    """Tile configuration of the prefill template (fixed per head dim; chosen from rocprof
+    """Tile configuration of a prefill template (fixed per head dim; chosen from rocprof
     measurements rather than tuned at run time)."""
+    template: str = "ae_prefill.hip"   # direct-to-LDS kernel
     n_waves: int = 4
-    row_blocks: int = 1      # 32-row blocks per wave (AE_RB)
     block_n: int = 64
     waves_per_eu: int = 2
-    k_pad: int = 16
-    v_pad: int = 64
+    k_pad: int = 0
+    v_pad: int = 0
 
     @property
     def block_m(self):
-        return 32 * self.row_blocks * self.n_waves
+        return 32 * self.n_waves
 
     def lds_bytes(self, d: int, dv: int) -> int:
-        return 2 * (self.block_n * (2 * d + self.k_pad) + self.block_n * (2 * dv + self.v_pad))
+        return 2 * self.block_n * ((2 * d + self.k_pad) + (2 * dv + self.v_pad))
 
 
 def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0) -> PrefillTiles:
-    """One 32-row block per wave and two waves per SIMD; wide heads get the whole register file
-    (one wave per SIMD) and a shorter kv tile."""
-    t = PrefillTiles()
+    """The direct-to-LDS kernel handles 128- and 256-byte K/V rows (head dims 64 and 128); other
+    head dims use the register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one
+    wave per SIMD and a shorter kv tile once the accumulators outgrow 256 registers."""
+    if d in (64, 128) and dv in (64, 128):
+        return PrefillTiles()
+    t = PrefillTiles(template="ae_prefill_simple.hip", k_pad=16)
     if max(d, dv) > 128:
-        t.row_blocks, t.waves_per_eu, t.block_n = 1, 1, 32
+        t.block_n, t.waves_per_eu = 32, 1
     # V rows must land on distinct LDS bank groups for the transpose reads: pitch = 64 mod 256
     t.v_pad = (64 - (2 * dv) % 256) % 256
     if t.v_pad == 0:
@@ -273,7 +276,6 @@ def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, h
         f"#define AE_DV {dv}",
         f"#define AE_BN {tiles.block_n}",
         f"#define AE_NWAVES {tiles.n_waves}",
-        f"#define AE_RB {tiles.row_blocks}",
         f"#define AE_DTYPE_BF16 {1 if dtype == torch.bfloat16 else 0}",
         f"#define AE_MASK_MODE {mask_mode}",
         f"#define AE_HAS_MASK_MOD {1 if has_mask_mod else 0}",

@@ -41,14 +41,11 @@ class PrefillOp:
         self.functor_src = L.render_functors(self.functors)
         self.tiles = L.choose_prefill_tiles(self.D, self.DV, 0 if isinstance(q_meta.shape[2], str) else int(q_meta.shape[2]))
         if self.extern_block_mask:
-            # a q tile must sit inside one block-mask row, a kv tile inside one column
-            if self.tiles.block_m > self.mask_block[0] and self.tiles.row_blocks > 1:
-                self.tiles.row_blocks, self.tiles.waves_per_eu = 1, 2
-            while self.tiles.block_m > self.mask_block[0] and self.tiles.n_waves > 1:
-                self.tiles.n_waves //= 2
+            # a q tile covers whole block-mask rows, a kv tile sits inside one block-mask column
             while self.tiles.block_n > self.mask_block[1] and self.tiles.block_n > 32:
                 self.tiles.block_n //= 2
-            if self.mask_block[0] % self.tiles.block_m or self.mask_block[1] % self.tiles.block_n:
+            if (self.tiles.block_m % self.mask_block[0] and self.mask_block[0] % self.tiles.block_m) or \
+                    self.mask_block[1] % self.tiles.block_n:
                 raise NotImplementedError(f"block mask granularity {self.mask_block} does not fit the tiles")
         self.n_rowscales = len(self.functors.final_rowscale_names)
         if self.n_rowscales > rt.AE_MAX_ROWSCALES or len(self.functors.customs) > rt.AE_MAX_CUSTOM:
@@ -113,7 +110,7 @@ class PrefillOp:
             has_mask_mod = self.elementwise_mask and mask_mode != 1
             cfg_src = L.render_config(self.D, self.DV, self.dtype, self.tiles, mask_mode, has_mask_mod,
                                       self.n_rowscales, self.functors.o_scale_one, even_q, even_kv)
-            module = rt.compile_module("ae_prefill.hip", {"ae_config.h": cfg_src,
+            module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,
                                                           "ae_functors.h": self.functor_src})
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
                              threads=64 * self.tiles.n_waves,

@@ -1,40 +1,36 @@
-// Flash-style attention forward (prefill) for gfx950 / CDNA4.
+// Flash-style attention forward (prefill) for gfx950 / CDNA4 with direct-to-LDS tile loads.
 //
 // Takes the place of the reference's TileLang prefill template
 // (attention_engine/core/template/tl_template/attn/attn_tl.py:76-174) and its block-sparse
-// sibling (blockattn_tl.py:49-160). Per KV tile it keeps the reference's order of operations
+// sibling (blockattn_tl.py:49-160).  Per KV tile it keeps the reference's order of operations
 // (attn_tl.py:124-164): mask -> +QK^T -> score_mod -> online_func -> cast P -> rescale O ->
 // O += P V, then the epilogue and the final-rowscale store.
 //
 // The user-defined parts arrive in "ae_config.h" / "ae_functors.h", generated from the traced
 // score_mod / mask_mod / OnlineFunc graphs:
-//   configuration  AE_D AE_DV AE_BN AE_NWAVES AE_RB AE_DTYPE_BF16 AE_MASK_MODE AE_HAS_MASK_MOD
+//   configuration  AE_D AE_DV AE_BN AE_NWAVES AE_DTYPE_BF16 AE_MASK_MODE AE_HAS_MASK_MOD
 //                  AE_N_ROWSCALES AE_O_SCALE_ONE AE_EVEN_Q AE_EVEN_KV AE_WAVES_PER_EU
-//                  AE_K_PAD AE_V_PAD
 //   functors       ae_rowstate, ae_rowstate_init, ae_mask_mod, ae_score_mod, ae_online_fwd,
 //                  ae_epilogue, ae_load_custom
 //
-// Mapping to the hardware
-//   * one workgroup = AE_NWAVES waves of one (batch, head); a wave owns AE_RB blocks of 32
-//     query rows.  Every K / V fragment read from LDS feeds one MFMA per row block, so AE_RB = 2
-//     halves the LDS (and HBM/L2) bytes moved per flop -- LDS read bandwidth (128 B/clk per CU,
-//     exactly what four SIMDs of 32x32x16 MFMAs consume with one row block) is what bounds the
-//     one-block variant;
-//   * scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16: in the
-//     accumulator layout every lane then owns ONE query row (column l%32) and 16 kv
-//     positions per 32x32 block, so row max / row sum are in-register reductions plus one
-//     exchange with lane l^32, and the online row state (m, r, o_scale, ...) is a scalar
-//     per lane;
-//   * the same registers, converted to fp16/bf16, are directly the B operand of
-//     O^T += V^T P^T (the contraction index only has to be enumerated in the same order by
-//     both operands), so P never goes through LDS;
-//   * Q stays in registers as B-operand fragments for the whole kernel; K and V tiles are
-//     staged HBM -> VGPR -> LDS with 16-byte coalesced loads, double-buffered so the loads
-//     of tile j+1 are in flight while tile j is being multiplied; K rows are read back with
-//     ds_read_b128, V is read through ds_read_b64_tr_b16 (LDS transpose load), which hands
-//     each lane four kv-consecutive values of its dv column from the row-major tile.
-//   * causal and block-sparse masks skip whole tiles; the elementwise mask is evaluated
-//     only on tiles that are not known to be fully visible.
+// Same mapping to the matrix cores as ae_prefill_simple.hip (which documents the register layouts
+// in full): S^T = K Q^T and O^T += V^T P^T with v_mfma_f32_32x32x16, one query row per lane, Q in
+// registers, P handed from the first product to the second without leaving registers.
+//
+// What differs is how K / V tiles reach LDS.  Measured on MI355X, staging a tile through VGPRs
+// (global_load -> 32 registers -> ds_write_b128) costs this kernel a third of its throughput: the
+// wave issues in order, so the extra loads, the wait for them and the LDS writes all sit on the
+// critical path of the two waves that share a SIMD.  Here every lane issues
+// `global_load_lds_dwordx4` instead: 16 bytes go from HBM/L2 straight into LDS at
+// (wave-uniform base) + lane*16, no VGPRs, no ds_write, and the only wait is one vmcnt(0) in front
+// of the barrier that publishes the tile.  A direct load cannot pad rows (64 lanes fill 1 KiB
+// contiguously), so bank conflicts are avoided by permuting WHICH 16-byte chunk of its row a lane
+// fetches:
+//     K tile: LDS chunk c' of row r holds global chunk c' ^ (r mod chunks_per_row), so the
+//             ds_read_b128 of 16 consecutive rows at one d offset hits 16 different bank groups;
+//     V tile: the permutation works on 32-byte pairs, (c'/2) ^ (r mod pairs_per_row), which keeps
+//             the 4 rows x 32 bytes of one ds_read_b64_tr_b16 group on distinct banks.
+// Tiles are double buffered: tile j+1 streams in while tile j is multiplied.
 
 #include "ae_hip.h"
 #include "ae_config.h"    // generated: the AE_* configuration macros
@@ -51,22 +47,26 @@
 #define AE_NS (AE_NB * 16)        // score elements per lane per tile
 #define AE_NDB (AE_DV / 32)       // 32-wide dv blocks
 #define AE_NO (AE_NDB * 16)       // output elements per lane
-#define AE_KSTR (AE_D * 2 + AE_K_PAD)    // LDS row pitch of the K tile, bytes
-#define AE_VSTR (AE_DV * 2 + AE_V_PAD)   // LDS row pitch of the V tile, bytes
+#define AE_KSTR (AE_D * 2)        // LDS row pitch of the K tile, bytes (no padding: swizzled)
+#define AE_VSTR (AE_DV * 2)       // LDS row pitch of the V tile, bytes
 #define AE_K_BYTES (AE_BN * AE_KSTR)
 #define AE_V_BYTES (AE_BN * AE_VSTR)
 #define AE_STAGE_BYTES (AE_K_BYTES + AE_V_BYTES)
 #define AE_KCPR (AE_D / 8)        // 16-byte chunks per K row
 #define AE_VCPR (AE_DV / 8)
-#define AE_K_LOADS ((AE_BN * AE_KCPR) / AE_NT)
+#define AE_K_LOADS ((AE_BN * AE_KCPR) / AE_NT)   // direct loads per lane per K tile
 #define AE_V_LOADS ((AE_BN * AE_VCPR) / AE_NT)
+#define AE_K_RPI (64 / AE_KCPR)   // K rows one wave instruction (64 lanes x 16 B) covers
+#define AE_V_RPI (64 / AE_VCPR)
+#define AE_VPPR (AE_VCPR / 2)     // 32-byte pairs per V row
 
 static_assert(AE_D % 16 == 0, "head dim must be a multiple of 16");
 static_assert(AE_DV % 32 == 0, "value head dim must be a multiple of 32");
 static_assert(AE_BN % 32 == 0, "kv tile must be a multiple of 32");
 static_assert((AE_BN * AE_KCPR) % AE_NT == 0, "K tile must split evenly over the workgroup");
 static_assert((AE_BN * AE_VCPR) % AE_NT == 0, "V tile must split evenly over the workgroup");
-static_assert(AE_KSTR % 16 == 0 && AE_VSTR % 8 == 0, "LDS pitches must keep vector alignment");
+static_assert(AE_KCPR == 8 || AE_KCPR == 16, "swizzle is written for 128- or 256-byte K rows");
+static_assert(AE_VCPR == 8 || AE_VCPR == 16, "swizzle is written for 128- or 256-byte V rows");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 
@@ -140,55 +140,63 @@ void ae_prefill_kernel(const ae_attn_params p) {
   }
 #endif
 #if AE_MASK_MODE == 2
-  const int8_t* bm_row = p.block_mask +
-      (((int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : h)) * p.mask_nq +
-       q0 / p.mask_block_m) * (int64_t)p.mask_nkv;
-#define AE_TILE_CLASS(j) ((int)bm_row[((j) * AE_BN) / p.mask_block_n])
+  // Tile class from the block table: 0 = skip, 1 = visit with the elementwise mask, 2 = fully
+  // visible.  A q-tile may span several table rows: it is skipped only if every row says so and
+  // fully visible only if every row says so.
+  const int8_t* bm_base = p.block_mask +
+      ((int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : h)) * p.mask_nq * (int64_t)p.mask_nkv;
+  const int bm_r0 = q0 / p.mask_block_m;
+  int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
+  bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
+  auto tile_class = [&](int j) -> int {
+    const int col = (j * AE_BN) / p.mask_block_n;
+    int any = 0, all = 2;
+    for (int r = bm_r0; r <= bm_r1; r++) {
+      int c = bm_base[(int64_t)r * p.mask_nkv + col];
+      any |= c;
+      all = c < all ? c : all;
+    }
+    return any == 0 ? 0 : (all == 2 ? 2 : 1);
+  };
+#define AE_TILE_CLASS(j) tile_class(j)
 #endif
 
   const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
   const ae_elem* vbase = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
 
-  ae_u32x4 kreg[AE_K_LOADS];
-  ae_u32x4 vreg[AE_V_LOADS];
-
-  auto load_tile = [&](int j) {
+  // Direct HBM -> LDS tile load.  Wave w, instruction i covers rows (w*LOADS + i)*RPI ...+RPI-1;
+  // lane L lands in LDS chunk c' = L % CPR of row (L / CPR) and fetches the permuted global chunk.
+  auto load_tile = [&](int j, int stage) {
     const int kv0 = j * AE_BN;
-#pragma unroll
-    for (int i = 0; i < AE_K_LOADS; i++) {
-      int c = tid + i * AE_NT;
-      int row = c / AE_KCPR, col = c % AE_KCPR;
-      int kv = kv0 + row;
-#if !AE_EVEN_KV
-      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
-#endif
-      kreg[i] = *(const ae_u32x4*)(kbase + (int64_t)kv * p.k_stride_s + col * 8);
-    }
-#pragma unroll
-    for (int i = 0; i < AE_V_LOADS; i++) {
-      int c = tid + i * AE_NT;
-      int row = c / AE_VCPR, col = c % AE_VCPR;
-      int kv = kv0 + row;
-#if !AE_EVEN_KV
-      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
-#endif
-      vreg[i] = *(const ae_u32x4*)(vbase + (int64_t)kv * p.v_stride_s + col * 8);
-    }
-  };
-  auto store_tile = [&](int stage) {
     ae_lds_byte* ks = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* vs = ks + AE_K_BYTES;
 #pragma unroll
     for (int i = 0; i < AE_K_LOADS; i++) {
-      int c = tid + i * AE_NT;
-      int row = c / AE_KCPR, col = c % AE_KCPR;
-      *(__attribute__((address_space(3))) ae_u32x4*)(ks + row * AE_KSTR + col * 16) = kreg[i];
+      const int blk = wave * AE_K_LOADS + i;                 // wave-uniform 1 KiB block of the tile
+      const int row = blk * AE_K_RPI + lane / AE_KCPR;
+      const int cp = lane % AE_KCPR;                          // LDS chunk
+      const int c = cp ^ (row & (AE_KCPR - 1));               // global chunk
+      int kv = kv0 + row;
+#if !AE_EVEN_KV
+      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
+#endif
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(kbase + (int64_t)kv * p.k_stride_s + c * 8),
+          (__attribute__((address_space(3))) void*)(ks + blk * 1024), 16, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < AE_V_LOADS; i++) {
-      int c = tid + i * AE_NT;
-      int row = c / AE_VCPR, col = c % AE_VCPR;
-      *(__attribute__((address_space(3))) ae_u32x4*)(vs + row * AE_VSTR + col * 16) = vreg[i];
+      const int blk = wave * AE_V_LOADS + i;
+      const int row = blk * AE_V_RPI + lane / AE_VCPR;
+      const int cp = lane % AE_VCPR;
+      const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
+      int kv = kv0 + row;
+#if !AE_EVEN_KV
+      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
+#endif
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(vbase + (int64_t)kv * p.v_stride_s + c * 8),
+          (__attribute__((address_space(3))) void*)(vs + blk * 1024), 16, 0, 0);
     }
   };
   // next tile index >= j that has work (block table) or j itself
@@ -218,17 +226,20 @@ void ae_prefill_kernel(const ae_attn_params p) {
       for (int r = 0; r < 16; r++) oacc[rb][db][r] = 0.f;
   }
 
-  // lane-constant LDS offsets
-  const int k_rd_off = l32 * AE_KSTR + hf * 16;                     // + nb*32*KSTR + ks*32
-  const int v_rd_off = (4 * hf + ((lane & 15) >> 2)) * AE_VSTR +     // + rowbase*VSTR + db*64
-                       ((l32 >> 4) * 16 + 4 * (lane & 3)) * 2;
+  // lane-constant pieces of the swizzled LDS read addresses
+  // K fragment (row l32 of a 32-row block, d chunk 2*ks+hf): chunk' = (2*ks+hf) ^ (l32 mod CPR)
+  const int k_row_off = l32 * AE_KSTR;
+  const int k_sw = l32 & (AE_KCPR - 1);
+  // V transpose read: lane i of a 16-lane group reads row 4*hf + i/4 (+8), 8 bytes at pair
+  // (2*db + g) ^ (row mod PPR), g = (lane%32)/16; rows of one group differ only in their low bits
+  const int v_row = 4 * hf + ((lane & 15) >> 2);
+  const int v_row_off = v_row * AE_VSTR + (lane & 3) * 8;
+  const int v_sw = v_row & (AE_VPPR - 1);
+  const int v_g = l32 >> 4;
 
   int j = next_tile(0);
   bool any_tile = j < j_end;
-  if (any_tile) {
-    load_tile(j);
-    store_tile(0);
-  }
+  if (any_tile) load_tile(j, 0);
   // Drain every outstanding load (Q fragments, first tile) before the loop: with loads still
   // pending at the loop header the compiler's wait-count insertion makes the QK^T MFMAs of every
   // iteration wait for that iteration's K/V prefetch, which serialises the pipeline.
@@ -238,7 +249,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   int stage = 0;
   while (j < j_end) {
     const int jn = next_tile(j + 1);
-    if (jn < j_end) load_tile(jn);
+    if (jn < j_end) load_tile(jn, stage ^ 1);   // streams into the other stage while this one is used
 
     ae_lds_byte* ks_ = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* vs_ = ks_ + AE_K_BYTES;
@@ -257,7 +268,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int nb = 0; nb < AE_NB; nb++) {
         ae_elem8 kf = *(__attribute__((address_space(3))) ae_elem8*)(
-            ks_ + k_rd_off + nb * 32 * AE_KSTR + ks * 32);
+            ks_ + k_row_off + nb * 32 * AE_KSTR + (((2 * ks + hf) ^ k_sw) << 4));
 #pragma unroll
         for (int rb = 0; rb < AE_RB; rb++) sacc[rb][nb] = ae_mfma32(kf, qf[rb][ks], sacc[rb][nb]);
       }
@@ -334,7 +345,8 @@ void ae_prefill_kernel(const ae_attn_params p) {
       const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
 #pragma unroll
       for (int db = 0; db < AE_NDB; db++) {
-        ae_lds_byte* a0 = vs_ + v_rd_off + rb0 * AE_VSTR + db * 64;
+        // (rb0 and +8 are multiples of 8 >= pairs per row, so they do not change the swizzle)
+        ae_lds_byte* a0 = vs_ + v_row_off + rb0 * AE_VSTR + (((2 * db + v_g) ^ v_sw) << 5);
         ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) ae_s16x4*)a0);
         ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -346,7 +358,8 @@ void ae_prefill_kernel(const ae_attn_params p) {
       }
     }
 
-    if (jn < j_end) store_tile(stage ^ 1);
+    // the next tile must have landed before anyone reads it: direct loads are tracked by vmcnt
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00 | 0x0000);  // vmcnt(0), expcnt/lgkmcnt untouched
     __syncthreads();
     stage ^= 1;
     j = jn;
