@@ -12,10 +12,24 @@ Register model.  In the kernels every lane owns ONE query row, so a value is eit
               the dv axis (the output accumulator in the epilogue).
 A value is an array iff its ``shape_idx`` names one of the array axes given to the emitter.
 All loops are fully unrolled, so the arrays live in VGPRs.
+
+Two rewrites keep the per-element instruction count of the common graphs at its minimum:
+  * affine folding: ``x * c``, ``x + y``, ``x - y``, ``-x`` with a constant c and a per-row y are
+    carried symbolically as ``base[e] * mul + add`` and only materialised where a non-affine
+    consumer needs them.  ``exp`` consumes the affine form as one fma + exp2 per element (the
+    per-row part ``add * log2e`` is hoisted) and ``ReduceMax`` as ``rowmax(base) * mul + add`` for
+    mul > 0, so ``softmax(scale * s)`` costs no multiply by the scale at all;
+  * lazy running maximum (``lazy_max``): where the lowering has proved that the graph is the online
+    softmax (results invariant under the choice of the reference point m), the update
+    ``m_new = max(m, x)`` becomes ``m_new = (x > m + tau) ? x : m``.  The exponentials then stay
+    below e^tau, the running sum and the output are rescaled only when a row's maximum grows by
+    more than tau, and the kernels skip the rescale of the accumulator when o_scale == 1.
 """
 from __future__ import annotations
 
 import math
+
+LOG2E = 1.4426950408889634
 
 from ..transform.core import SymbolScalar
 from ..transform.graph import COL_REDUCTIONS, ELEMENTWISE_BINARY, ELEMENTWISE_UNARY, ROW_REDUCTIONS
@@ -86,6 +100,8 @@ class Emitter:
         self.prefix = prefix
         self.lines = []
         self.done = {}   # id(symbol) -> (expr, is_array)
+        self.affine = {}  # id(symbol) -> (base array expr, mul: float, add: scalar expr or None)
+        self.lazy_max = {}  # id(Max symbol) -> tau: emit the thresholded update
         self.counter = 0
         self._keep = []  # keep traced symbols alive so ids stay unique
 
@@ -107,7 +123,7 @@ class Emitter:
         return f"{expr}[e]" if is_arr else expr
 
     # ---- graph walk ---------------------------------------------------------------------
-    def value(self, sym: SymbolScalar):
+    def _value_plain(self, sym: SymbolScalar):
         """(expression, is_array) of ``sym``, emitting whatever it depends on first."""
         key = id(sym)
         if key in self.done:
@@ -130,12 +146,135 @@ class Emitter:
         self.done[key] = val
         return val
 
+    # ---- affine forms -------------------------------------------------------------------
+    def _as_affine(self, sym: SymbolScalar):
+        """(base, mul, add) if ``sym`` is an array that can be carried as base[e]*mul + add."""
+        key = id(sym)
+        if key in self.affine:
+            return self.affine[key]
+        if key in self.done:
+            expr, is_arr = self.done[key]
+            return (expr, 1.0, None) if is_arr else None
+        if not self._is_array(sym):
+            return None
+        t = sym.code.type
+        if key in self.leaves or t in ("Var", "Const") or not sym.prev:
+            expr, is_arr = self.value(sym)
+            return (expr, 1.0, None) if is_arr else None
+        aff = None
+        if t in ("Mul", "Div") and len(sym.prev) == 2:
+            a, b = sym.prev
+            ca = a.code.value if a.code.type == "Const" else None
+            cb = b.code.value if b.code.type == "Const" else None
+            if cb is not None and (t == "Mul" or float(cb) != 0.0):
+                inner = self._as_affine(a)
+                if inner is not None:
+                    f = float(cb) if t == "Mul" else 1.0 / float(cb)
+                    aff = self._scale(inner, f)
+            elif ca is not None and t == "Mul":
+                inner = self._as_affine(b)
+                if inner is not None:
+                    aff = self._scale(inner, float(ca))
+        elif t in ("Add", "Sub") and len(sym.prev) == 2:
+            a, b = sym.prev
+            if self._is_array(a) and not self._is_array(b):
+                inner = self._as_affine(a)
+                if inner is not None:
+                    y = self.value(b)[0]
+                    aff = (inner[0], inner[1], self._sum(inner[2], y, "+" if t == "Add" else "-"))
+            elif t == "Add" and self._is_array(b) and not self._is_array(a):
+                inner = self._as_affine(b)
+                if inner is not None:
+                    aff = (inner[0], inner[1], self._sum(inner[2], self.value(a)[0], "+"))
+            elif t == "Sub" and self._is_array(b) and not self._is_array(a):
+                inner = self._as_affine(b)
+                if inner is not None:
+                    neg = self._scale(inner, -1.0)
+                    aff = (neg[0], neg[1], self._sum(neg[2], self.value(a)[0], "+"))
+        elif t == "Neg":
+            inner = self._as_affine(sym.prev[0])
+            if inner is not None:
+                aff = self._scale(inner, -1.0)
+        if aff is not None:
+            self.affine[key] = aff
+            self._keep.append(sym)
+        return aff
+
+    def _scale(self, aff, f: float):
+        base, mul, add = aff
+        if add is not None:
+            t = self._tmp()
+            self.lines.append(f"const float {t} = ({add}) * {float_literal(f)};")
+            add = t
+        return (base, mul * f, add)
+
+    def _sum(self, add, y: str, op: str):
+        t = self._tmp()
+        if add is None:
+            self.lines.append(f"const float {t} = {'' if op == '+' else '-'}({y});")
+        else:
+            self.lines.append(f"const float {t} = ({add}) {op} ({y});")
+        return t
+
+    def _materialise(self, sym: SymbolScalar):
+        """Array temp holding the value of an affine symbol."""
+        base, mul, add = self.affine[id(sym)]
+        out = self._tmp()
+        self.lines.append(f"float {out}[{self.n}];")
+        if add is None:
+            self._loop(f"{out}[e] = {base}[e] * {float_literal(mul)};")
+        else:
+            self._loop(f"{out}[e] = __builtin_fmaf({base}[e], {float_literal(mul)}, {add});")
+        return (out, True)
+
+    def value(self, sym: SymbolScalar):  # noqa: F811  (affine-aware front end of the graph walk)
+        key = id(sym)
+        if key in self.done:
+            return self.done[key]
+        if self._is_array(sym) and sym.code.type in ("Mul", "Div", "Add", "Sub", "Neg") and sym.prev:
+            aff = self._as_affine(sym)
+            if aff is not None and key in self.affine:
+                if aff[1] == 1.0 and aff[2] is None:
+                    val = (aff[0], True)
+                else:
+                    val = self._materialise(sym)
+                self.done[key] = val
+                return val
+        return self._value_plain(sym)
+
     def _emit_op(self, sym: SymbolScalar):
         t = sym.code.type
-        if t == "Exp":
-            fused = self._emit_exp_of_difference(sym)
-            if fused is not None:
-                return fused
+        if t in ("Exp", "Exp2") and self._is_array(sym.prev[0]):
+            aff = self._as_affine(sym.prev[0])
+            if aff is not None and not (aff[1] == 1.0 and aff[2] is None):
+                base, mul, add = aff
+                k = mul * (LOG2E if t == "Exp" else 1.0)
+                out = self._tmp()
+                if add is None:
+                    body = f"ae_exp2({base}[e] * {float_literal(k)})"
+                else:
+                    hoist = self._tmp()
+                    scale = " * AE_LOG2E" if t == "Exp" else ""
+                    self.lines.append(f"const float {hoist} = ({add}){scale};")
+                    body = f"ae_exp2(__builtin_fmaf({base}[e], {float_literal(k)}, {hoist}))"
+                self.lines.append(f"float {out}[{self.n}];")
+                self._loop(f"{out}[e] = {body};")
+                return (out, True)
+        if t == "ReduceMax" and not self.split_axis and self._is_array(sym.prev[0]):
+            aff = self._as_affine(sym.prev[0])
+            if aff is not None and aff[1] > 0.0 and not (aff[1] == 1.0 and aff[2] is None):
+                base, mul, add = aff
+                out = self._tmp()
+                tail = f" + ({add})" if add is not None else ""
+                self.lines.append(f"const float {out} = ae_row_max<{self.n}>({base}) * {float_literal(mul)}{tail};")
+                return (out, False)
+        if t == "Max" and id(sym) in self.lazy_max:
+            m_val = self.value(sym.prev[0])[0]
+            x_val = self.value(sym.prev[1])[0]
+            out = self._tmp()
+            tau = float_literal(self.lazy_max[id(sym)])
+            self.lines.append(f"const float {out} = (({x_val}) - ({m_val}) > {tau}) ? ({x_val}) : ({m_val});")
+            return (out, False)
         ins = [self.value(p) for p in sym.prev]
         out = self._tmp()
         if t in ROW_REDUCTIONS:
@@ -170,24 +309,6 @@ class Emitter:
         else:
             self.lines.append(f"const float {out} = {expr};")
         return (out, is_arr)
-
-    def _emit_exp_of_difference(self, sym: SymbolScalar):
-        """exp(x - y) with an array x and a per-row y becomes one fma + exp2 per element:
-        exp2(x*log2e + (-y*log2e)), the second term hoisted out of the loop."""
-        src = sym.prev[0]
-        if src.code.type != "Sub" or len(src.prev) != 2 or id(src) in self.done:
-            return None
-        if not self._is_array(src.prev[0]) or self._is_array(src.prev[1]):
-            return None
-        x = self.value(src.prev[0])
-        y = self.value(src.prev[1])
-        if not x[1] or y[1]:
-            return None
-        hoist, out = self._tmp(), self._tmp()
-        self.lines.append(f"const float {hoist} = -({y[0]}) * AE_LOG2E;")
-        self.lines.append(f"float {out}[{self.n}];")
-        self._loop(f"{out}[e] = ae_exp2(__builtin_fmaf({x[0]}[e], AE_LOG2E, {hoist}));")
-        return (out, True)
 
     def _elementwise(self, t: str, ins):
         a = self._at(ins[0])

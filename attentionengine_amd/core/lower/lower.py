@@ -89,6 +89,81 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
     return leaves, descs, loads, fields
 
 
+# threshold of the lazy running maximum, in the (natural-log) units of the user's exp():
+# exponentials stay below e^tau = 256, harmless for fp16/bf16 P and fp32 sums
+LAZY_MAX_TAU = 8.0 * 0.6931471805599453
+
+
+def find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale):
+    """Return the ``m_new = max(m, x)`` symbol if the traced online function is the online softmax
+    (attn_script/mha.py:47-72), whose outputs do not depend on the reference point m:
+
+        m_new = max(m, x)                 x: one value per row
+        o_scale = exp(m - m_new)
+        scores' = exp(S - m_new)
+        r_new = r * o_scale + rowsum(scores')
+        epilogue: o / r  and  lse = log(r) + m
+
+    Every use of m_new must be one of these.  Then m_new may lag behind the true maximum
+    (thresholded update, see codegen/hip_gen.py) without changing o or lse.  Anything else: None.
+    """
+    try:
+        if len(rowscales) != 2 or set(new_rowscales) != set(rowscales):
+            return None
+        (mk, m_new), = [(k, v) for k, v in new_rowscales.items() if v.code.type == "Max"]
+        (rk, r_new), = [(k, v) for k, v in new_rowscales.items() if k != mk]
+        m, r = rowscales[mk], rowscales[rk]
+        if m_new.prev[0] is not m or "block_N" in m_new.prev[1].shape_idx:
+            return None
+
+        def is_exp_minus(sym, lhs_is):
+            return (sym.code.type == "Exp" and sym.prev[0].code.type == "Sub"
+                    and sym.prev[0].prev[1] is m_new and lhs_is(sym.prev[0].prev[0]))
+        if not (isinstance(o_scale, SymbolScalar) and is_exp_minus(o_scale, lambda x: x is m)):
+            return None
+        if not is_exp_minus(new_scores, lambda x: "block_N" in x.shape_idx):
+            return None
+        if r_new.code.type != "Add":
+            return None
+        a, bsum = r_new.prev
+        if not (a.code.type == "Mul" and a.prev[0] is r and is_exp_minus(a.prev[1], lambda x: x is m)):
+            return None
+        if not (bsum.code.type == "ReduceSum" and bsum.prev[0] is new_scores):
+            return None
+        # every use of m_new: the two Sub nodes feeding exp (and being the new rowscale)
+        for use in m_new.use_list:
+            if not (use.code.type == "Sub" and use.prev[1] is m_new and
+                    all(u.code.type == "Exp" for u in use.use_list) and use.use_list):
+                return None
+        # epilogue shape
+        from ..transform.core import SymbolicArray as _SA
+        for v in rowscales.values():
+            v.clear_codegen()
+        acc = _SA("acc_o", Var("acc_o"), shape_idx=["block_M", "dimv"])
+        dummy = SymbolScalar("b", Var("b"), shape_idx=[])
+        o_new, finals = online_func.online_fwd_epilogue(acc, rowscales, dummy, dummy, dummy)
+        if not (o_new.code.type == "Div" and o_new.prev[0] is acc and o_new.prev[1] is r):
+            return None
+        if len(finals) != 1:
+            return None
+        (lse,) = finals.values()
+        if lse.code.type != "Add":
+            return None
+        x, y = lse.prev
+        ok = (x.code.type == "Log" and x.prev[0] is r and y is m) or (y.code.type == "Log" and y.prev[0] is r and x is m)
+        if not ok:
+            return None
+        # m and r must not be used for anything else in the epilogue
+        if len(m.use_list) != 1 or len(r.use_list) != 2:
+            return None
+        return m_new
+    except (ValueError, IndexError, AttributeError):
+        return None
+    finally:
+        for v in rowscales.values():
+            v.clear_codegen()
+
+
 def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO, in_dtype,
                    mask_value: str = "-inf") -> LoweredFunctors:
     """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
@@ -104,32 +179,19 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
                   id(q_idx): ("(float)ctx.q_idx", False), id(kv_idx): ("kvf", True)}
         return b, h, q_idx, kv_idx, leaves
 
-    # ---- score_mod ------------------------------------------------------------------------
+    # ---- score_mod + online_fwd, traced as ONE graph -------------------------------------------
+    # (the reference emits two macros, lower.py:475-558 and 318-472; fusing them lets the emitter
+    # fold the score scaling into the exponent of the online function)
     b, h, q_idx, kv_idx, leaves = index_leaves()
     scores = SymbolicArray("scores", Var("scores"), shape_idx=["block_M", "block_N"])
     leaves[id(scores)] = ("s", True)
     leaves.update(cust_leaves)
-    if score_mod is not None:
-        out = score_mod(scores, custom_fwd_inputs, b, h, q_idx, kv_idx)
-    else:
-        out = scores
-    em = Emitter(leaves, {}, ["block_N"], n="N", prefix="sm")
-    val = em.value(out)
-    body = []
-    if id(kv_idx) in em.done:
-        body += ["  float kvf[N];", "#pragma unroll",
-                 "  for (int e = 0; e < N; e++) kvf[e] = (float)(ctx.kv_base + ae_kv_off(e));"]
-    body.append(em.code())
-    if val[0] != "s":
-        src = f"{val[0]}[e]" if val[1] else val[0]
-        body += ["#pragma unroll", f"  for (int e = 0; e < N; e++) s[e] = {src};"]
-    score_mod_body = "\n".join(body)
-
-    # ---- online_fwd -----------------------------------------------------------------------
-    b, h, q_idx, _, leaves = index_leaves()
-    scores = SymbolicArray("scores", Var("scores"), shape_idx=["block_M", "block_N"])
-    leaves[id(scores)] = ("s", True)
-    leaves.update(cust_leaves)
+    scores_mod = score_mod(scores, custom_fwd_inputs, b, h, q_idx, kv_idx) if score_mod is not None else scores
+    if not isinstance(scores_mod, SymbolScalar):
+        raise TypeError("score_mod must return the (modified) scores symbol")
+    if not isinstance(scores_mod, SymbolicArray):
+        # e.g. `0.5 * scores`: keep the reduction interface of the score tile
+        scores_mod.__class__ = SymbolicArray
     rowscales = online_func.online_rowscales
     fields, inits = [], []
     for k, v in rowscales.items():
@@ -137,8 +199,11 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
         leaves[id(v)] = (f"st.{k}", False)
         fields.append(k)
         inits.append(init_literal(v.code.name))
-    new_scores, new_rowscales, o_scale = online_func.online_fwd(scores, rowscales, b, h, q_idx)
+    new_scores, new_rowscales, o_scale = online_func.online_fwd(scores_mod, rowscales, b, h, q_idx)
     em = Emitter(leaves, {}, ["block_N"], n="N", prefix="of")
+    lazy = find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale)
+    if lazy is not None:
+        em.lazy_max[id(lazy)] = LAZY_MAX_TAU
     new_vals = {k: em.value(v) for k, v in new_rowscales.items()}
     sval = em.value(new_scores)
     o_scale_const = var_as_constant(o_scale) if isinstance(o_scale, SymbolScalar) else float(o_scale)
@@ -146,7 +211,11 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     oval = em.value(o_scale) if isinstance(o_scale, SymbolScalar) else (repr(float(o_scale)) + "f", False)
     if oval[1]:
         raise NotImplementedError("o_scale must be one value per row")
-    body = [em.code()]
+    body = []
+    if id(kv_idx) in em.done:
+        body += ["  float kvf[N];", "#pragma unroll",
+                 "  for (int e = 0; e < N; e++) kvf[e] = (float)(ctx.kv_base + ae_kv_off(e));"]
+    body.append(em.code())
     if sval[0] != "s":
         src = f"{sval[0]}[e]" if sval[1] else sval[0]
         body += ["#pragma unroll", f"  for (int e = 0; e < N; e++) s[e] = {src};"]
@@ -159,6 +228,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
         if expr != f"st.{k}":
             body.append(f"  st.{k} = {expr};")
     online_fwd_body = "\n".join(body)
+    score_mod_body = "  // score_mod is fused into ae_online_fwd"
 
     # ---- epilogue -------------------------------------------------------------------------
     b, h, q_idx, _, leaves = index_leaves()

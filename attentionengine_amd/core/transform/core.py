@@ -22,6 +22,24 @@ from .graph import (Abs, Add, ColReduceAbsSum, ColReduceMax, ColReduceSum, Const
                     ReduceSum, Sub, Tanh, Var)
 
 
+_DIM_ORDER = {"num_split": 0, "block_M": 1, "seq_len": 1, "block_N": 2, "seq_len_kv": 2, "dimv": 2}
+
+
+def _broadcast_shape(shapes):
+    """Ordered union of dimension names; "1" entries are dropped when another dimension exists.
+    Known names are ordered (split, row, column); unknown names keep their order of appearance."""
+    dims = []
+    for sh in shapes:
+        for d in sh:
+            if d != "1" and d not in dims:
+                dims.append(d)
+    if not dims:
+        return ["1"] if any("1" in sh for sh in shapes) else []
+    if all(d in _DIM_ORDER for d in dims):
+        dims.sort(key=lambda d: _DIM_ORDER[d])
+    return dims
+
+
 class SymbolScalar:
     """A traced value: scalar per row (``shape_idx=["block_M"]``), a score tile
     (``["block_M","block_N"]``), a constant (``[]``) or a custom input tensor."""
@@ -83,11 +101,9 @@ class SymbolScalar:
                 raise TypeError(f"cannot trace operand of type {type(other).__name__}")
             operands.append(other)
         if shape_idx is None:
-            # elementwise result takes the widest operand shape (row op tile -> tile)
-            shape_idx = self.shape_idx
-            for o in operands:
-                if len(o.shape_idx) > len(shape_idx):
-                    shape_idx = o.shape_idx
+            # elementwise result broadcasts by dimension NAME (core/codegen/tl_gen.py:44-62):
+            # ordered union of the operands' dimensions, e.g. [block_M] op [block_N] -> tile
+            shape_idx = _broadcast_shape([self.shape_idx] + [o.shape_idx for o in operands])
         stem = self.varname if varname_suffix is None else f"{self.varname}_{varname_suffix}"
         node = code(*[x.code for x in [self] + operands])
         out = self.__class__.__new__(self.__class__)

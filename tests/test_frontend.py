@@ -116,9 +116,15 @@ def test_emitted_softmax_functors():
                           torch.float16)
     assert lf.rowstate_fields == ["m", "r"] and lf.rowstate_init == ["-1e38f", "0.0f"]
     assert lf.final_rowscale_names == ["lse"] and not lf.o_scale_one
-    assert "ae_row_max<N>(s)" in lf.online_fwd_body and "ae_row_sum<N>" in lf.online_fwd_body
-    # exp(scores - m_new) is fused into one fma + exp2 per element
-    assert "ae_exp2(__builtin_fmaf(s[e], AE_LOG2E" in lf.online_fwd_body
+    body = lf.online_fwd_body
+    assert "ae_row_sum<N>" in body
+    # affine folding: the score scale is applied to the row maximum (one multiply per row) and
+    # folded with log2(e) into the exponent, one fma + exp2 per element, no separate scaling pass
+    assert "ae_row_max<N>(s) * 0.125f" in body
+    assert f"ae_exp2(__builtin_fmaf(s[e], {0.125 * 1.4426950408889634!r}f" in body
+    assert "s[e] * 0.125f" not in body
+    # the graph is recognised as the online softmax: thresholded (lazy) running maximum
+    assert "> 5.545177444479562f) ?" in body and "ae_max(st.m" not in body
     assert "frs[0]" in lf.epilogue_body and "ae_log(st.r)" in lf.epilogue_body
     src = L.render_functors(lf)
     for name in ("ae_score_mod", "ae_online_fwd", "ae_epilogue", "ae_mask_mod", "ae_rowstate_init"):
@@ -130,7 +136,7 @@ def test_emitted_identity_and_custom_scalar():
                           CustomIO({"softmax_bias": (1,)}), torch.float16)
     assert lf.o_scale_one and lf.rowstate_fields == [] and lf.final_rowscale_names == []
     assert lf.customs[0].name == "softmax_bias" and lf.customs[0].torch_dtype == torch.float32
-    assert "ae_tanh" in lf.score_mod_body and "cust.softmax_bias" in lf.score_mod_body
+    assert "ae_tanh" in lf.online_fwd_body and "cust.softmax_bias" in lf.online_fwd_body
 
 
 def test_unsupported_graphs_raise():
@@ -202,3 +208,29 @@ def test_engine_error_behaviour():
     q = torch.zeros(1, 128, 2, 64, dtype=torch.float16)
     with pytest.raises(RuntimeError, match="no CPU path"):   # the product never falls back to the CPU
         mod(q, q, q)
+
+
+def test_lazy_maximum_only_for_the_online_softmax():
+    """The thresholded running maximum is applied only when the traced graph is provably the online
+    softmax; a function that exports m itself keeps the exact update."""
+    from attn_engine import OnlineFunc
+
+    class SoftmaxExportingMax(C.OnlineSoftmax):
+        @staticmethod
+        def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+            o_new = o / online_rowscales["r"]
+            return o_new, {"m": online_rowscales["m"] + 0.0}
+    lf = L.trace_functors(C.make_scale_score_mod(0.125), None, SoftmaxExportingMax(), CustomIO({}), torch.float16)
+    assert "ae_max(st.m" in lf.online_fwd_body and "5.545" not in lf.online_fwd_body
+    lf = L.trace_functors(C.make_scale_score_mod(0.125), None, C.OnlineAbsNorm(), CustomIO({}), torch.float16)
+    assert "5.545" not in lf.online_fwd_body
+
+
+def test_shapes_broadcast_by_name():
+    q = SymbolScalar("q_idx", Var("q_idx"), shape_idx=["block_M"])
+    kv = SymbolScalar("kv_idx", Var("kv_idx"), shape_idx=["block_N"])
+    assert (q - kv).shape_idx == ["block_M", "block_N"]
+    assert (kv - q).shape_idx == ["block_M", "block_N"]
+    s = SymbolicArray("s", Var("s"), shape_idx=["block_M", "block_N"])
+    assert (s - q).shape_idx == ["block_M", "block_N"] and (q * 2).shape_idx == ["block_M"]
+    assert s.get_reduce("max").shape_idx == ["block_M"]
