@@ -378,10 +378,15 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
 
 int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                       const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
-  if (!split || !combine || !combine_cfg)
+  if (!split || !combine_cfg)
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: kernel/cfg is NULL");
   int rc = check_common("ae_mla_decode_fwd", p, cfg);
   if (rc) return rc;
+  // with one split the kernel writes `out` itself and no merge pass runs
+  const bool direct = p->num_splits == 1;
+  if (!direct && !combine)
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: combine kernel is NULL with %d splits",
+                p->num_splits);
   if (!p->q2 || !p->k2)
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: rope pointers q2/k2 are NULL");
   if (p->seqlen_q != 1)
@@ -394,7 +399,7 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
   if (combine_cfg->block_n != p->num_splits)
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: combine kernel built for %d splits, got %d",
                 combine_cfg->block_n, p->num_splits);
-  if (!p->partial_o || !p->partial_rs)
+  if (!direct && (!p->partial_o || !p->partial_rs))
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: split-KV work buffers are NULL");
   if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: bad combine workgroup size %d",
@@ -412,7 +417,7 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
   uint32_t grid[3] = {(uint32_t)total, 1, 1};
   uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
   rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
-  if (rc) return rc;
+  if (rc || direct) return rc;
   uint32_t cgrid[3] = {(uint32_t)p->heads_q, (uint32_t)p->batch, 1};
   uint32_t cblock[3] = {(uint32_t)combine_cfg->threads, 1, 1};
   return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);

@@ -254,6 +254,25 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
 #pragma unroll
     for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
   }
+#if AE_NSPLIT == 1
+  // a single split needs no merge: write the output row and its rowscales directly
+  if (head_ok) {
+    ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)hq * p.o_stride_h +
+                    dvh * (AE_DV / 2);
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++) {
+      ae_elem4 w;
+#pragma unroll
+      for (int r = 0; r < 4; r++) w[r] = (ae_elem)o[db * 4 + r];
+      *(ae_elem4*)(optr + db * 16 + g4 * 4) = w;
+    }
+    if (g4 == 0 && dvh == 0) {
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+        if (p.rowscale_out[i]) p.rowscale_out[i][(int64_t)b * p.heads_q + hq] = frs[i];
+    }
+  }
+#else
   if (head_ok) {
     const int64_t row = ((int64_t)b * p.heads_q + hq) * p.num_splits + split;
     float* po = p.partial_o + row * AE_DV + dvh * (AE_DV / 2);
@@ -268,6 +287,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         p.partial_rs[(int64_t)i * p.batch * p.heads_q * p.num_splits + row] = frs[i];
     }
   }
+#endif
 }
 
 #include "ae_combine.h"

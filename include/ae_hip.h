@@ -191,6 +191,8 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
  *   kernel (mla_decode_tl.py:326-335) or `fwd_kvcache_mla`
  *   (cute_template_kvshared/flash_api.cpp:61-210). Every workgroup covers cfg->block_m query heads
  *   of one (batch, kv head, split); 1-D grid ordered so workgroups sharing a KV range run on one XCD.
+ *   With num_splits == 1 the split kernel writes `out` / `rowscale_out` itself: no merge pass runs,
+ *   `combine` may be NULL and the partial buffers are not touched.
  */
 int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                       const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
