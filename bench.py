@@ -112,6 +112,27 @@ def measure(name, steps, warmup):
     return res
 
 
+COPY_PROBE_BYTES = 256 << 20
+
+
+def copy_probe():
+    """One launch of a plain copy kernel over COPY_PROBE_BYTES (reads that many bytes, writes that many)."""
+    import ctypes
+    import torch
+    from core.runtime import hip_rt as rt
+
+    class CopyParams(ctypes.Structure):
+        _fields_ = [("src", ctypes.c_void_p), ("dst", ctypes.c_void_p), ("n_vec", ctypes.c_uint64)]
+    src = torch.ones(COPY_PROBE_BYTES // 4, dtype=torch.float32, device="cuda:0")
+    dst = torch.empty_like(src)
+    kern = rt.compile_module("ae_copy_probe.hip", {}).kernel("ae_copy_probe_kernel")
+    torch.cuda.synchronize()
+    kern.launch(CopyParams(src.data_ptr(), dst.data_ptr(), COPY_PROBE_BYTES // 16), (4096, 1, 1), (256, 1, 1), 0,
+                torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(src, dst)
+
+
 def cpu_baseline(name):
     """The CPU oracle on a bounded sample of the workload (one batch entry; heads in chunks so the
     [heads, S, S] fp32 score tensor stays below ~1 GiB), fp32 compute on the rounded inputs."""
@@ -177,6 +198,9 @@ def main():
     ap.add_argument("--workload", default="c2_causal", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one plain 256 MiB copy kernel (ae_copy_probe_kernel) so that a "
+                         "hardware-counter run can scale FETCH_SIZE / WRITE_SIZE by a known transfer")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the attention forward path on ONE GPU; "
@@ -191,6 +215,8 @@ def main():
     info = rt.device_info(0)
 
     head = measure(a.workload, a.steps, a.warmup)
+    if a.copy_probe:
+        copy_probe()
     unit = head["roofline"]["unit"]
     value = head["tflops"] if unit == "TFLOP/s" else head["gbs"]
     line = {
