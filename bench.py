@@ -41,6 +41,17 @@ WORKLOADS = {
 }
 
 
+# HBM bytes per launch of each workload's dominant kernel, measured once with the hardware counters
+# FETCH_SIZE and WRITE_SIZE (rocprofv3 --pmc, one counter per run, `--copy-probe` in the same run so
+# that a 256 MiB copy kernel calibrates the counter: FETCH_SIZE reads half the bytes moved, factor
+# 2.0; WRITE_SIZE factor 1.0).  Fetched + written.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {
+    "c2_causal": 204.2e6 + 68.2e6,       # algorithmic Q+K+V+O+lse: 269.5e6
+    "c4_gqa_decode": 2147.9e6 + 4.2e6,   # algorithmic K+V: 2147.5e6 (fp32 partials written: 4.2e6)
+    "c5_mla_decode": 622.9e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
+}
+
+
 def _inputs(name, device):
     """Synthetic N(0,1) inputs of the workload's shape, generated on the CPU with seed 0 in the
     order q, k, v (MLA: q, q_pe, kv, k_pe), rounded to the compute dtype, copied to the GPU."""
@@ -100,11 +111,11 @@ def measure(name, steps, warmup):
     if kind == "prefill":
         ach = info["flops"] / (ev_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                           "frac": ach / PEAK_MFMA_TFLOPS, "traffic": None}
+                           "frac": ach / PEAK_MFMA_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
     else:
         ach = info["bytes"] / (ev_ms * 1e-3) / 1e9
         res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                           "frac": ach / PEAK_HBM_GBS, "traffic": None}
+                           "frac": ach / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
         if kind == "mla_decode":
             res["mfma_frac"] = info["flops"] / (ev_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS
     del args, mod
