@@ -9,11 +9,13 @@ host needs at launch time.
 """
 from __future__ import annotations
 
+import math
+import os
 from dataclasses import dataclass, field
 
 import torch
 
-from ..codegen.hip_gen import Emitter, init_literal, var_as_constant
+from ..codegen.hip_gen import Emitter, float_literal, init_literal, var_as_constant
 from ..transform.core import CustomIO, SymbolicArray, SymbolScalar
 from ..transform.graph import Var
 from .mask import MASK_HELPERS, LoweredMask, MaskPlan, lower_mask_mod, plan_mask
@@ -46,6 +48,9 @@ class LoweredFunctors:
     o_scale_one: bool
     customs: list = field(default_factory=list)
     mask: LoweredMask = None
+    # (scale, max field, sum field) when the graph is the online softmax of `scores * scale`,
+    # scale > 0: the case the software-pipelined prefill kernel is written for
+    softmax: tuple = None
 
 
 def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
@@ -164,6 +169,25 @@ def find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale
             v.clear_codegen()
 
 
+def _pure_scale(sym, scores):
+    """The constant c if ``sym`` is ``scores`` multiplied / divided by python numbers only, else None."""
+    c = 1.0
+    while sym is not scores:
+        t = sym.code.type
+        if t not in ("Mul", "Div") or len(sym.prev) != 2:
+            return None
+        a, b = sym.prev
+        if b.code.type == "Const" and (t == "Mul" or float(b.code.value) != 0.0):
+            c = c * float(b.code.value) if t == "Mul" else c / float(b.code.value)
+            sym = a
+        elif a.code.type == "Const" and t == "Mul":
+            c *= float(a.code.value)
+            sym = b
+        else:
+            return None
+    return c
+
+
 def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO, in_dtype,
                    mask_value: str = "-inf") -> LoweredFunctors:
     """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
@@ -202,8 +226,14 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     new_scores, new_rowscales, o_scale = online_func.online_fwd(scores_mod, rowscales, b, h, q_idx)
     em = Emitter(leaves, {}, ["block_N"], n="N", prefix="of")
     lazy = find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale)
+    softmax = None
     if lazy is not None:
         em.lazy_max[id(lazy)] = LAZY_MAX_TAU
+        scale = _pure_scale(scores_mod, scores)
+        if scale is not None and scale > 0.0 and math.isfinite(scale):
+            (mk,) = [k for k, v in new_rowscales.items() if v is lazy]
+            (rk,) = [k for k in new_rowscales if k != mk]
+            softmax = (scale, mk, rk)
     new_vals = {k: em.value(v) for k, v in new_rowscales.items()}
     sval = em.value(new_scores)
     o_scale_const = var_as_constant(o_scale) if isinstance(o_scale, SymbolScalar) else float(o_scale)
@@ -257,6 +287,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
                          [k for k, _ in fvals], o_scale_one, customs, lowered_mask)
     lf.custom_fields = cust_fields
     lf.custom_loads = cust_loads
+    lf.softmax = softmax
     return lf
 
 
@@ -312,20 +343,35 @@ class PrefillTiles:
     waves_per_eu: int = 2
     k_pad: int = 0
     v_pad: int = 0
+    rows_per_wave: int = 32
 
     @property
     def block_m(self):
-        return 32 * self.n_waves
+        return self.rows_per_wave * self.n_waves
 
     def lds_bytes(self, d: int, dv: int) -> int:
         return 2 * self.block_n * ((2 * d + self.k_pad) + (2 * dv + self.v_pad))
 
 
-def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0) -> PrefillTiles:
-    """The direct-to-LDS kernel handles 128- and 256-byte K/V rows (head dims 64 and 128); other
-    head dims use the register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one
-    wave per SIMD and a shorter kv tile once the accumulators outgrow 256 registers."""
+# Compute units of an MI355X: the pipelined kernel's 256-row tiles are only chosen when there are
+# enough of them to occupy the chip.
+_MI355X_CUS = 256
+
+
+def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0) -> PrefillTiles:
+    """The direct-to-LDS kernels handle 128- and 256-byte K/V rows (head dims 64 and 128): the
+    software-pipelined one (64 rows per wave, 256-row q tiles, one wave per SIMD) when the graph is
+    the online softmax of scaled scores and the problem has enough q tiles to occupy the chip
+    (measured on B2 H32 S4096 D128 fp16: 1.0 against 0.86 PFLOP/s non-causal), otherwise the generic
+    one (32 rows per wave, two waves per SIMD, runs any functor).  Other head dims use the
+    register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one wave per SIMD and a
+    shorter kv tile once the accumulators outgrow 256 registers.  AE_PREFILL_KERNEL=generic|pipelined
+    overrides the choice between the first two (tests)."""
     if d in (64, 128) and dv in (64, 128):
+        force = os.environ.get("AE_PREFILL_KERNEL", "")
+        n_tiles = batch_heads * ((seqlen_q + 255) // 256)
+        if softmax is not None and force != "generic" and (force == "pipelined" or n_tiles >= (3 * _MI355X_CUS) // 4):
+            return PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)
         return PrefillTiles()
     t = PrefillTiles(template="ae_prefill_simple.hip", k_pad=16)
     if max(d, dv) > 128:
@@ -338,8 +384,12 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0) -> PrefillTiles:
 
 
 def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, has_mask_mod: bool,
-                  n_rowscales: int, o_scale_one: bool, even_q: bool, even_kv: bool) -> str:
+                  n_rowscales: int, o_scale_one: bool, even_q: bool, even_kv: bool, softmax=None) -> str:
     """Text of ae_config.h."""
+    extra = []
+    if softmax is not None:
+        extra = [f"#define AE_SM_SCALE {float_literal(softmax[0])}", f"#define AE_SM_M {softmax[1]}",
+                 f"#define AE_SM_R {softmax[2]}"]
     return "\n".join([
         "// generated by core/lower/lower.py -- do not edit",
         f"#define AE_D {d}",
@@ -356,5 +406,6 @@ def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, h
         f"#define AE_WAVES_PER_EU {tiles.waves_per_eu}",
         f"#define AE_K_PAD {tiles.k_pad}",
         f"#define AE_V_PAD {tiles.v_pad}",
+        *extra,
         "",
     ])

@@ -39,7 +39,12 @@ class PrefillOp:
         self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
                                          self.dtype, mask_value)
         self.functor_src = L.render_functors(self.functors)
-        self.tiles = L.choose_prefill_tiles(self.D, self.DV, 0 if isinstance(q_meta.shape[2], str) else int(q_meta.shape[2]))
+        self.tiles = L.choose_prefill_tiles(self.D, self.DV, _dim(q_meta.shape[2], 0), self.functors.softmax,
+                                            _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1))
+        if self.extern_block_mask and self.tiles.rows_per_wave != 32 and (
+                self.mask_block[1] % self.tiles.block_n or
+                (self.tiles.block_m % self.mask_block[0] and self.mask_block[0] % self.tiles.block_m)):
+            self.tiles = L.PrefillTiles()     # the pipelined kernel's kv tile is fixed; use the generic one
         if self.extern_block_mask:
             # a q tile covers whole block-mask rows, a kv tile sits inside one block-mask column
             while self.tiles.block_n > self.mask_block[1] and self.tiles.block_n > 32:
@@ -109,7 +114,8 @@ class PrefillOp:
         if v is None:
             has_mask_mod = self.elementwise_mask and mask_mode != 1
             cfg_src = L.render_config(self.D, self.DV, self.dtype, self.tiles, mask_mode, has_mask_mod,
-                                      self.n_rowscales, self.functors.o_scale_one, even_q, even_kv)
+                                      self.n_rowscales, self.functors.o_scale_one, even_q, even_kv,
+                                      self.functors.softmax if self.tiles.rows_per_wave == 64 else None)
             module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,
                                                           "ae_functors.h": self.functor_src})
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,

@@ -52,6 +52,19 @@ AE_DEV ae_f32x4 ae_mfma16(ae_elem8 a, ae_elem8 b, ae_f32x4 c) {
 #endif
 }
 
+// ---- direct HBM -> LDS load --------------------------------------------------------------------
+// 16 bytes per lane from `gptr` (any per-lane address) to LDS at lds_base + lane*16, lds_base wave
+// uniform.  Issued as inline assembly rather than through __builtin_amdgcn_global_load_lds: when the
+// compiler knows about a pending LDS-DMA write it makes every LDS read it cannot prove disjoint
+// (all ds_read_tr*, which carry no precise memory operand) wait for vmcnt(0), i.e. for the tile that
+// was just requested for LATER, which serialises the prefetch.  Callers order these loads against
+// their consumers themselves: s_waitcnt vmcnt(..) followed by a workgroup barrier.
+typedef __attribute__((address_space(3))) unsigned char ae_lds_u8;
+AE_DEV void ae_load_lds16(const void* gptr, ae_lds_u8* lds_base) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(m0v) : "memory");
+}
+
 // ---- transcendentals ------------------------------------------------------------------
 AE_DEV float ae_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 AE_DEV float ae_exp(float x) { return __builtin_amdgcn_exp2f(x * AE_LOG2E); }

@@ -123,8 +123,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
       kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
       const ae_elem* src = c < AE_CPR1 ? k1 + (int64_t)kv * p.k_stride_s + c * 8
                                        : k2 + (int64_t)kv * p.k2_stride_s + (c - AE_CPR1) * 8;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)(dst + blk * 1024), 16, 0, 0);
+      ae_load_lds16(src, dst + blk * 1024);
     }
   };
 
@@ -153,6 +152,10 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   const int v_c0 = (lane & 3) >> 1;
 
   // ---- pipeline: AE_NSTAGE - 1 tiles in flight ahead of the one being multiplied -----------------
+  // The tile loads are invisible to the compiler's wait-count bookkeeping (see ae_load_lds16), so
+  // everything it does know about (the Q fragments) is drained first: otherwise it would wait for
+  // "its" loads with a vmcnt(0) inside the loop, which also waits for every tile in flight.
+  __builtin_amdgcn_s_waitcnt(0x0F70);
 #pragma unroll
   for (int t = 0; t < AE_NSTAGE - 1; t++)
     if (t < n_tiles) load_tile(t, t);

@@ -1,0 +1,606 @@
+// Software-pipelined flash attention forward (prefill) for gfx950 / CDNA4: online softmax only.
+//
+// Same role and operation order as ae_prefill.hip (the reference's TileLang prefill template,
+// attention_engine/core/template/tl_template/attn/attn_tl.py:76-174, and its block-sparse sibling
+// blockattn_tl.py:49-160), specialised for the case the lowering has PROVEN to be the online
+// softmax of attn_script/mha.py:47-72 applied to `score * constant`:
+//     m' = max(m, rowmax(s*c)), p = exp(s*c - m'), r' = r*exp(m - m') + rowsum(p), O' = O*exp(m - m') + pV
+// Any other score_mod / OnlineFunc graph uses ae_prefill.hip, which runs the generated functors.
+//
+// Why a second kernel: with 32 query rows per wave every 32x32x16 MFMA needs a fresh 1 KiB A
+// fragment (K or V^T) from LDS, and four SIMDs issuing MFMAs back to back then ask LDS for exactly
+// its peak bandwidth.  Here a wave owns 64 query rows, so every fragment feeds two MFMAs and LDS
+// traffic per flop halves.  The price is 128 (O) + 64 (S) accumulator registers + 64 for Q: one wave
+// per SIMD, so no second wave hides the softmax arithmetic.  It is hidden by software pipelining
+// inside the wave instead.  Measured on MI355X: a wave issues one instruction per 4 cycles, a
+// 32x32x16 MFMA keeps the matrix pipe busy for 32 cycles but the wave's issue port for only about 16,
+// v_exp_f32 costs 8; so the rest of an MFMA's time is free for independent VALU work.  One loop
+// iteration therefore interleaves, MFMA by MFMA,
+//     phase 1:  S(j+1) = K(j+1) Q^T   with   p(j) = exp2(s(j)*c*log2e - m*log2e), row sums, fp16 cast
+//     phase 2:  O += V(j)^T p(j)^T     with   reading S(j+1) out of its accumulators, row maxima
+// with `sched_barrier` fences pinning the interleaving, the exponentiation split into stages (fma,
+// exp2, pack + sum) that run in different MFMA slots so no instruction waits for the one just
+// issued, A fragments read from LDS a few MFMAs ahead of their use into a small register ring, and
+// the tile loads (HBM -> LDS direct) issued one instruction at a time from the phase-1 slots.
+// The rescale of O happens outside the hot loop (lazy running maximum: it is rare).
+//
+// Configuration ("ae_config.h"): AE_D AE_DV AE_BN(=64) AE_NWAVES AE_DTYPE_BF16 AE_MASK_MODE
+// AE_HAS_MASK_MOD AE_N_ROWSCALES AE_EVEN_Q AE_EVEN_KV, plus AE_SM_SCALE (the constant c > 0) and
+// AE_SM_M / AE_SM_R (names of the running-max and running-sum fields of ae_rowstate).
+// Functors used ("ae_functors.h"): ae_rowstate, ae_rowstate_init, ae_mask_mod, ae_epilogue,
+// ae_load_custom.
+
+#include "ae_hip.h"
+#include "ae_config.h"
+#include "ae_device.h"
+#include "ae_functors.h"
+
+#define AE_WROWS 64                // query rows per wave (two 32-row blocks)
+#define AE_BM (AE_NWAVES * AE_WROWS)
+#define AE_NT (AE_NWAVES * 64)
+#define AE_NKS (AE_D / 16)         // k-steps of S^T = K Q^T
+#define AE_NKF (AE_NKS * 2)        // K fragments per tile (two 32-row kv blocks per k-step)
+#define AE_NDB (AE_DV / 32)        // 32-wide dv blocks
+#define AE_NVF (4 * AE_NDB)        // V^T fragments per tile (four 16-deep k-steps)
+#define AE_NO (AE_NDB * 16)
+#define AE_KSTR (AE_D * 2)
+#define AE_VSTR (AE_DV * 2)
+#define AE_K_BYTES (AE_BN * AE_KSTR)
+#define AE_V_BYTES (AE_BN * AE_VSTR)
+#define AE_KCPR (AE_D / 8)
+#define AE_VCPR (AE_DV / 8)
+#define AE_K_LOADS ((AE_BN * AE_KCPR) / AE_NT)
+#define AE_V_LOADS ((AE_BN * AE_VCPR) / AE_NT)
+#define AE_K_RPI (64 / AE_KCPR)
+#define AE_V_RPI (64 / AE_VCPR)
+#define AE_VPPR (AE_VCPR / 2)
+#define AE_VPS1 (32 / AE_NKF)      // scores per row handled next to one phase-1 MFMA
+#define AE_VPS2 (32 / AE_NVF)      // scores per row read back next to one phase-2 MFMA
+#ifndef AE_AHEAD
+#define AE_AHEAD 3                 // fragments in flight ahead of the MFMA that uses them
+#endif
+#define AE_RING (AE_AHEAD + 1)
+#ifndef AE_EXP_SPAN
+#define AE_EXP_SPAN (2 * AE_NKF + 8)   // MFMA slots over which the 32 exponentiation units of a tile start
+#endif
+#define AE_TAU 5.545177444479562f  // 8 ln 2: the running maximum is refreshed only when it moved by more
+
+static_assert(AE_BN == 64, "the pipelined kernel is written for 64-wide kv tiles");
+static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
+static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
+static_assert((AE_BN * AE_KCPR) % AE_NT == 0 && (AE_BN * AE_VCPR) % AE_NT == 0, "tile / workgroup split");
+static_assert(AE_VPS2 >= 2, "work split");
+// k-step kk of O^T += V^T P^T starts in slot 2*NKF + 2*NDB*kk; its last unit (8*kk+7) must be done
+static_assert(((7 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF, "exp units of k-step 0 finish in phase 1");
+static_assert(((31 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 6 * AE_NDB, "exp units of k-step 3 finish in time");
+static_assert(((23 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 4 * AE_NDB, "exp units of k-step 2 finish in time");
+static_assert(((15 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 2 * AE_NDB, "exp units of k-step 1 finish in time");
+
+typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
+#define AE_SB() __builtin_amdgcn_sched_barrier(0)
+
+struct ae_tag_true { static constexpr bool value = true; };
+struct ae_tag_false { static constexpr bool value = false; };
+
+extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void ae_prefill_kernel(const ae_attn_params p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
+  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // [2][K tile] then [2][V tile]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hf = lane >> 5;
+
+  // ---- which (q-tile, head, batch): ids dealt so that the heads sharing K/V meet in one XCD's L2,
+  // heavy causal q-tiles first (see ae_prefill.hip) -------------------------------------------
+  const int n_qt = (p.seqlen_q + AE_BM - 1) / AE_BM;
+  const int n_bh = p.batch * p.heads_q;
+  const int wg = blockIdx.x;
+  const int xcd = wg & 7;
+  const int slot = wg >> 3;
+  const int qt_i = slot % n_qt;
+  const int bh = (slot / n_qt) * 8 + xcd;
+  if (bh >= n_bh) return;
+#if AE_MASK_MODE == 1
+  const int qt = n_qt - 1 - qt_i;
+#else
+  const int qt = qt_i;
+#endif
+  const int h = bh % p.heads_q;
+  const int b = bh / p.heads_q;
+  const int hk = h / (p.heads_q / p.heads_kv);
+  const int q0 = qt * AE_BM;
+  const int q0w = q0 + wave * AE_WROWS;
+  int qrow[2];
+  bool q_ok[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    qrow[qb] = q0w + qb * 32 + l32;
+#if AE_EVEN_Q
+    q_ok[qb] = true;
+#else
+    q_ok[qb] = qrow[qb] < p.seqlen_q;
+#endif
+  }
+
+  // ---- Q fragments (B operand of S^T = K Q^T), resident ------------------------------------
+  ae_elem8 qf[2][AE_NKS];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    const int qr = q_ok[qb] ? qrow[qb] : p.seqlen_q - 1;
+    const ae_elem* qptr = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)qr * p.q_stride_s +
+                          (int64_t)h * p.q_stride_h;
+#pragma unroll
+    for (int ks = 0; ks < AE_NKS; ks++) qf[qb][ks] = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
+  }
+
+  // ---- KV tile range and tile classes --------------------------------------------------------
+  const int n_kvt = (p.seqlen_kv + AE_BN - 1) / AE_BN;
+  int j_end = n_kvt;
+#if AE_MASK_MODE == 1
+  {
+    int lim = (q0 + AE_BM + AE_BN - 1) / AE_BN;   // attn_tl.py:113-115
+    j_end = lim < n_kvt ? lim : n_kvt;
+  }
+#endif
+#if AE_MASK_MODE == 2
+  const int8_t* bm_base = p.block_mask +
+      ((int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : h)) * p.mask_nq * (int64_t)p.mask_nkv;
+  const int bm_r0 = q0 / p.mask_block_m;
+  int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
+  bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
+  auto tile_class = [&](int j) -> int {   // 0 skip, 1 elementwise mask, 2 fully visible
+    const int col = (j * AE_BN) / p.mask_block_n;
+    int any = 0, all = 2;
+    for (int r = bm_r0; r <= bm_r1; r++) {
+      int c = bm_base[(int64_t)r * p.mask_nkv + col];
+      any |= c;
+      all = c < all ? c : all;
+    }
+    return any == 0 ? 0 : (all == 2 ? 2 : 1);
+  };
+#endif
+  auto next_tile = [&](int j) {
+#if AE_MASK_MODE == 2
+    while (j < j_end && tile_class(j) == 0) j++;
+#endif
+    return j < j_end ? j : j_end;
+  };
+  // does tile j need the elementwise mask for this wave's rows?
+  auto needs_mask = [&](int j) -> bool {
+    bool nm = false;
+#if AE_MASK_MODE == 1
+    nm = j * AE_BN + AE_BN - 1 > q0w;
+#elif AE_MASK_MODE == 2
+    // the table may be finer than the 256-row q tile (user block masks): rows of one workgroup, even of
+    // one wave, can differ in class, so anything but "every table row of this wave says fully visible"
+    // takes the masked path, which looks the class up per row
+    {
+      const int col = (j * AE_BN) / p.mask_block_n;
+      int r1 = (q0w + AE_WROWS - 1) / p.mask_block_m;
+      r1 = r1 < p.mask_nq ? r1 : p.mask_nq - 1;
+      for (int r = q0w / p.mask_block_m; r <= r1; r++) nm = nm || (bm_base[(int64_t)r * p.mask_nkv + col] != 2);
+    }
+#elif AE_HAS_MASK_MOD
+    nm = true;
+#endif
+#if !AE_EVEN_KV
+    nm = nm || (j * AE_BN + AE_BN > p.seqlen_kv);
+#endif
+    return nm;
+  };
+
+  const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
+  const ae_elem* vbase = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
+
+  // Direct HBM -> LDS tile loads with the chunk swizzles of ae_prefill.hip.  A lane's byte offset
+  // inside a tile never changes, so it is computed once; per tile only a wave-uniform base moves.
+  unsigned koff[AE_K_LOADS], voff[AE_V_LOADS];
+#pragma unroll
+  for (int i = 0; i < AE_K_LOADS; i++) {
+    const int row = (wave * AE_K_LOADS + i) * AE_K_RPI + lane / AE_KCPR;
+    const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
+    koff[i] = (unsigned)(row * (int)p.k_stride_s + c * 8) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < AE_V_LOADS; i++) {
+    const int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
+    const int cp = lane % AE_VCPR;
+    const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
+    voff[i] = (unsigned)(row * (int)p.v_stride_s + c * 8) * 2u;
+  }
+  auto load_k_part = [&](int j, int stage, int i) {
+    ae_lds_byte* ks = lds + stage * AE_K_BYTES;
+    const char* g = (const char*)kbase + (int64_t)j * AE_BN * p.k_stride_s * 2;
+    const int blk = wave * AE_K_LOADS + i;
+    unsigned off = koff[i];
+#if !AE_EVEN_KV
+    if (j * AE_BN + AE_BN > p.seqlen_kv) {   // rows past the end re-read the last row (masked later)
+      const int row = blk * AE_K_RPI + lane / AE_KCPR;
+      const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
+      const int last = p.seqlen_kv - 1 - j * AE_BN;
+      off = (unsigned)((row < last ? row : last) * (int)p.k_stride_s + c * 8) * 2u;
+    }
+#endif
+    ae_load_lds16(g + off, ks + blk * 1024);
+  };
+  auto load_k = [&](int j, int stage) {
+#pragma unroll
+    for (int i = 0; i < AE_K_LOADS; i++) load_k_part(j, stage, i);
+  };
+  auto load_v_part = [&](int j, int stage, int i) {
+    ae_lds_byte* vs = lds + 2 * AE_K_BYTES + stage * AE_V_BYTES;
+    const char* g = (const char*)vbase + (int64_t)j * AE_BN * p.v_stride_s * 2;
+    const int blk = wave * AE_V_LOADS + i;
+    unsigned off = voff[i];
+#if !AE_EVEN_KV
+    if (j * AE_BN + AE_BN > p.seqlen_kv) {
+      const int row = blk * AE_V_RPI + lane / AE_VCPR;
+      const int cp = lane % AE_VCPR;
+      const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
+      const int last = p.seqlen_kv - 1 - j * AE_BN;
+      off = (unsigned)((row < last ? row : last) * (int)p.v_stride_s + c * 8) * 2u;
+    }
+#endif
+    ae_load_lds16(g + off, vs + blk * 1024);
+  };
+  auto load_v = [&](int j, int stage) {
+#pragma unroll
+    for (int i = 0; i < AE_V_LOADS; i++) load_v_part(j, stage, i);
+  };
+
+  // ---- state ------------------------------------------------------------------------------
+  ae_ctx ctx[2];
+  ae_custom cust[2];
+  ae_rowstate st[2];
+  ae_f32x16 oacc[2][AE_NDB];
+  float m_run[2], r_run[2], negm2[2], osc[2];
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    ctx[qb].b = b;
+    ctx[qb].h = h;
+    ctx[qb].q_idx = qrow[qb];
+    ctx[qb].kv_base = 0;
+    ae_load_custom(cust[qb], p, ctx[qb]);
+    ae_rowstate_init(st[qb]);
+    m_run[qb] = st[qb].AE_SM_M;
+    r_run[qb] = st[qb].AE_SM_R;       // per-lane partial sum; the two halves of a row meet in the epilogue
+    negm2[qb] = 0.f;
+    osc[qb] = 1.f;
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[qb][db][r] = 0.f;
+  }
+
+  // lane-constant pieces of the swizzled LDS fragment addresses (see ae_prefill.hip)
+  const int k_row_off = l32 * AE_KSTR;
+  const int k_sw = l32 & (AE_KCPR - 1);
+  const int v_row = 4 * hf + ((lane & 15) >> 2);
+  const int v_row_off = v_row * AE_VSTR + (lane & 3) * 8;
+  const int v_sw = v_row & (AE_VPPR - 1);
+  const int v_g = l32 >> 4;
+
+  // K fragment f = (k-step f/2, kv block f%2); V^T fragment f = (k-step f/NDB, dv block f%NDB)
+  auto read_kfrag = [&](int f, const ae_lds_byte* kt) -> ae_elem8 {
+    const int ks = f >> 1, nb = f & 1;
+    return *(const __attribute__((address_space(3))) ae_elem8*)(
+        kt + k_row_off + nb * 32 * AE_KSTR + (((2 * ks + hf) ^ k_sw) << 4));
+  };
+  auto read_vfrag = [&](int f, const ae_lds_byte* vt) -> ae_elem8 {
+    const int kk = f / AE_NDB, db = f % AE_NDB;
+    const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
+    const ae_lds_byte* a0 = vt + v_row_off + rb0 * AE_VSTR + (((2 * db + v_g) ^ v_sw) << 5);
+    ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)a0);
+    ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) ae_s16x4*)(a0 + 8 * AE_VSTR));
+    return __builtin_bit_cast(ae_elem8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  ae_f32x16 sacc[2][2];     // [kv block][q block] accumulators of the tile being multiplied
+  float sv[2][32];          // [q block][score]: the tile being exponentiated (raw scores, masked)
+  float mx[2];              // lane-local maxima of sv
+  ae_elem8 pf[2][4];        // [q block][k-step] P^T fragments (B operand of O^T += V^T P^T)
+  ae_elem8 ring[AE_RING];
+  bool rescale = false;
+
+  // read S out of its accumulators (q block qb, scores e0 .. e0+n-1) and track the maximum
+  auto read_scores = [&](int qb, int e0, int n) {
+#pragma unroll
+    for (int e = e0; e < e0 + n; e++) {
+      float x = sacc[e >> 4][qb][e & 15];
+      // pin the copy into an ordinary VGPR here, in the MFMA shadow; otherwise the register
+      // allocator keeps the value in the accumulator file and re-reads it at the top of the loop
+      asm volatile("" : "+v"(x));
+      sv[qb][e] = x;
+      mx[qb] = __builtin_fmaxf(mx[qb], x);
+    }
+  };
+  // p = exp2(s*c*log2e - m*log2e), two scores at a time ("unit" u: q block u%2, k-step u/8, pair
+  // (u/2)%4 of that k-step's 8 scores), in three stages that run in DIFFERENT MFMA slots so that no
+  // instruction waits for the one just issued: A = fma, B = exp2, C = convert + row sum.  Unit u
+  // starts in slot ae_unit_slot(u); units are ordered by k-step, the order O^T += V^T P^T needs them.
+  float rsum[2];
+  float xa[32][2];
+  auto stage_a = [&](int u) {
+    const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
+    xa[u][0] = __builtin_fmaf(sv[qb][e], AE_SM_SCALE * AE_LOG2E, negm2[qb]);
+    xa[u][1] = __builtin_fmaf(sv[qb][e + 1], AE_SM_SCALE * AE_LOG2E, negm2[qb]);
+  };
+  auto stage_b = [&](int u) {
+    xa[u][0] = ae_exp2(xa[u][0]);
+    xa[u][1] = ae_exp2(xa[u][1]);
+  };
+  auto stage_c = [&](int u) {
+    const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
+    const ae_elem h0 = (ae_elem)xa[u][0], h1 = (ae_elem)xa[u][1];
+    pf[qb][e >> 3][e & 7] = h0;
+    pf[qb][e >> 3][(e & 7) + 1] = h1;
+#if AE_DTYPE_BF16
+    // bf16 keeps 8 significant bits: summing the rounded values would put ~1e-3 into lse for rows
+    // with few visible keys, so the fp32 values are summed (fp16 sums the rounded pairs in one v_dot2)
+    rsum[qb] += xa[u][0] + xa[u][1];
+#else
+    typedef _Float16 ae_h2 __attribute__((ext_vector_type(2)));
+    ae_h2 hv = {h0, h1};
+    ae_h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+    rsum[qb] = __builtin_amdgcn_fdot2(hv, one, rsum[qb], false);
+#endif
+  };
+  auto exp_slot = [&](int g) {      // the stages that belong to MFMA slot g of an iteration
+#pragma unroll
+    for (int u = 0; u < 32; u++) {
+      const int a = (u * AE_EXP_SPAN) / 32;
+      if (a + 2 == g) stage_c(u);
+      if (a + 1 == g) stage_b(u);
+      if (a == g) stage_a(u);
+    }
+  };
+  auto exp_all = [&]() {            // all stages back to back (no MFMA to hide behind)
+#pragma unroll
+    for (int u = 0; u < 32; u++) stage_a(u);
+#pragma unroll
+    for (int u = 0; u < 32; u++) stage_b(u);
+#pragma unroll
+    for (int u = 0; u < 32; u++) stage_c(u);
+  };
+  // mask fix-up of sv for tile j, then the row maxima, the (lazy) running maximum and the factors
+  auto finish_scores = [&](int j) {
+    const int kvb = j * AE_BN + 4 * hf;
+    if (needs_mask(j)) {
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        mx[qb] = AE_NEG_INF;
+#if AE_MASK_MODE == 2
+        int rr = qrow[qb] / p.mask_block_m;
+        rr = rr < p.mask_nq ? rr : p.mask_nq - 1;
+        const int cls = bm_base[(int64_t)rr * p.mask_nkv + (j * AE_BN) / p.mask_block_n];   // this row's class
+#endif
+#pragma unroll
+        for (int e = 0; e < 32; e++) {
+          const int kv = kvb + ae_kv_off(e);
+          bool vis = true;
+#if AE_MASK_MODE == 1
+          vis = qrow[qb] >= kv;
+#elif AE_MASK_MODE == 2
+#if AE_HAS_MASK_MOD
+          vis = cls == 2 || (cls == 1 && ae_mask_mod(b, h, qrow[qb], kv));
+#else
+          vis = cls != 0;
+#endif
+#elif AE_HAS_MASK_MOD
+          vis = ae_mask_mod(b, h, qrow[qb], kv);
+#endif
+#if !AE_EVEN_KV
+          vis = vis && (kv < p.seqlen_kv);
+#endif
+          sv[qb][e] = vis ? sv[qb][e] : AE_NEG_INF;
+          mx[qb] = __builtin_fmaxf(mx[qb], sv[qb][e]);
+        }
+      }
+    }
+    bool any_need = false;
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      float hi;
+      const float lo = ae_swap32_lo_hi(mx[qb], hi);
+      const float sc = __builtin_fmaxf(lo, hi) * AE_SM_SCALE;
+      const bool need = (sc - m_run[qb]) > AE_TAU;
+      const float mn = need ? sc : m_run[qb];
+      osc[qb] = need ? ae_exp(m_run[qb] - mn) : 1.0f;
+      m_run[qb] = mn;
+      negm2[qb] = -mn * AE_LOG2E;
+      any_need = any_need || need;
+    }
+    rescale = __builtin_amdgcn_ballot_w64(any_need) != 0;
+  };
+
+  // ---- prologue: first tile's scores ------------------------------------------------------------
+  int j0 = next_tile(0);                  // tile whose scores are in sv (exp + PV next)
+  const bool any_tile = j0 < j_end;
+  int j1 = any_tile ? next_tile(j0 + 1) : j_end;   // tile multiplied by Q next
+  if (any_tile) {
+    load_k(j0, 0);
+    load_v(j0, 0);
+    if (j1 < j_end) load_k(j1, 1);
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (any_tile) {
+#pragma unroll
+    for (int f = 0; f < AE_NKF; f++) {
+      const ae_elem8 kf = read_kfrag(f, lds);
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        ae_f32x16 c = sacc[f & 1][qb];
+        if (f < 2) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) c[r] = 0.f;
+        }
+        sacc[f & 1][qb] = ae_mfma32(kf, qf[qb][f >> 1], c);
+      }
+    }
+    mx[0] = mx[1] = AE_NEG_INF;
+    read_scores(0, 0, 32);
+    read_scores(1, 0, 32);
+    finish_scores(j0);
+    rescale = false;                       // O is still zero
+  }
+  __syncthreads();                         // everyone is done with K stage 0 before it is refilled
+
+  // ---- main loop ----------------------------------------------------------------------------------
+  // iteration n: loads K(n+2) -> K stage n%2, V(n+1) -> V stage (n+1)%2;
+  //              phase 1 multiplies K(n+1) (K stage (n+1)%2), phase 2 multiplies V(n) (V stage n%2).
+  int n = 0;
+  auto iteration = [&](auto has_next_tag) {
+    constexpr bool HN = decltype(has_next_tag)::value;
+    const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
+    const ae_lds_byte* vt = lds + 2 * AE_K_BYTES + (n & 1) * AE_V_BYTES;
+    const int j2 = HN ? next_tile(j1 + 1) : j_end;
+    // Nothing is in flight here on the back edge (the iteration ends with vmcnt(0)); saying so
+    // also clears loads still pending on loop ENTRY (Q fragments, spill reloads), which the
+    // compiler's wait-count insertion would otherwise wait for after this iteration's tile loads
+    // have been issued, i.e. with a vmcnt(0) that serialises them.
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);
+    // The tile loads of this iteration, K(j2) and V(j1), are issued one instruction at a time from
+    // the phase-1 slots below (a burst here costs ~600 cycles of issue that nothing hides).  When
+    // there is no tile j2 the K stage is refilled with the last tile, which nobody reads.
+    const int j2l = j2 < j_end ? j2 : j_end - 1;
+    // fragment stream of this iteration: K fragments 0..NKF-1 (if HN) then V fragments
+    constexpr int NF1 = HN ? AE_NKF : 0;
+    constexpr int NF = NF1 + AE_NVF;
+    auto read_frag = [&](int f) -> ae_elem8 {
+      return f < NF1 ? read_kfrag(f, kt) : read_vfrag(f - NF1, vt);
+    };
+#pragma unroll
+    for (int f = 0; f < AE_AHEAD && f < NF; f++) ring[f % AE_RING] = read_frag(f);
+    rsum[0] = rsum[1] = 0.f;
+    AE_SB();
+
+    // ---- phase 1: S(j1)^T = K Q^T  ||  p(j0) --------------------------------------------------
+    if (HN) {
+#pragma unroll
+      for (int f = 0; f < AE_NKF; f++) {
+        if (f + AE_AHEAD < NF) ring[(f + AE_AHEAD) % AE_RING] = read_frag(f + AE_AHEAD);
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+          ae_f32x16 c = sacc[f & 1][qb];
+          if (f < 2) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) c[r] = 0.f;
+          }
+          sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], c);
+          exp_slot(2 * f + qb);
+          {
+            constexpr int NL = AE_K_LOADS + AE_V_LOADS, EVERY = (2 * AE_NKF) / NL;
+            const int g = 2 * f + qb;
+            if (g % EVERY == EVERY - 1 && g / EVERY < NL) {
+              const int i = g / EVERY;
+              if (i < AE_K_LOADS) load_k_part(j2l, n & 1, i);
+              else load_v_part(j1, (n + 1) & 1, i - AE_K_LOADS);
+            }
+          }
+          AE_SB();
+        }
+      }
+    } else {
+      exp_all();
+    }
+    if (HN) mx[0] = mx[1] = AE_NEG_INF;
+    AE_SB();
+    // ---- phase 2: O^T += V(j0)^T P^T  ||  read S(j1) -----------------------------------------------
+#pragma unroll
+    for (int f = 0; f < AE_NVF; f++) {
+      const int fs = NF1 + f;
+      if (fs + AE_AHEAD < NF) ring[(fs + AE_AHEAD) % AE_RING] = read_frag(fs + AE_AHEAD);
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        oacc[qb][f % AE_NDB] = ae_mfma32(ring[fs % AE_RING], pf[qb][f / AE_NDB], oacc[qb][f % AE_NDB]);
+        if (HN) {
+          exp_slot(2 * AE_NKF + 2 * f + qb);
+          read_scores(qb, f * AE_VPS2, AE_VPS2);
+        }
+        AE_SB();
+      }
+    }
+    // running sums (with the factor that belongs to tile j0), then the next tile's maxima and factors
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) r_run[qb] = r_run[qb] * osc[qb] + rsum[qb];
+    if (HN) finish_scores(j1);
+    // tiles for the next iteration must have landed, and everyone must be done with this one's
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);   // vmcnt(0)
+    __syncthreads();
+    j0 = j1;
+    j1 = j2;
+    n++;
+  };
+
+  // The rescale of O (rare once the running maximum has settled) stays OUTSIDE the hot loop: inside
+  // it, O would have to be reachable by VALU instructions on every iteration and the register
+  // allocator then shuttles all 128 accumulator registers between the two register files per tile.
+  auto rescale_o = [&]() {
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+      for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[qb][db][r] *= osc[qb];
+    rescale = false;
+  };
+  if (any_tile) {
+    while (true) {
+      while (j1 < j_end && !rescale) iteration(ae_tag_true{});
+      if (rescale) {
+        rescale_o();
+        continue;
+      }
+      break;
+    }
+    iteration(ae_tag_false{});
+  }
+
+  // ---- epilogue -------------------------------------------------------------------------------
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++) {
+    float o[AE_NO];
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[db * 16 + r] = oacc[qb][db][r];
+    float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+    frs[0] = 0.f;
+    if (any_tile) {
+      st[qb].AE_SM_M = m_run[qb];
+      st[qb].AE_SM_R = ae_group_sum(r_run[qb]);
+      ae_epilogue<AE_NO>(o, st[qb], frs, ctx[qb], cust[qb]);
+      // a row that saw tiles but no visible key: out = 0 (as for a q tile without any tile), not 0/0
+      if (st[qb].AE_SM_R == 0.f) {
+#pragma unroll
+        for (int e = 0; e < AE_NO; e++) o[e] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
+    }
+    if (q_ok[qb]) {
+      ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow[qb] * p.o_stride_s +
+                      (int64_t)h * p.o_stride_h;
+#pragma unroll
+      for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int t = 0; t < 4; t++) w[t] = (ae_elem)o[db * 16 + rg * 4 + t];
+          *(ae_elem4*)(optr + db * 32 + rg * 8 + hf * 4) = w;
+        }
+      if (hf == 0) {
+#pragma unroll
+        for (int i = 0; i < AE_N_ROWSCALES; i++)
+          p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[qb]] = frs[i];
+      }
+    }
+  }
+}

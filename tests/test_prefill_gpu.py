@@ -214,3 +214,34 @@ def test_abs_norm_online_func(cuda_device):
     ref, finals = online_attention(q, k, v, sm, None, C.OnlineAbsNorm(), block_n=64)
     assert (mod.final_rowscales["r"].cpu() - finals["r"].float()).abs().max().item() <= 1e-3 * finals["r"].max().item()
     assert (out - ref.float()).abs().max().item() <= OUT_TOL
+
+
+@pytest.mark.parametrize("case", ["causal_d128_fp16", "full_d64_bf16", "window_d128_bf16", "ragged_d128_fp16",
+                                  "gqa_causal_d128_fp16", "shifted_d64_fp16"])
+def test_pipelined_kernel(cuda_device, monkeypatch, case):
+    """The software-pipelined softmax kernel (64 rows per wave, 256-row q tiles) is normally chosen
+    only for problems that fill the chip; here it is forced on small shapes, including a sequence
+    length that is no multiple of any tile, grouped kv heads and rows without a visible key."""
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    B, H, Hkv, S, D, dtype, mask_mod = {
+        "causal_d128_fp16": (1, 4, 4, 1024, 128, torch.float16, C.causal_mask),
+        "full_d64_bf16": (2, 2, 2, 768, 64, torch.bfloat16, None),
+        "window_d128_bf16": (1, 2, 2, 1024, 128, torch.bfloat16, C.make_sliding_window_mask(200)),
+        "ragged_d128_fp16": (1, 2, 2, 1000, 128, torch.float16, C.causal_mask),
+        "gqa_causal_d128_fp16": (1, 8, 2, 512, 128, torch.float16, C.causal_mask),
+        "shifted_d64_fp16": (1, 2, 2, 512, 64, torch.float16, C.causal_shifted_mask),
+    }[case]
+    print(f"case pipelined {case}", flush=True)
+    q, k, v = C.make_inputs(B, S, S, H, Hkv, D, D, dtype)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod, C.OnlineSoftmax(), Hkv=Hkv)
+    assert mod._op.tiles.template == "ae_prefill_pipe.hip"
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    lse = mod.final_rowscales["lse"].cpu()
+    dense = _dense(mask_mod, B, H, S, S) if mask_mod is not None else torch.ones(B, H, S, S, dtype=torch.bool)
+    ref, lref = R.softmax_attention(q, k, v, mask=dense)
+    visible = dense.any(-1)
+    assert (out - ref)[visible.permute(0, 2, 1)].abs().max().item() <= OUT_TOL
+    assert (lse - lref)[visible].abs().max().item() <= LSE_TOL
+    if (~visible).any():
+        assert out[~visible.permute(0, 2, 1)].abs().max().item() == 0.0
+        assert torch.isinf(lse[~visible]).all()
