@@ -100,14 +100,17 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int wg = blockIdx.x;
   const int xcd = wg & 7;
   const int slot = wg >> 3;
-  const int qt_i = slot % n_qt;
-  const int bh = (slot / n_qt) * 8 + xcd;
-  if (bh >= n_bh) return;
 #if AE_MASK_MODE == 1
-  const int qt = n_qt - 1 - qt_i;
+  // causal: q tiles differ in work by up to n_qt : 1, so ids go heaviest tile first across ALL heads
+  // (longest-job-first keeps the tail short); the heads of one XCD still meet in its L2
+  const int n_bg = (n_bh + 7) >> 3;
+  const int qt = n_qt - 1 - slot / n_bg;
+  const int bh = (slot % n_bg) * 8 + xcd;
 #else
-  const int qt = qt_i;
+  const int qt = slot % n_qt;
+  const int bh = (slot / n_qt) * 8 + xcd;
 #endif
+  if (bh >= n_bh) return;
   const int h = bh % p.heads_q;
   const int b = bh / p.heads_q;
   const int hk = h / (p.heads_q / p.heads_kv);
