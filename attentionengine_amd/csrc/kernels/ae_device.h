@@ -65,6 +65,30 @@ AE_DEV void ae_load_lds16(const void* gptr, ae_lds_u8* lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(m0v) : "memory");
 }
 
+// N (1..8) such loads behind ONE write of M0.  Every write of M0 makes the wave wait for its LDS reads
+// in flight, which costs a kernel that keeps its LDS pipe busy about 40 ns per load; a burst pays that
+// once.  Load i lands at lds_mid + (i - N/2) KiB + lane*16.  The instruction's immediate offset moves
+// the LDS address AND the global address, so the caller passes g[i] = source pointer - (i - N/2) KiB
+// (the sum is what is dereferenced).  g must have 8 entries; those from N on are ignored.
+template <int N>
+AE_DEV void ae_load_lds16_burst(const void* const* g, ae_lds_u8* lds_mid) {
+  static_assert(N >= 1 && N <= 8, "the 13-bit signed immediate offset reaches -4 KiB .. +3 KiB");
+  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)lds_mid);
+  asm volatile(
+      "s_mov_b32 m0, %8\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, off offset:(0-%9/2)*1024\n\t"
+      ".if %9 > 1\n\tglobal_load_lds_dwordx4 %1, off offset:(1-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 2\n\tglobal_load_lds_dwordx4 %2, off offset:(2-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 3\n\tglobal_load_lds_dwordx4 %3, off offset:(3-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 4\n\tglobal_load_lds_dwordx4 %4, off offset:(4-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 5\n\tglobal_load_lds_dwordx4 %5, off offset:(5-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 6\n\tglobal_load_lds_dwordx4 %6, off offset:(6-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 7\n\tglobal_load_lds_dwordx4 %7, off offset:(7-%9/2)*1024\n\t.endif"
+      :
+      : "v"(g[0]), "v"(g[1]), "v"(g[2]), "v"(g[3]), "v"(g[4]), "v"(g[5]), "v"(g[6]), "v"(g[7]), "s"(m0v), "n"(N)
+      : "memory");
+}
+
 // ---- transcendentals ------------------------------------------------------------------
 AE_DEV float ae_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 AE_DEV float ae_exp(float x) { return __builtin_amdgcn_exp2f(x * AE_LOG2E); }

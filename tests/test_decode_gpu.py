@@ -99,13 +99,18 @@ def _mla_engine(B, H, G, S, D, DV, dtype, scale, **kw):
     (3, 16, 1, 200, torch.float16),       # fewer heads than a workgroup covers, ragged KV
     (2, 64, 2, 96, torch.bfloat16),       # two latent heads
 ])
-def test_mla_decode_tl_convention(cuda_device, B, H, G, S, dtype):
+@pytest.mark.parametrize("kernel,template", [("", "ae_mla_decode_ws.hip"), ("generic", "ae_mla_decode.hip")])
+def test_mla_decode_tl_convention(cuda_device, monkeypatch, B, H, G, S, dtype, kernel, template):
+    """Both kernel templates: the wave-specialised one chosen for scaled softmax and the generic one
+    (any functor graph), forced through AE_MLA_KERNEL."""
     D, DV = 576, 512
     scale = 1 / math.sqrt(192)            # BASELINE config 5 scale
-    print(f"case mla B{B} H{H} G{G} S{S} {dtype}", flush=True)
+    print(f"case mla B{B} H{H} G{G} S{S} {dtype} kernel={kernel or 'default'}", flush=True)
+    monkeypatch.setenv("AE_MLA_KERNEL", kernel)
     q, q_pe, kv, k_pe = _mla_inputs(B, H, G, S, DV, D - DV, dtype)
     mod = _mla_engine(B, H, G, S, D, DV, dtype, scale)
     out = mod(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda())
+    assert mod.attention.template == template
     ref, lse = R.mla_decode(q[:, 0], q_pe[:, 0], kv, k_pe, scale=scale)
     assert out.shape == (B, 1, H, DV) and out.dtype == dtype
     assert (out[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL
