@@ -89,6 +89,35 @@ AE_DEV void ae_load_lds16_burst(const void* const* g, ae_lds_u8* lds_mid) {
       : "memory");
 }
 
+// The same burst for loads whose lanes all read from one wave-uniform base: address = base (SGPR pair)
+// + off[i] (unsigned 32-bit, per lane) + immediate.  No 64-bit address arithmetic and one VGPR per load.
+// The caller passes off[i] = byte offset from base - (i - N/2) KiB, which must not be negative.
+template <int N>
+AE_DEV void ae_load_lds16_burst_base(const void* base, const unsigned* off, ae_lds_u8* lds_mid) {
+  static_assert(N >= 1 && N <= 8, "the 13-bit signed immediate offset reaches -4 KiB .. +3 KiB");
+  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)lds_mid);
+  // the base must sit in scalar registers even where the compiler cannot prove it wave uniform
+  const unsigned long bv = (unsigned long)base;
+  // (readfirstlane returns a signed int: go through unsigned, or the low half sign-extends into the high)
+  const unsigned b_hi = (unsigned)__builtin_amdgcn_readfirstlane((unsigned)(bv >> 32));
+  const unsigned b_lo = (unsigned)__builtin_amdgcn_readfirstlane((unsigned)bv);
+  const unsigned long ub = ((unsigned long)b_hi << 32) | (unsigned long)b_lo;
+  asm volatile(
+      "s_mov_b32 m0, %8\n\ts_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %10 offset:(0-%9/2)*1024\n\t"
+      ".if %9 > 1\n\tglobal_load_lds_dwordx4 %1, %10 offset:(1-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 2\n\tglobal_load_lds_dwordx4 %2, %10 offset:(2-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 3\n\tglobal_load_lds_dwordx4 %3, %10 offset:(3-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 4\n\tglobal_load_lds_dwordx4 %4, %10 offset:(4-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 5\n\tglobal_load_lds_dwordx4 %5, %10 offset:(5-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 6\n\tglobal_load_lds_dwordx4 %6, %10 offset:(6-%9/2)*1024\n\t.endif\n\t"
+      ".if %9 > 7\n\tglobal_load_lds_dwordx4 %7, %10 offset:(7-%9/2)*1024\n\t.endif"
+      :
+      : "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "v"(off[4]), "v"(off[5]), "v"(off[6]), "v"(off[7]),
+        "s"(m0v), "n"(N), "s"(ub)
+      : "memory");
+}
+
 // ---- transcendentals ------------------------------------------------------------------
 AE_DEV float ae_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 AE_DEV float ae_exp(float x) { return __builtin_amdgcn_exp2f(x * AE_LOG2E); }

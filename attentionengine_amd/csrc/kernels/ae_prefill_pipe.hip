@@ -21,7 +21,7 @@
 // with `sched_barrier` fences pinning the interleaving, the exponentiation split into stages (fma,
 // exp2, pack + sum) that run in different MFMA slots so no instruction waits for the one just
 // issued, A fragments read from LDS a few MFMAs ahead of their use into a small register ring, and
-// the tile loads (HBM -> LDS direct) issued one instruction at a time from the phase-1 slots.
+// the tile loads (HBM -> LDS direct) issued as two bursts from phase-1 slots.
 // The rescale of O happens outside the hot loop (lazy running maximum: it is rare).
 //
 // Configuration ("ae_config.h"): AE_D AE_DV AE_BN(=64) AE_NWAVES AE_DTYPE_BF16 AE_MASK_MODE
@@ -63,6 +63,10 @@
 #ifndef AE_EXP_SPAN
 #define AE_EXP_SPAN (2 * AE_NKF + 8)   // MFMA slots over which the 32 exponentiation units of a tile start
 #endif
+#ifndef AE_KLOAD_SLOT
+#define AE_KLOAD_SLOT 7            // phase-1 MFMA slots after which the K and the V tile loads go out
+#define AE_VLOAD_SLOT (AE_NKF + 7)
+#endif
 #define AE_TAU 5.545177444479562f  // 8 ln 2: the running maximum is refreshed only when it moved by more
 
 static_assert(AE_BN == 64, "the pipelined kernel is written for 64-wide kv tiles");
@@ -70,6 +74,7 @@ static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
 static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
 static_assert((AE_BN * AE_KCPR) % AE_NT == 0 && (AE_BN * AE_VCPR) % AE_NT == 0, "tile / workgroup split");
 static_assert(AE_VPS2 >= 2, "work split");
+static_assert(AE_K_LOADS >= 1 && AE_K_LOADS <= 8 && AE_V_LOADS >= 1 && AE_V_LOADS <= 8, "one burst per tile and wave");
 // k-step kk of O^T += V^T P^T starts in slot 2*NKF + 2*NDB*kk; its last unit (8*kk+7) must be done
 static_assert(((7 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF, "exp units of k-step 0 finish in phase 1");
 static_assert(((31 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 6 * AE_NDB, "exp units of k-step 3 finish in time");
@@ -198,60 +203,59 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
   const ae_elem* vbase = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
 
-  // Direct HBM -> LDS tile loads with the chunk swizzles of ae_prefill.hip.  A lane's byte offset
-  // inside a tile never changes, so it is computed once; per tile only a wave-uniform base moves.
-  unsigned koff[AE_K_LOADS], voff[AE_V_LOADS];
-#pragma unroll
-  for (int i = 0; i < AE_K_LOADS; i++) {
-    const int row = (wave * AE_K_LOADS + i) * AE_K_RPI + lane / AE_KCPR;
+  // Direct HBM -> LDS tile loads with the chunk swizzles of ae_prefill.hip: wave w fills the AE_K_LOADS
+  // (AE_V_LOADS) consecutive 1 KiB blocks starting at block w*AE_K_LOADS of a K (V) tile.  A lane's byte
+  // offset inside a tile never changes, so it is computed once; per tile only a wave-uniform base moves.
+  // A tile's loads go out as one burst behind a single write of M0 (see ae_load_lds16_burst; the offsets
+  // carry the compensation for its immediate offsets).
+  // (bases are passed 4 KiB low and the offsets 4 KiB high, so that the compensated offsets stay >= 0)
+  auto k_lane_off = [&](int i, int last_row) -> unsigned {
+    int row = (wave * AE_K_LOADS + i) * AE_K_RPI + lane / AE_KCPR;
     const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
-    koff[i] = (unsigned)(row * (int)p.k_stride_s + c * 8) * 2u;
-  }
-#pragma unroll
-  for (int i = 0; i < AE_V_LOADS; i++) {
-    const int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
+    row = row < last_row ? row : last_row;
+    return (unsigned)((row * (int)p.k_stride_s + c * 8) * 2 + 4096 - (i - AE_K_LOADS / 2) * 1024);
+  };
+  auto v_lane_off = [&](int i, int last_row) -> unsigned {
+    int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
     const int cp = lane % AE_VCPR;
     const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
-    voff[i] = (unsigned)(row * (int)p.v_stride_s + c * 8) * 2u;
-  }
-  auto load_k_part = [&](int j, int stage, int i) {
-    ae_lds_byte* ks = lds + stage * AE_K_BYTES;
-    const char* g = (const char*)kbase + (int64_t)j * AE_BN * p.k_stride_s * 2;
-    const int blk = wave * AE_K_LOADS + i;
-    unsigned off = koff[i];
-#if !AE_EVEN_KV
-    if (j * AE_BN + AE_BN > p.seqlen_kv) {   // rows past the end re-read the last row (masked later)
-      const int row = blk * AE_K_RPI + lane / AE_KCPR;
-      const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
-      const int last = p.seqlen_kv - 1 - j * AE_BN;
-      off = (unsigned)((row < last ? row : last) * (int)p.k_stride_s + c * 8) * 2u;
-    }
-#endif
-    ae_load_lds16(g + off, ks + blk * 1024);
+    row = row < last_row ? row : last_row;
+    return (unsigned)((row * (int)p.v_stride_s + c * 8) * 2 + 4096 - (i - AE_V_LOADS / 2) * 1024);
   };
-  auto load_k = [&](int j, int stage) {
+  unsigned koff[AE_K_LOADS], voff[AE_V_LOADS];
 #pragma unroll
-    for (int i = 0; i < AE_K_LOADS; i++) load_k_part(j, stage, i);
-  };
-  auto load_v_part = [&](int j, int stage, int i) {
-    ae_lds_byte* vs = lds + 2 * AE_K_BYTES + stage * AE_V_BYTES;
-    const char* g = (const char*)vbase + (int64_t)j * AE_BN * p.v_stride_s * 2;
-    const int blk = wave * AE_V_LOADS + i;
-    unsigned off = voff[i];
+  for (int i = 0; i < AE_K_LOADS; i++) koff[i] = k_lane_off(i, AE_BN);
+#pragma unroll
+  for (int i = 0; i < AE_V_LOADS; i++) voff[i] = v_lane_off(i, AE_BN);
+  auto load_k = [&](int j, int stage) {
+    const char* g = (const char*)kbase + (int64_t)j * AE_BN * p.k_stride_s * 2 - 4096;
+    unsigned gp[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int ii = i < AE_K_LOADS ? i : 0;
+      unsigned off = koff[ii];
 #if !AE_EVEN_KV
-    if (j * AE_BN + AE_BN > p.seqlen_kv) {
-      const int row = blk * AE_V_RPI + lane / AE_VCPR;
-      const int cp = lane % AE_VCPR;
-      const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
-      const int last = p.seqlen_kv - 1 - j * AE_BN;
-      off = (unsigned)((row < last ? row : last) * (int)p.v_stride_s + c * 8) * 2u;
-    }
+      // rows past the end re-read the last row (masked later)
+      if (j * AE_BN + AE_BN > p.seqlen_kv) off = k_lane_off(ii, p.seqlen_kv - 1 - j * AE_BN);
 #endif
-    ae_load_lds16(g + off, vs + blk * 1024);
+      gp[i] = off;
+    }
+    ae_load_lds16_burst_base<AE_K_LOADS>(g, gp, lds + stage * AE_K_BYTES + (wave * AE_K_LOADS + AE_K_LOADS / 2) * 1024);
   };
   auto load_v = [&](int j, int stage) {
+    const char* g = (const char*)vbase + (int64_t)j * AE_BN * p.v_stride_s * 2 - 4096;
+    unsigned gp[8];
 #pragma unroll
-    for (int i = 0; i < AE_V_LOADS; i++) load_v_part(j, stage, i);
+    for (int i = 0; i < 8; i++) {
+      const int ii = i < AE_V_LOADS ? i : 0;
+      unsigned off = voff[ii];
+#if !AE_EVEN_KV
+      if (j * AE_BN + AE_BN > p.seqlen_kv) off = v_lane_off(ii, p.seqlen_kv - 1 - j * AE_BN);
+#endif
+      gp[i] = off;
+    }
+    ae_load_lds16_burst_base<AE_V_LOADS>(
+        g, gp, lds + 2 * AE_K_BYTES + stage * AE_V_BYTES + (wave * AE_V_LOADS + AE_V_LOADS / 2) * 1024);
   };
 
   // ---- state ------------------------------------------------------------------------------
@@ -467,9 +471,8 @@ void ae_prefill_kernel(const ae_attn_params p) {
     // compiler's wait-count insertion would otherwise wait for after this iteration's tile loads
     // have been issued, i.e. with a vmcnt(0) that serialises them.
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);
-    // The tile loads of this iteration, K(j2) and V(j1), are issued one instruction at a time from
-    // the phase-1 slots below (a burst here costs ~600 cycles of issue that nothing hides).  When
-    // there is no tile j2 the K stage is refilled with the last tile, which nobody reads.
+    // The tile loads of this iteration, K(j2) and V(j1), are issued as two bursts from phase-1 slots
+    // below.  When there is no tile j2 the K stage is refilled with the last tile, which nobody reads.
     const int j2l = j2 < j_end ? j2 : j_end - 1;
     // fragment stream of this iteration: K fragments 0..NKF-1 (if HN) then V fragments
     constexpr int NF1 = HN ? AE_NKF : 0;
@@ -496,15 +499,8 @@ void ae_prefill_kernel(const ae_attn_params p) {
           }
           sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], c);
           exp_slot(2 * f + qb);
-          {
-            constexpr int NL = AE_K_LOADS + AE_V_LOADS, EVERY = (2 * AE_NKF) / NL;
-            const int g = 2 * f + qb;
-            if (g % EVERY == EVERY - 1 && g / EVERY < NL) {
-              const int i = g / EVERY;
-              if (i < AE_K_LOADS) load_k_part(j2l, n & 1, i);
-              else load_v_part(j1, (n + 1) & 1, i - AE_K_LOADS);
-            }
-          }
+          if (2 * f + qb == AE_KLOAD_SLOT) load_k(j2l, n & 1);
+          if (2 * f + qb == AE_VLOAD_SLOT) load_v(j1, (n + 1) & 1);
           AE_SB();
         }
       }
