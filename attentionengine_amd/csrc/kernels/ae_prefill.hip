@@ -65,6 +65,7 @@ static_assert(AE_DV % 32 == 0, "value head dim must be a multiple of 32");
 static_assert(AE_BN % 32 == 0, "kv tile must be a multiple of 32");
 static_assert((AE_BN * AE_KCPR) % AE_NT == 0, "K tile must split evenly over the workgroup");
 static_assert((AE_BN * AE_VCPR) % AE_NT == 0, "V tile must split evenly over the workgroup");
+static_assert(AE_K_LOADS >= 1 && AE_K_LOADS <= 8 && AE_V_LOADS >= 1 && AE_V_LOADS <= 8, "one burst per tile and wave");
 static_assert(AE_KCPR == 8 || AE_KCPR == 16, "swizzle is written for 128- or 256-byte K rows");
 static_assert(AE_VCPR == 8 || AE_VCPR == 16, "swizzle is written for 128- or 256-byte V rows");
 
@@ -169,38 +170,48 @@ void ae_prefill_kernel(const ae_attn_params p) {
 
   // Direct HBM -> LDS tile load.  Wave w, instruction i covers rows (w*LOADS + i)*RPI ...+RPI-1;
   // lane L lands in LDS chunk c' = L % CPR of row (L / CPR) and fetches the permuted global chunk.
+  // A lane's byte offset inside a tile never changes, so it is computed once; per tile only a
+  // wave-uniform base moves.  The K loads and the V loads of a wave each go out as one burst behind a
+  // single write of M0 (see ae_load_lds16_burst_base: bases are passed 4 KiB low and the offsets 4 KiB
+  // high, so that the offsets, which carry the compensation for the immediate offsets, stay >= 0).
+  auto k_lane_off = [&](int i, int last_row) -> unsigned {
+    int row = (wave * AE_K_LOADS + i) * AE_K_RPI + lane / AE_KCPR;
+    const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
+    row = row < last_row ? row : last_row;
+    return (unsigned)((row * (int)p.k_stride_s + c * 8) * 2 + 4096 - (i - AE_K_LOADS / 2) * 1024);
+  };
+  auto v_lane_off = [&](int i, int last_row) -> unsigned {
+    int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
+    const int cp = lane % AE_VCPR;
+    const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
+    row = row < last_row ? row : last_row;
+    return (unsigned)((row * (int)p.v_stride_s + c * 8) * 2 + 4096 - (i - AE_V_LOADS / 2) * 1024);
+  };
+  unsigned koff[AE_K_LOADS], voff[AE_V_LOADS];
+#pragma unroll
+  for (int i = 0; i < AE_K_LOADS; i++) koff[i] = k_lane_off(i, AE_BN);
+#pragma unroll
+  for (int i = 0; i < AE_V_LOADS; i++) voff[i] = v_lane_off(i, AE_BN);
   auto load_tile = [&](int j, int stage) {
-    const int kv0 = j * AE_BN;
     ae_lds_byte* ks = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* vs = ks + AE_K_BYTES;
+    const char* gk = (const char*)kbase + (int64_t)j * AE_BN * p.k_stride_s * 2 - 4096;
+    const char* gv = (const char*)vbase + (int64_t)j * AE_BN * p.v_stride_s * 2 - 4096;
+    unsigned ko[8], vo[8];
 #pragma unroll
-    for (int i = 0; i < AE_K_LOADS; i++) {
-      const int blk = wave * AE_K_LOADS + i;                 // wave-uniform 1 KiB block of the tile
-      const int row = blk * AE_K_RPI + lane / AE_KCPR;
-      const int cp = lane % AE_KCPR;                          // LDS chunk
-      const int c = cp ^ (row & (AE_KCPR - 1));               // global chunk
-      int kv = kv0 + row;
+    for (int i = 0; i < 8; i++) {
+      ko[i] = koff[i < AE_K_LOADS ? i : 0];
+      vo[i] = voff[i < AE_V_LOADS ? i : 0];
 #if !AE_EVEN_KV
-      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
+      // rows past the end re-read the last row (masked later)
+      if (j * AE_BN + AE_BN > p.seqlen_kv) {
+        ko[i] = k_lane_off(i < AE_K_LOADS ? i : 0, p.seqlen_kv - 1 - j * AE_BN);
+        vo[i] = v_lane_off(i < AE_V_LOADS ? i : 0, p.seqlen_kv - 1 - j * AE_BN);
+      }
 #endif
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(kbase + (int64_t)kv * p.k_stride_s + c * 8),
-          (__attribute__((address_space(3))) void*)(ks + blk * 1024), 16, 0, 0);
     }
-#pragma unroll
-    for (int i = 0; i < AE_V_LOADS; i++) {
-      const int blk = wave * AE_V_LOADS + i;
-      const int row = blk * AE_V_RPI + lane / AE_VCPR;
-      const int cp = lane % AE_VCPR;
-      const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
-      int kv = kv0 + row;
-#if !AE_EVEN_KV
-      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
-#endif
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(vbase + (int64_t)kv * p.v_stride_s + c * 8),
-          (__attribute__((address_space(3))) void*)(vs + blk * 1024), 16, 0, 0);
-    }
+    ae_load_lds16_burst_base<AE_K_LOADS>(gk, ko, ks + (wave * AE_K_LOADS + AE_K_LOADS / 2) * 1024);
+    ae_load_lds16_burst_base<AE_V_LOADS>(gv, vo, vs + (wave * AE_V_LOADS + AE_V_LOADS / 2) * 1024);
   };
   // next tile index >= j that has work (block table) or j itself
   auto next_tile = [&](int j) {
