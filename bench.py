@@ -46,10 +46,10 @@ WORKLOADS = {
 # that a 256 MiB copy kernel calibrates the counter: FETCH_SIZE reads half the bytes moved, factor
 # 2.0; WRITE_SIZE factor 1.0).  Fetched + written.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "c2_causal": 428.7e6 + 68.2e6,       # algorithmic Q+K+V+O+lse: 269.5e6 (K/V are fetched twice: the
+    "c2_causal": 423.5e6 + 68.2e6,       # algorithmic Q+K+V+O+lse: 269.5e6 (K/V are fetched twice: the
                                          # heaviest-first causal order spreads a head's q tiles in time)
     "c4_gqa_decode": 2147.9e6 + 4.2e6,   # algorithmic K+V: 2147.5e6 (fp32 partials written: 4.2e6)
-    "c5_mla_decode": 623.0e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
+    "c5_mla_decode": 623.2e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
 }
 
 
