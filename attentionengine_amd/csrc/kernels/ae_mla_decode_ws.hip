@@ -9,19 +9,21 @@
 // Why a second kernel: in ae_mla_decode.hip every one of 8 waves reads the whole KV tile from LDS for
 // both products (416 KiB of LDS reads per 32-token tile and workgroup) and the two value halves of a
 // head block compute the same scores; LDS bandwidth bounds it at ~0.21 ms for B128 H128 S4096.  Here
-// the 8 waves of a workgroup (64 query heads of one (batch, kv head, split)) have different jobs:
-//   * waves 0-3 ("score waves", 16 heads each): S^T[kv,head] = K Q^T with v_mfma_f32_16x16x32 (Q^T in
-//     registers for the whole kernel, K fragments from LDS), lazy online softmax, P^T written to LDS as
-//     the B operand of the second product, per-head rescale factors next to it;
-//   * waves 4-7 ("value waves", a quarter of the value columns each, all 64 heads): O^T[dv,head] += V^T P^T
-//     with v_mfma_f32_32x32x16, V^T fragments read from the SAME LDS rows through ds_read_b64_tr_b16,
-//     every fragment feeding both 32-head blocks.
-// Wave i runs on SIMD i % 4, so every SIMD hosts one wave of each kind and their MFMA work (576 + 512
-// matrix-pipe cycles per tile) interleaves.  The score waves run one tile ahead of the value waves: one
-// workgroup barrier per tile hands P over.  Scores are computed once: 196 KiB of LDS reads per tile
-// instead of 416.  KV tiles go HBM -> LDS directly (16 B per lane, chunk-swizzled as in
-// ae_mla_decode.hip), AE_NSTAGE tiles deep; a trip ends by waiting until only the newest tile request
-// is outstanding.
+// the waves of a workgroup (64 query heads of one (batch, kv head, split)) have different jobs:
+//   * 2 "score waves" (32 heads each): S^T[kv,head] = K Q^T with v_mfma_f32_32x32x16 (Q^T in registers for
+//     the whole kernel, K fragments from LDS, each feeding a 32x32 block: with 16 heads per wave the four
+//     waves' fragment reads, 144 KiB per tile, took 2.6x the time of their MFMAs), lazy online softmax,
+//     P^T written to LDS as the B operand of the second product, per-head rescale factors next to it;
+//   * 4 "value waves" (a quarter of the value columns each, all 64 heads): O^T[dv,head] += V^T P^T with
+//     v_mfma_f32_32x32x16, V^T fragments read from the SAME LDS rows through ds_read_b64_tr_b16, every
+//     fragment feeding both 32-head blocks.
+// Wave i runs on SIMD i % 4.  The workgroup is launched with 8 waves: waves 0, 1 are the score waves
+// (SIMD 0, 1: 1152 matrix-pipe cycles per tile each), waves 2, 3, 6, 7 the value waves (two each on SIMD
+// 2, 3: 2 x 512 cycles), waves 4, 5 leave at once - so the four SIMDs carry about the same MFMA work.
+// The score waves run one tile ahead of the value waves: one workgroup barrier per tile hands P over.
+// Scores are computed once: 124 KiB of LDS reads per tile instead of 416.  KV tiles go HBM -> LDS
+// directly (16 B per lane, chunk-swizzled as in ae_mla_decode.hip), AE_NSTAGE tiles deep; a trip ends by
+// waiting until only the newest tile request is outstanding.
 //
 // Configuration ("ae_config.h"): AE_D1 AE_D2 AE_DV AE_DTYPE_BF16 AE_N_ROWSCALES AE_NSPLIT
 // AE_COMBINE_THREADS, plus AE_SM_SCALE (the constant c > 0) and AE_SM_M / AE_SM_R (names of the
@@ -39,7 +41,8 @@
 #define AE_NT (AE_NWAVES * 64)
 #define AE_HEADS_PER_WG 64
 #define AE_BN 32                          // kv rows per tile
-#define AE_NKS (AE_D / 32)                // 32-deep k-steps of S^T = K Q^T
+#define AE_NKS (AE_D / 16)                // 16-deep k-steps of S^T = K Q^T
+#define AE_NLOADERS 4                     // the value waves also request the KV tiles
 #define AE_DVW (AE_DV / 4)                // value columns of one value wave
 #define AE_NDB (AE_DVW / 32)              // 32-wide dv blocks of a value wave
 #define AE_NO (AE_NDB * 16)               // output elements per lane and head block
@@ -48,26 +51,29 @@
 #define AE_CPR (AE_D / 8)                 // 16-byte chunks per K row
 #define AE_CPR1 (AE_D1 / 8)
 #define AE_BLOCKS ((AE_BN * AE_CPR) / 64) // 1 KiB blocks per tile
-#define AE_LOADS ((AE_BLOCKS + AE_NWAVES - 1) / AE_NWAVES)
+#define AE_LOADS ((AE_BLOCKS + AE_NLOADERS - 1) / AE_NLOADERS)
+#define AE_L1 ((AE_LOADS + 1) / 2)        // a wave's loads of one tile go out as two bursts
+#define AE_L2 (AE_LOADS - AE_L1)
 #ifndef AE_NSTAGE
 #define AE_NSTAGE 4
 #endif
 #define AE_PSTR 80                        // LDS pitch of one head's P row (32 kv * 2 B, padded against bank conflicts)
 #define AE_P_BYTES (AE_HEADS_PER_WG * AE_PSTR)
-#define AE_X_BYTES (AE_HEADS_PER_WG * 4 + 16)   // per-head rescale factors + one flag word per score wave
+#define AE_X_BYTES (AE_HEADS_PER_WG * 4 + 16)   // per-head rescale factors + one flag word per score wave (2 used)
 #define AE_TAU2 8.0f                      // the running maximum (log2 units) is refreshed only when it moved by more
 #define AE_SWZ(r) ((((r) >> 1) & 3) * 2 + (((r) >> 3) & 1))
 #define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 #ifndef AE_AHEAD
-#define AE_AHEAD 6
+#define AE_AHEAD 4
 #endif
 #define AE_RING (AE_AHEAD + 1)
 
 static_assert(AE_D1 % 32 == 0 && AE_D2 % 32 == 0, "latent / rope dims must be multiples of 32");
+static_assert(AE_NKS % 2 == 0, "two accumulation chains over the k-steps");
 static_assert(AE_DV % 128 == 0 && AE_DV <= AE_D1, "V must be a prefix of the latent part, four 32-column blocks wide");
 static_assert(AE_CPR % 8 == 0 && AE_CPR1 % 8 == 0, "chunk groups of eight must not straddle the two K tensors");
 static_assert((AE_BN * AE_CPR) % 64 == 0, "tile must be a whole number of 1 KiB blocks");
-static_assert(AE_LOADS <= 8 && AE_BLOCKS >= AE_LOADS, "one burst of at most eight loads per wave and tile");
+static_assert(AE_L1 <= 8 && AE_L2 >= 1 && AE_BLOCKS >= AE_LOADS, "two bursts of at most eight loads per wave and tile");
 static_assert(AE_NSTAGE >= 3, "a tile is multiplied by K one trip before it is multiplied as V");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
@@ -85,7 +91,8 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const bool score_wave = wave < 4;
+  const bool score_wave = wave < 2;
+  if (wave == 4 || wave == 5) return;      // placeholders: they only steer the value waves onto SIMD 2, 3
 
   // ---- which (head tile, split, kv head, batch): 1-D grid, ids 8 apart share their KV range ---------
   const int group = p.heads_q / p.heads_kv;
@@ -106,32 +113,144 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   kv_end = kv_end < p.seqlen_kv ? kv_end : p.seqlen_kv;
   const int n_tiles = kv_end > kv_begin ? (kv_end - kv_begin + AE_BN - 1) / AE_BN : 0;
 
-  // Direct HBM -> LDS tile load: wave w fills AE_LOADS consecutive 1 KiB blocks of the tile, starting at
-  // block min(w*AE_LOADS, AE_BLOCKS-AE_LOADS) (the last waves overlap, so every wave issues the same
-  // number of loads); LDS chunk c' of row r receives global chunk c' ^ f(r).  Which row and chunk a lane
-  // fetches never changes, so its source pointer inside tile 0 and its row stride are computed once; per
-  // tile only kv0 * stride is added.  All loads of a wave go out as one burst behind a single write of
-  // M0 (see ae_load_lds16_burst; the pointers carry the compensation for its immediate offsets).  Tiles
-  // past the end re-read the last tile, so every trip issues the same number of loads; rows past
-  // seqlen_kv re-read the last row.
-  const int blk0 = wave * AE_LOADS < AE_BLOCKS - AE_LOADS ? wave * AE_LOADS : AE_BLOCKS - AE_LOADS;
-  const char* ld_base[AE_LOADS];
-  int ld_stride[AE_LOADS];      // bytes per kv row of the tensor this lane reads from
-  int ld_row[AE_LOADS];
+  if (score_wave) {
+    // =============================== score wave: 32 heads ==============================================
+    const int l32s = lane & 31;
+    const int hfs = lane >> 5;
+    const int head_in_group = ht * AE_HEADS_PER_WG + wave * 32 + l32s;
+    const bool head_ok = head_in_group < group;
+    const int hq = hk * group + (head_ok ? head_in_group : 0);
+    // Q^T fragments: B operand (n = head = lane%32, k = d = 16*ks + 8*(lane/32) + j)
+    const ae_elem* q1 = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)hq * p.q_stride_h;
+    const ae_elem* q2 = (const ae_elem*)p.q2 + (int64_t)b * p.q2_stride_b + (int64_t)hq * p.q2_stride_h;
+    ae_elem8 qf[AE_NKS];
+#pragma unroll
+    for (int ks = 0; ks < AE_D1 / 16; ks++) qf[ks] = *(const ae_elem8*)(q1 + ks * 16 + hfs * 8);
+#pragma unroll
+    for (int ks = 0; ks < AE_D2 / 16; ks++) qf[AE_D1 / 16 + ks] = *(const ae_elem8*)(q2 + ks * 16 + hfs * 8);
+
+    ae_rowstate st;
+    ae_rowstate_init(st);
+    float m2 = st.AE_SM_M * AE_LOG2E;   // running reference, log2 units
+    float r_run = st.AE_SM_R;           // this lane's part of the row sum (a row lives in lanes l, l^32)
+
+    // (the value waves request the tiles: this wave's registers are taken by Q^T)
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // Q has landed
+    __syncthreads();                           // tile 0 has landed
+
+#ifdef AE_SCORE_PRIO
+    __builtin_amdgcn_s_setprio(AE_SCORE_PRIO);
+#endif
+    // K fragment of k-step ks: row lane%32, global chunk 2*ks + lane/32
+    const int k_row_off = l32s * AE_KSTR;
+    const int k_sw = AE_SWZ(l32s);
+    for (int t = -1; t < n_tiles; t++) {
+      const int tn = t + 1;                      // the tile this wave multiplies by Q now
+      if (tn < n_tiles) {
+        const ae_lds_byte* kt = lds + (tn % AE_NSTAGE) * AE_STAGE_BYTES + k_row_off;
+        ae_f32x16 sacc[2];   // even / odd k-steps: two independent MFMA chains
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) sacc[c][r] = 0.f;
+        // read AE_AHEAD fragments before the MFMA that uses them (the compiler on its own keeps one read
+        // in flight, which leaves the LDS latency exposed)
+        auto read_kfrag = [&](int ks) -> ae_elem8 {
+          return *(const __attribute__((address_space(3))) ae_elem8*)(kt + (((2 * ks + hfs) ^ k_sw) << 4));
+        };
+        ae_elem8 ring[AE_RING];
+#pragma unroll
+        for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < AE_NKS; f++) {
+          if (f + AE_AHEAD < AE_NKS) ring[(f + AE_AHEAD) % AE_RING] = read_kfrag(f + AE_AHEAD);
+          sacc[f & 1] = ae_mfma32(ring[f % AE_RING], qf[f], sacc[f & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        // lane owns head lane%32 and kv rows 8*(e/4) + 4*(lane/32) + e%4 of the tile
+        float x[16];
+        const int kvb = kv_begin + tn * AE_BN + 4 * hfs;
+        const bool tail = kv_begin + tn * AE_BN + AE_BN > kv_end;
+        float mx = AE_NEG_INF;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          x[e] = (sacc[0][e] + sacc[1][e]) * (AE_SM_SCALE * AE_LOG2E);
+          if (tail) x[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
+          mx = __builtin_fmaxf(mx, x[e]);
+        }
+        {
+          float hi;
+          const float lo = ae_swap32_lo_hi(mx, hi);
+          mx = __builtin_fmaxf(lo, hi);
+        }
+        const bool need = (mx - m2) > AE_TAU2;
+        const float mn = need ? mx : m2;
+        const float osc = need ? ae_exp2(m2 - mn) : 1.0f;
+        m2 = mn;
+        float rs = 0.f;
+        ae_lds_byte* prow = pbuf + (tn & 1) * AE_P_BYTES + (wave * 32 + l32s) * AE_PSTR + 8 * hfs;
+#pragma unroll
+        for (int rb = 0; rb < 4; rb++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const float pv = ae_exp2(x[4 * rb + i] - mn);
+            rs += pv;
+            w[i] = (ae_elem)pv;
+          }
+          *(__attribute__((address_space(3))) ae_elem4*)(prow + 16 * rb) = w;
+        }
+        r_run = r_run * osc + rs;
+        ae_lds_byte* xb = xbuf + (tn & 1) * AE_X_BYTES;
+        if (hfs == 0) ((ae_lds_f32*)xb)[wave * 32 + l32s] = osc;
+        const bool any = __builtin_amdgcn_ballot_w64(need) != 0;
+        if (lane == 0) ((ae_lds_i32*)(xb + AE_HEADS_PER_WG * 4))[wave] = any ? 1 : 0;
+      }
+      __syncthreads();                           // end of the trip: P is handed over, tile tn + 1 has landed
+    }
+    // final row state for the value waves
+    {
+      float hi;
+      const float lo = ae_swap32_lo_hi(r_run, hi);
+      if (hfs == 0) {
+        fin[(wave * 32 + l32s) * 2] = m2 * AE_LN2;
+        fin[(wave * 32 + l32s) * 2 + 1] = lo + hi;
+      }
+    }
+    __syncthreads();
+    return;
+  }
+
+  // ================================= value wave: AE_DVW value columns, 64 heads ========================
+  const int l32 = lane & 31;
+  const int hf = lane >> 5;
+  const int dvw = wave < 4 ? wave - 2 : wave - 4;   // waves 2, 3, 6, 7
+  // Direct HBM -> LDS tile load, by the four value waves: wave w fills AE_LOADS consecutive 1 KiB blocks of
+  // the tile, starting at block min(w*AE_LOADS, AE_BLOCKS-AE_LOADS) (the last wave overlaps its neighbour, so
+  // every wave issues the same number of loads); LDS chunk c' of row r receives global chunk c' ^ f(r).
+  // Which row and chunk a lane fetches never changes, so its source pointer inside the split's first tile
+  // is computed once; per tile only tile * 32 rows * stride is added.  The loads of a wave go out as two
+  // bursts, each behind a single write of M0 (see ae_load_lds16_burst; the pointers carry the
+  // compensation for its immediate offsets).  Tiles past the end re-read the last tile, so every trip
+  // issues the same number of loads; rows past seqlen_kv re-read the last row.
+  const int blk0 = dvw * AE_LOADS < AE_BLOCKS - AE_LOADS ? dvw * AE_LOADS : AE_BLOCKS - AE_LOADS;
+  const char* ld_ptr[AE_LOADS];   // this lane's source of load i in the first tile of the split
+  unsigned ld_rope = 0;           // bit i: load i reads from the rope tensor (k2), else from the latent (k1)
+  const unsigned stride1 = (unsigned)p.k_stride_s * 2, stride2 = (unsigned)p.k2_stride_s * 2;   // bytes per kv row
 #pragma unroll
   for (int i = 0; i < AE_LOADS; i++) {
     const int sidx = (blk0 + i) * 64 + lane;
     const int row = sidx / AE_CPR, cp = sidx % AE_CPR;
     const int c = cp ^ AE_SWZ(row);
-    ld_row[i] = row;
     if (c < AE_CPR1) {
-      ld_base[i] = (const char*)(k1 + c * 8);
-      ld_stride[i] = (int)p.k_stride_s * 2;
+      ld_ptr[i] = (const char*)(k1 + c * 8) + (int64_t)(kv_begin + row) * stride1;
     } else {
-      ld_base[i] = (const char*)(k2 + (c - AE_CPR1) * 8);
-      ld_stride[i] = (int)p.k2_stride_s * 2;
+      ld_ptr[i] = (const char*)(k2 + (c - AE_CPR1) * 8) + (int64_t)(kv_begin + row) * stride2;
+      ld_rope |= 1u << i;
     }
-    ld_base[i] -= (i - AE_LOADS / 2) * 1024;
+    // immediate offset of load i inside its burst
+    ld_ptr[i] -= i < AE_L1 ? (i - AE_L1 / 2) * 1024 : (i - AE_L1 - AE_L2 / 2) * 1024;
   }
   auto load_tile = [&](int t) {
     int tt = t < n_tiles ? t : n_tiles - 1;
@@ -139,15 +258,21 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     const int kv0 = kv_begin + tt * AE_BN;
     ae_lds_byte* dst = lds + (t % AE_NSTAGE) * AE_STAGE_BYTES;
     const bool ragged = kv0 + AE_BN > p.seqlen_kv;     // wave-uniform
-    const void* g[8];
+    const void* g[16];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const int j = i < AE_LOADS ? i : 0;
-      int kv = kv0 + ld_row[j];
-      if (ragged) kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
-      g[i] = ld_base[j] + (int64_t)kv * ld_stride[j];
+    for (int i = 0; i < 16; i++) {
+      const int j = i < 8 ? (i < AE_L1 ? i : 0) : (i - 8 < AE_L2 ? AE_L1 + i - 8 : AE_L1);
+      const unsigned stride = ((ld_rope >> j) & 1u) ? stride2 : stride1;
+      g[i] = ld_ptr[j] + (uint64_t)((unsigned)(tt * AE_BN) * (uint64_t)stride);
+      if (__builtin_expect(ragged, 0)) {                      // rows past the end re-read the last row
+        const int row = ((blk0 + j) * 64 + lane) / AE_CPR;
+        int over = kv0 + row - (p.seqlen_kv - 1);
+        over = over > 0 ? over : 0;
+        g[i] = (const char*)g[i] - (uint64_t)((unsigned)over * (uint64_t)stride);
+      }
     }
-    ae_load_lds16_burst<AE_LOADS>(g, dst + (blk0 + AE_LOADS / 2) * 1024);
+    ae_load_lds16_burst<AE_L1>(g, dst + (blk0 + AE_L1 / 2) * 1024);
+    ae_load_lds16_burst<AE_L2>(g + 8, dst + (blk0 + AE_L1 + AE_L2 / 2) * 1024);
   };
   // end of a trip: tile t+2 has landed when only the newest request is outstanding; after the barrier
   // everyone is done with tile t, whose stage takes the next request
@@ -157,116 +282,6 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     load_tile(t + AE_NSTAGE);
   };
 
-  if (score_wave) {
-    // =============================== score wave: 16 heads ==============================================
-    const int l16 = lane & 15;
-    const int g4 = lane >> 4;
-    const int head_in_group = ht * AE_HEADS_PER_WG + wave * 16 + l16;
-    const bool head_ok = head_in_group < group;
-    const int hq = hk * group + (head_ok ? head_in_group : 0);
-    // Q^T fragments: B operand (n = head = l16, k = d = 32*ks + 8*g4 + j)
-    const ae_elem* q1 = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)hq * p.q_stride_h;
-    const ae_elem* q2 = (const ae_elem*)p.q2 + (int64_t)b * p.q2_stride_b + (int64_t)hq * p.q2_stride_h;
-    ae_elem8 qf[AE_NKS];
-#pragma unroll
-    for (int ks = 0; ks < AE_D1 / 32; ks++) qf[ks] = *(const ae_elem8*)(q1 + ks * 32 + g4 * 8);
-#pragma unroll
-    for (int ks = 0; ks < AE_D2 / 32; ks++) qf[AE_D1 / 32 + ks] = *(const ae_elem8*)(q2 + ks * 32 + g4 * 8);
-
-    ae_rowstate st;
-    ae_rowstate_init(st);
-    float m2 = st.AE_SM_M * AE_LOG2E;   // running reference, log2 units
-    float r_run = st.AE_SM_R;           // this lane's part of the row sum (a row lives in 4 lanes)
-
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // Q has landed: from here on only tile loads are in flight
-#pragma unroll
-    for (int t = 0; t < AE_NSTAGE - 1; t++) load_tile(t);
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT((AE_NSTAGE - 2) * AE_LOADS));   // tile 0
-    __syncthreads();
-
-#ifdef AE_SCORE_PRIO
-    __builtin_amdgcn_s_setprio(AE_SCORE_PRIO);
-#endif
-    // K fragment (k-step ks, kv block rb): row 16*rb + l16, global chunk 4*ks + g4
-    const int k_row_off = l16 * AE_KSTR;
-    const int k_sw = AE_SWZ(l16);                // rows 16*rb + l16: same low bits
-    for (int t = -1; t < n_tiles; t++) {
-      const int tn = t + 1;                      // the tile this wave multiplies by Q now
-      if (tn < n_tiles) {
-        const ae_lds_byte* kt = lds + (tn % AE_NSTAGE) * AE_STAGE_BYTES + k_row_off;
-        ae_f32x4 sacc[4];    // [k-step parity][kv block]: four independent MFMA chains
-#pragma unroll
-        for (int rb = 0; rb < 4; rb++) sacc[rb] = (ae_f32x4){0.f, 0.f, 0.f, 0.f};
-        // fragment f = (k-step f/2, kv block f%2), read AE_AHEAD fragments before the MFMA that uses it
-        // (the compiler on its own keeps one read in flight, which leaves the LDS latency exposed)
-        auto read_kfrag = [&](int f) -> ae_elem8 {
-          return *(const __attribute__((address_space(3))) ae_elem8*)(
-              kt + (f & 1) * 16 * AE_KSTR + (((4 * (f >> 1) + g4) ^ k_sw) << 4));
-        };
-        ae_elem8 ring[AE_RING];
-#pragma unroll
-        for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int f = 0; f < 2 * AE_NKS; f++) {
-          if (f + AE_AHEAD < 2 * AE_NKS) ring[(f + AE_AHEAD) % AE_RING] = read_kfrag(f + AE_AHEAD);
-          sacc[f & 3] = ae_mfma16(ring[f % AE_RING], qf[f >> 1], sacc[f & 3]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        // lane owns head l16 and kv rows 16*rb + 4*g4 + r of the tile
-        float x[8];
-        const int kvb = kv_begin + tn * AE_BN + 4 * g4;
-        const bool tail = kv_begin + tn * AE_BN + AE_BN > kv_end;
-        float mx = AE_NEG_INF;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-          x[e] = (sacc[e >> 2][e & 3] + sacc[2 + (e >> 2)][e & 3]) * (AE_SM_SCALE * AE_LOG2E);
-          if (tail) x[e] = (kvb + 16 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
-          mx = __builtin_fmaxf(mx, x[e]);
-        }
-        mx = ae_group_max(mx);
-        const bool need = (mx - m2) > AE_TAU2;
-        const float mn = need ? mx : m2;
-        const float osc = need ? ae_exp2(m2 - mn) : 1.0f;
-        m2 = mn;
-        float rs = 0.f;
-        ae_lds_byte* prow = pbuf + (tn & 1) * AE_P_BYTES + (wave * 16 + l16) * AE_PSTR + 8 * g4;
-#pragma unroll
-        for (int rb = 0; rb < 2; rb++) {
-          ae_elem4 w;
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const float pv = ae_exp2(x[4 * rb + i] - mn);
-            rs += pv;
-            w[i] = (ae_elem)pv;
-          }
-          *(__attribute__((address_space(3))) ae_elem4*)(prow + 32 * rb) = w;
-        }
-        r_run = r_run * osc + rs;
-        ae_lds_byte* xb = xbuf + (tn & 1) * AE_X_BYTES;
-        if (g4 == 0) ((ae_lds_f32*)xb)[wave * 16 + l16] = osc;
-        const bool any = __builtin_amdgcn_ballot_w64(need) != 0;
-        if (lane == 0) ((ae_lds_i32*)(xb + AE_HEADS_PER_WG * 4))[wave] = any ? 1 : 0;
-      }
-      end_trip(t);
-    }
-    // final row state for the value waves
-    {
-      const float r_tot = ae_group_sum(r_run);
-      if (g4 == 0) {
-        fin[(wave * 16 + l16) * 2] = m2 * AE_LN2;
-        fin[(wave * 16 + l16) * 2 + 1] = r_tot;
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // surplus tile requests must not outlive the workgroup's LDS
-    __syncthreads();
-    return;
-  }
-
-  // ================================= value wave: AE_DVW value columns, 64 heads ========================
-  const int l32 = lane & 31;
-  const int hf = lane >> 5;
-  const int dvw = wave - 4;
   ae_f32x16 oacc[2][AE_NDB];     // [head block][dv block]: O^T
 #pragma unroll
   for (int hb = 0; hb < 2; hb++)
@@ -304,7 +319,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
       const ae_lds_byte* xb = xbuf + (t & 1) * AE_X_BYTES;
       // rescale O for the heads whose reference moved (rare once the maxima have settled)
       const ae_lds_i32* flags = (const ae_lds_i32*)(xb + AE_HEADS_PER_WG * 4);
-      if (__builtin_amdgcn_readfirstlane(flags[0] | flags[1] | flags[2] | flags[3]) != 0) {
+      if (__builtin_amdgcn_readfirstlane(flags[0] | flags[1]) != 0) {
 #pragma unroll
         for (int hb = 0; hb < 2; hb++) {
           const float osc = ((const ae_lds_f32*)xb)[hb * 32 + l32];
