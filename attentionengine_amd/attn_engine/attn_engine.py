@@ -115,14 +115,18 @@ class AttentionEngine:
             assert q_seqlen == 1
             from core.lower.lower_decode import GQADecodeOp
             return GQADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value)
-        if not dynamic and q_seqlen != kv_len and head == head_kv:
+        # MHA decode (attn_engine.py:273-290 of the reference): a few query tokens against a long KV,
+        # split over the kv axis and merged with the user's combine()
+        # (an online function that does not override combine() cannot merge splits: it runs unsplit)
+        has_combine = online_func is not None and getattr(type(online_func), "combine", None) is not OnlineFunc.combine
+        split_kv = not dynamic and q_seqlen != kv_len and head == head_kv and has_combine
+        if split_kv:
             assert q_seqlen < kv_len
-            raise NotImplementedError(
-                "MHA decode with q_len > 1 (attn_script/mha_inference.py) is not built yet")
         from core.lower.prefill_op import PrefillOp
         return PrefillOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                          infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
-                         infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask)
+                         infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
+                         split_kv=split_kv)
 
     def __call__(self, *args, **kargs):
         if kargs.get("block_mask") is not None:

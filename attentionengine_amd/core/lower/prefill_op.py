@@ -23,7 +23,7 @@ def _dim(x, default):
 class PrefillOp:
     def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
-                 extern_block_mask=False):
+                 extern_block_mask=False, split_kv=False, target_workgroups=512):
         q_meta, k_meta, v_meta = qkv_meta
         self.dtype = q_meta.dtype
         self.D = int(q_meta.shape[3])
@@ -41,6 +41,19 @@ class PrefillOp:
         self.functor_src = L.render_functors(self.functors)
         self.tiles = L.choose_prefill_tiles(self.D, self.DV, _dim(q_meta.shape[2], 0), self.functors.softmax,
                                             _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1))
+        # Split-KV ("MHA decode": a few query tokens against a long KV, attn_engine.py:273-290 and
+        # core/lower/lower_decode.py:287-313 of the reference): the kv axis is shared out over several
+        # workgroups per q tile and the partial results are merged with the user's combine().
+        self.split_kv = bool(split_kv)
+        self.target_workgroups = int(target_workgroups)
+        if self.split_kv:
+            if self.tiles.template == "ae_prefill_simple.hip":
+                raise NotImplementedError("split-KV prefill needs head dims 64 or 128")
+            if not hasattr(online_func, "combine"):
+                raise NotImplementedError("split-KV needs OnlineFunc.combine to merge the partial results")
+            from .lower_decode import lower_combine
+            self.tiles = L.PrefillTiles()          # the generic kernel carries the split-KV mode
+            self.functor_src += lower_combine(online_func, self.functors.final_rowscale_names)
         if self.extern_block_mask and self.tiles.rows_per_wave != 32 and (
                 self.mask_block[1] % self.tiles.block_n or
                 (self.tiles.block_m % self.mask_block[0] and self.mask_block[0] % self.tiles.block_m)):
@@ -68,7 +81,8 @@ class PrefillOp:
         if Sq > 0:
             plan = self._plan(B, H, Sq, Skv, device=None)
             mode = 2 if self.extern_block_mask else plan.mode
-            _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0)
+            n_split, _ = self.plan_splits(B, H, Sq, Skv)
+            _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split)
             self.source = cfg_src + "\n" + self.functor_src
             if infer_mask and mask_mod is not None and not self.extern_block_mask:
                 self.block_mask = self._reference_block_mask(B, H, Sq, Skv)
@@ -108,14 +122,30 @@ class PrefillOp:
         return blocks.contiguous()
 
     # ---- kernels -------------------------------------------------------------------------
-    def _variant(self, mask_mode, even_q, even_kv):
-        key = (mask_mode, even_q, even_kv)
+    COMBINE_THREADS = 128
+
+    def plan_splits(self, B, Hq, Sq, Skv):
+        """(number of KV splits, kv positions per split): enough workgroups to fill the chip, whole
+        kv tiles per split, no empty split."""
+        if not self.split_kv:
+            return 1, Skv
+        bn = self.tiles.block_n
+        kv_tiles = -(-Skv // bn)
+        wgs = -(-Sq // self.tiles.block_m) * (-(-(B * Hq) // 8) * 8)
+        want = max(1, min(kv_tiles, -(-self.target_workgroups // wgs)))
+        per = -(-kv_tiles // want)
+        return -(-kv_tiles // per), per * bn
+
+    def _variant(self, mask_mode, even_q, even_kv, n_split=1):
+        key = (mask_mode, even_q, even_kv, n_split)
         v = self._variants.get(key)
         if v is None:
             has_mask_mod = self.elementwise_mask and mask_mode != 1
             cfg_src = L.render_config(self.D, self.DV, self.dtype, self.tiles, mask_mode, has_mask_mod,
                                       self.n_rowscales, self.functors.o_scale_one, even_q, even_kv,
                                       self.functors.softmax if self.tiles.rows_per_wave == 64 else None)
+            if n_split > 1:
+                cfg_src += f"#define AE_NSPLIT {n_split}\n#define AE_COMBINE_THREADS {self.COMBINE_THREADS}\n"
             module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,
                                                           "ae_functors.h": self.functor_src})
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
@@ -163,11 +193,14 @@ class PrefillOp:
         else:
             plan = self._plan(B, Hq, Sq, Skv, dev)
             mode, table, mbm, mbn = plan.mode, plan.table, plan.block_m, plan.block_n
-        module, cfg, _ = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0)
+        n_split, kv_per_split = self.plan_splits(B, Hq, Sq, Skv)
+        module, cfg, _ = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split)
         kern = module.kernel("ae_prefill_kernel")
 
         out = torch.empty((B, Sq, Hq, self.DV), dtype=self.dtype, device=dev)
-        rowscales = [torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev) for _ in range(self.n_rowscales)]
+        # the merge kernel of the split-KV path writes rowscales in (batch, q position, head) order
+        rs_shape = (B, Sq, Hq) if n_split > 1 else (B, Hq, Sq)
+        rowscales = [torch.empty(rs_shape, dtype=torch.float32, device=dev) for _ in range(self.n_rowscales)]
         p = rt.AttnParams()
         p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
         for i, r in enumerate(rowscales):
@@ -187,7 +220,20 @@ class PrefillOp:
             p.mask_b, p.mask_h, p.mask_nq, p.mask_nkv = table.shape
             p.mask_block_m, p.mask_block_n = mbm, mbn
             keep.append(table)
-        rt.prefill_fwd(kern, p, cfg, torch.cuda.current_stream(dev).cuda_stream)
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        if n_split > 1:
+            partial_o = torch.empty((B, Sq, Hq, n_split, self.DV), dtype=torch.float32, device=dev)
+            partial_rs = torch.empty((max(1, self.n_rowscales), B, Sq, Hq, n_split), dtype=torch.float32, device=dev)
+            p.partial_o, p.partial_rs = partial_o.data_ptr(), partial_rs.data_ptr()
+            p.num_splits, p.kv_per_split = n_split, kv_per_split
+            keep += [partial_o, partial_rs]
+            ccfg = rt.TileCfg(block_m=1, block_n=n_split, threads=self.COMBINE_THREADS, lds_bytes=0,
+                              head_dim=self.D, head_dim_v=self.DV, elem_bytes=2,
+                              n_rowscales=self.n_rowscales, mask_mode=0)
+            rt.prefill_split_fwd(kern, module.kernel("ae_decode_combine_kernel"), p, cfg, ccfg, stream)
+            rowscales = [r.transpose(1, 2).contiguous() for r in rowscales]
+        else:
+            rt.prefill_fwd(kern, p, cfg, stream)
         self.final_rowscales = dict(zip(self.functors.final_rowscale_names, rowscales))
         self._keepalive = keep
         return out

@@ -108,6 +108,8 @@ _SIGNATURES = {
                                 C.POINTER(TileCfg), _VP]),
     "ae_mla_decode_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
                                     C.POINTER(TileCfg), _VP]),
+    "ae_prefill_split_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
+                                       C.POINTER(TileCfg), _VP]),
     "ae_event_create": (C.c_int, [C.POINTER(_VP)]),
     "ae_event_record": (C.c_int, [_VP, _VP]),
     "ae_event_elapsed_ms": (C.c_int, [_VP, _VP, C.POINTER(C.c_float)]),
@@ -312,6 +314,12 @@ def decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
     _check(lib().ae_decode_fwd(split.handle, combine.handle if combine else None, C.byref(params),
                                C.byref(cfg), C.byref(combine_cfg) if combine_cfg else None,
                                _VP(stream)))
+
+
+def prefill_split_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
+                      combine_cfg: TileCfg, stream: int = 0):
+    _check(lib().ae_prefill_split_fwd(split.handle, combine.handle, C.byref(params), C.byref(cfg),
+                                      C.byref(combine_cfg), _VP(stream)))
 
 
 def mla_decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,

@@ -376,6 +376,53 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
   return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
 }
 
+int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                         const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
+  if (!split || !combine || !combine_cfg)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: kernel/cfg is NULL");
+  int rc = check_common("ae_prefill_split_fwd", p, cfg);
+  if (rc) return rc;
+  if (p->num_splits <= 1 || p->kv_per_split <= 0 ||
+      (int64_t)p->num_splits * p->kv_per_split < p->seqlen_kv)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: %d splits of %d do not cover Skv=%d",
+                p->num_splits, p->kv_per_split, p->seqlen_kv);
+  if (p->kv_per_split % cfg->block_n != 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: kv_per_split=%d is not a multiple of block_n=%d",
+                p->kv_per_split, cfg->block_n);
+  if (combine_cfg->block_n != p->num_splits)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: combine kernel built for %d splits, got %d",
+                combine_cfg->block_n, p->num_splits);
+  if (!p->partial_o || !p->partial_rs)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: split-KV work buffers are NULL");
+  if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: bad combine workgroup size %d",
+                combine_cfg->threads);
+  for (int i = 0; i < combine_cfg->n_rowscales; i++)
+    if (!p->rowscale_out[i])
+      return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: rowscale_out[%d] is NULL", i);
+  if (p->o_stride_h != cfg->head_dim_v || p->o_stride_s != (int64_t)p->heads_q * cfg->head_dim_v ||
+      p->o_stride_b != (int64_t)p->seqlen_q * p->heads_q * cfg->head_dim_v)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: out must be contiguous [B,Sq,Hq,DV]");
+  uint64_t q_tiles = ((uint64_t)p->seqlen_q + cfg->block_m - 1) / cfg->block_m;
+  uint64_t bh = (uint64_t)p->heads_q * (uint64_t)p->batch;
+  uint64_t total = q_tiles * ((bh + 7) / 8) * 8 * (uint64_t)p->num_splits;
+  uint64_t rows = (uint64_t)p->seqlen_q * (uint64_t)p->heads_q;
+  if (total == 0 || total > 0x7fffffffull || rows > 0x7fffffffull)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: grid of %llu workgroups",
+                (unsigned long long)total);
+  uint32_t grid[3] = {(uint32_t)total, 1, 1};
+  uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
+  rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+  if (rc) return rc;
+  // the merge kernel sees the (q position, head) pairs as the heads of a one-token decode
+  ae_attn_params cp = *p;
+  cp.heads_q = (int32_t)rows;
+  cp.seqlen_q = 1;
+  uint32_t cgrid[3] = {(uint32_t)rows, (uint32_t)p->batch, 1};
+  uint32_t cblock[3] = {(uint32_t)combine_cfg->threads, 1, 1};
+  return ae_launch(combine, &cp, sizeof cp, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
+}
+
 int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                       const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
   if (!split || !combine_cfg)

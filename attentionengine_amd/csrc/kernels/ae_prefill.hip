@@ -34,6 +34,9 @@
 
 #include "ae_hip.h"
 #include "ae_config.h"    // generated: the AE_* configuration macros
+#ifndef AE_NSPLIT
+#define AE_NSPLIT 1                // > 1: split-KV, fp32 partial results + the merge kernel of ae_combine.h
+#endif
 #include "ae_device.h"
 #include "ae_functors.h"  // generated: the functor bodies
 
@@ -92,7 +95,13 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // The grid is padded to 8*ceil(n_bh/8)*n_qt ids; surplus workgroups exit immediately.
   const int n_qt = (p.seqlen_q + AE_BM - 1) / AE_BM;
   const int n_bh = p.batch * p.heads_q;
+#if AE_NSPLIT > 1
+  // split-KV ("decode" with several query tokens): consecutive ids are the splits of one q tile
+  const int split = blockIdx.x % AE_NSPLIT;
+  const int wg = blockIdx.x / AE_NSPLIT;
+#else
   const int wg = blockIdx.x;
+#endif
   const int xcd = wg & 7;
   const int slot = wg >> 3;
 #if AE_MASK_MODE == 1
@@ -251,7 +260,17 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int v_sw = v_row & (AE_VPPR - 1);
   const int v_g = l32 >> 4;
 
+#if AE_NSPLIT > 1
+  // this workgroup's share of the kv axis: kv_per_split positions (a multiple of the tile)
+  const int j_begin = split * (p.kv_per_split / AE_BN);
+  {
+    const int lim = j_begin + p.kv_per_split / AE_BN;
+    j_end = lim < j_end ? lim : j_end;
+  }
+  int j = next_tile(j_begin);
+#else
   int j = next_tile(0);
+#endif
   bool any_tile = j < j_end;
   if (any_tile) load_tile(j, 0);
   // Drain every outstanding load (Q fragments, first tile) before the loop: with loads still
@@ -396,6 +415,26 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
     }
+#if AE_NSPLIT > 1
+    // partial result of this split: fp32, rows ordered (batch, q position, head) so that the merge
+    // kernel sees them as B x (Sq*Hq) "heads" of a one-token decode and writes out [B,Sq,Hq,DV]
+    if (q_ok[rb]) {
+      const int64_t prow = ((((int64_t)b * p.seqlen_q + qrow[rb]) * p.heads_q + h) * AE_NSPLIT) + split;
+      float* po = p.partial_o + prow * AE_DV;
+#pragma unroll
+      for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_f32x4 w = {o[db * 16 + rg * 4 + 0], o[db * 16 + rg * 4 + 1], o[db * 16 + rg * 4 + 2], o[db * 16 + rg * 4 + 3]};
+          *(ae_f32x4*)(po + db * 32 + rg * 8 + hf * 4) = w;
+        }
+      if (hf == 0) {
+#pragma unroll
+        for (int i = 0; i < AE_N_ROWSCALES; i++)
+          p.partial_rs[(int64_t)i * p.batch * p.seqlen_q * p.heads_q * AE_NSPLIT + prow] = frs[i];
+      }
+    }
+#else
     if (q_ok[rb]) {
       ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow[rb] * p.o_stride_s +
                       (int64_t)h * p.o_stride_h;
@@ -414,5 +453,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
           p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[rb]] = frs[i];
       }
     }
+#endif
   }
 }
+
+#if AE_NSPLIT > 1
+#include "ae_combine.h"
+#endif

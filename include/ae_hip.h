@@ -186,6 +186,18 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                   const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
 
 /*
+ * ae_prefill_split_fwd: split-KV attention for a FEW query tokens against a long KV ("MHA decode",
+ *   the reference's generic decode template core/template/tl_template/attn/attn_decode_tl.py:47-205,
+ *   selected in attn_engine/attn_engine.py:273-290).  The prefill kernel compiled with AE_NSPLIT =
+ *   num_splits runs once per (q tile, head, batch, split) on kv_per_split positions (a multiple of
+ *   block_n) and writes fp32 partials ordered (batch, q position, head, split); the combine kernel then
+ *   merges them with the user's combine() into `out`, which must be contiguous [B,Sq,Hq,DV], and writes
+ *   the merged rowscales in (batch, q position, head) order to rowscale_out (the caller transposes).
+ */
+int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                         const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
+
+/*
  * ae_mla_decode_fwd: shared-latent-KV (MLA) decode. K = [k | k2] (latent | rope), q = [q | q2],
  *   V = the first head_dim_v columns of k. Stands where the reference calls its TileLang MLA
  *   kernel (mla_decode_tl.py:326-335) or `fwd_kvcache_mla`

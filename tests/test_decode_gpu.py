@@ -134,3 +134,47 @@ def test_mla_decode_cute_convention(cuda_device):
     cos_diff = 1 - 2 * (x * y).sum().item() / max((x * x + y * y).sum().item(), 1e-12)
     assert cos_diff < 1e-5
     assert (x - y).abs().max().item() <= LSE_TOL
+
+
+def _mha_decode_engine(B, H, Sq, Skv, D, dtype, online, mask_mod=None):
+    meta = (meta_tensor(B, H, Sq, D, dtype=dtype), meta_tensor(B, H, Skv, D, dtype=dtype),
+            meta_tensor(B, H, Skv, D, dtype=dtype))
+    return AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)),
+                           mask_mod=mask_mod, online_func=online)
+
+
+@pytest.mark.parametrize("B,H,Sq,Skv,D,dtype", [
+    (1, 32, 128, 8192, 128, torch.float16),   # attn_script/mha_inference.py shape
+    (2, 4, 5, 1000, 128, torch.float16),      # q rows and kv length that are no multiple of any tile
+    (1, 2, 64, 4096, 64, torch.bfloat16),
+    (2, 3, 1, 300, 128, torch.float16),       # one query token, as many heads as kv heads
+])
+def test_mha_decode_split_kv(cuda_device, B, H, Sq, Skv, D, dtype):
+    """A few query tokens against a long KV with as many kv heads as q heads: the kv axis is split
+    over workgroups and merged with OnlineFunc.combine (attn_engine.py:273-290 and
+    core/template/tl_template/attn/attn_decode_tl.py:47-205 of the reference)."""
+    print(f"case mha decode B{B} H{H} Sq{Sq} Skv{Skv} D{D} {dtype}", flush=True)
+    q, k, v = C.make_inputs(B, Sq, Skv, H, H, D, D, dtype)
+    mod = _mha_decode_engine(B, H, Sq, Skv, D, dtype, C.OnlineSoftmax())
+    n_split, per = mod.attention.plan_splits(B, H, Sq, Skv)
+    assert n_split > 1 and n_split * per >= Skv and (n_split - 1) * per < Skv
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    ref, lse = R.softmax_attention(q, k, v, causal=False)
+    assert out.shape == (B, Sq, H, D) and out.dtype == dtype
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    got = mod.final_rowscales["lse"]
+    assert got.shape == (B, H, Sq)
+    assert (got.cpu() - lse).abs().max().item() <= LSE_TOL
+
+
+def test_mha_decode_matches_unsplit(cuda_device):
+    """Merge invariant: the split-KV result equals the same engine run without splitting."""
+    B, H, Sq, Skv, D, dtype = 1, 8, 32, 2048, 128, torch.float16
+    q, k, v = C.make_inputs(B, Sq, Skv, H, H, D, D, dtype)
+    mod = _mha_decode_engine(B, H, Sq, Skv, D, dtype, C.OnlineSoftmax())
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    lse = mod.final_rowscales["lse"].clone()
+    mod.attention.split_kv = False
+    out1 = mod(q.cuda(), k.cuda(), v.cuda())
+    assert (out.float() - out1.float()).abs().max().item() <= 2e-3
+    assert (lse - mod.final_rowscales["lse"]).abs().max().item() <= 1e-4

@@ -185,6 +185,13 @@ def test_engine_dispatch_and_compile_on_cpu():
     gqa = AttentionEngine(_meta(1, 8, 2, 256, 256, 64, 64, torch.float16), CustomIO({}), sm, C.causal_mask,
                           C.OnlineSoftmax())
     assert isinstance(gqa._op, PrefillOp)
+    # MHA decode (attn_script/mha_inference.py): a few query tokens against a long KV -> split-KV prefill
+    mhad = AttentionEngine(_meta(1, 32, 32, 128, 8192, 128, 128, torch.float16), CustomIO({}), sm, None,
+                           C.OnlineSoftmax())
+    assert isinstance(mhad._op, PrefillOp) and mhad._op.split_kv
+    assert mhad._op.plan_splits(1, 32, 128, 8192) == (16, 512)
+    assert mhad._op.plan_splits(2, 4, 5, 1000) == (16, 64)       # never an empty split, whole tiles
+    assert "#define AE_NSPLIT 16" in mhad.tl_code and "ae_combine" in mhad.tl_code
     # tuner / backend arguments of the reference scripts are accepted
     AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), sm, C.causal_mask,
                     C.OnlineSoftmax(), tune=True, tune_file="x.json", tune_bwd=True, backend="cute")
@@ -199,8 +206,10 @@ def test_engine_error_behaviour():
         AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float32), CustomIO({}), sm, None, C.OnlineSoftmax())
     with pytest.raises(AssertionError):  # decode asserts q_len == 1 (attn_engine.py:255)
         AttentionEngine(_meta(1, 8, 2, 4, 1024, 64, 64, torch.float16), CustomIO({}), sm, None, C.OnlineSoftmax())
-    with pytest.raises(NotImplementedError):
-        AttentionEngine(_meta(1, 2, 2, 128, 1024, 64, 64, torch.float16), CustomIO({}), sm, None, C.OnlineSoftmax())
+    # an online function without combine() cannot merge KV splits: the same shape runs unsplit
+    unsplit = AttentionEngine(_meta(1, 2, 2, 128, 1024, 64, 64, torch.float16), CustomIO({}), sm, None,
+                              C.OnlineIdentity())
+    assert not unsplit._op.split_kv and unsplit._op.plan_splits(1, 2, 128, 1024) == (1, 1024)
     with pytest.raises(ValueError):
         AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), sm, None,
                         C.OnlineSoftmax(), backend="triton")
