@@ -216,3 +216,30 @@ def do_bench_reluattn(attn, B, H, S, D, DV, dtype=torch.float16, causal=False, r
     latency_ref = do_bench(ref_program, warmup=50, rep=100)
     _report("eager torch", latency_ref, tflops)
     return latency, tflops / latency * 1e-9, latency_ref, tflops / latency_ref * 1e-9
+
+
+def do_bench_retention(attn, B, H, S, D, DV, dtype=torch.bfloat16):
+    """Retention with a decay-mask input (attn_script/retention.py); inputs, reference and flop
+    count as bench_utils.py:1025-1100 of the reference: q scaled by D^-0.5, mask = rand.tril()."""
+    tflops = (2 * B * H * S * S * D + 2 * B * H * S * S * DV) * 0.5
+    torch.cuda.manual_seed(0)
+    device = "cuda"
+    query = torch.randn(B, S, H, D, device=device, dtype=dtype) * ((1 / D) ** 0.5)
+    key = torch.randn(B, S, H, D, device=device, dtype=dtype)
+    value = torch.randn(B, S, H, DV, device=device, dtype=dtype)
+    torch.randn(B, S, H, DV, device=device, dtype=dtype)
+    mask = torch.rand(1, H, S, S, device=device, dtype=dtype).tril().contiguous()
+
+    o = attn(query, key, value, mask)
+
+    def ref_program():
+        qk = torch.einsum("bqhd,bkhd->bhqk", query, key)
+        qkm = qk * mask
+        r = qkm.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
+        return torch.einsum("bhqk,bkhd->bqhd", qkm / r, value).to(dtype)
+    print_debug(o, ref_program(), rtol=1e-2, atol=1e-2)
+    latency = do_bench(lambda: attn(query, key, value, mask), warmup=50, rep=100)
+    _report("hip", latency, tflops)
+    latency_ref = do_bench(ref_program, warmup=50, rep=100)
+    _report("eager torch", latency_ref, tflops)
+    return latency, tflops / latency * 1e-9, latency_ref, tflops / latency_ref * 1e-9

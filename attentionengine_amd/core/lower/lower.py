@@ -60,7 +60,7 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
     (fp32, like the reference's accum_dtype fragments, lower.py:580); one with a
     ``seq_len_kv`` dimension is read per element from global memory in the input dtype
     (lower.py:590-597)."""
-    leaves, descs, loads, fields = {}, [], [], []
+    leaves, descs, loads, fields, preambles = {}, [], [], [], {}
     for slot, (name, sym) in enumerate(custom_fwd_inputs.input_tensors.items()):
         slot += slot_offset
         dims = list(sym.shape_idx)
@@ -69,12 +69,15 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
         # row-major index over the declared shape
         extents = {"batch": "p.batch", "heads": "p.heads_q", "seq_len": "p.seqlen_q",
                    _KV_DIM: "p.seqlen_kv"}
+        kv_stride = None
         for d in reversed(dims):
             if d in _DIM_INDEX:
-                idx_terms.append(f"(int64_t)({_DIM_INDEX[d]}) * ({stride})")
+                # rows past seqlen_q (a ragged last q tile) compute on the last row and are never stored
+                ix = "(ctx.q_idx < p.seqlen_q ? ctx.q_idx : p.seqlen_q - 1)" if d == "seq_len" else _DIM_INDEX[d]
+                idx_terms.append(f"(int64_t)({ix}) * ({stride})")
                 stride = f"{stride} * (int64_t){extents[d]}"
             elif d == _KV_DIM:
-                idx_terms.append(f"(int64_t)(AE_KV) * ({stride})")
+                kv_stride = stride          # the kv term is added per element inside the tile loop
                 stride = f"{stride} * (int64_t){extents[d]}"
             elif d == "1":
                 pass
@@ -83,15 +86,40 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
                     f"custom input {name!r}: dimension {d!r} (use 1, 'batch', 'heads', 'seq_len', 'seq_len_kv')")
         index = " + ".join(idx_terms) if idx_terms else "0"
         if per_kv:
-            raise NotImplementedError(
-                f"custom input {name!r} has a seq_len_kv dimension; per-element custom tensors "
-                "(e.g. the retention decay mask) are not lowered yet")
+            # one element per score (e.g. the retention decay mask, attn_script/retention.py:14-16):
+            # the row's base pointer is kept per lane, elements are read in the input dtype where the
+            # scores are modified; kv positions past the end of a ragged tile read the last element
+            fields += [f"const ae_elem* {name}_row;", f"int64_t {name}_kvstride;", f"int {name}_kvlast;"]
+            loads += [f"c.{name}_row = (const ae_elem*)p.custom[{slot}] + ({index});",
+                      f"c.{name}_kvstride = {kv_stride};", f"c.{name}_kvlast = p.seqlen_kv - 1;"]
+            leaves[id(sym)] = (f"cm_{name}", True)
+            # a lane's elements come in groups of four consecutive kv positions (ae_kv_off): one 8-byte
+            # load per group where the tensor allows it (unit kv stride, aligned, inside the row)
+            preambles[id(sym)] = [
+                f"  float cm_{name}[N];", "#pragma unroll",
+                "  for (int g = 0; g < N / 4; g++) {",
+                "    const int kv = ctx.kv_base + ae_kv_off(4 * g);",
+                f"    const ae_elem* src = cust.{name}_row + (int64_t)kv * cust.{name}_kvstride;",
+                f"    if (cust.{name}_kvstride == 1 && kv + 3 <= cust.{name}_kvlast && ((unsigned long)src & 7) == 0) {{",
+                "      const ae_elem4 w = *(const ae_elem4*)src;",
+                "#pragma unroll",
+                f"      for (int i = 0; i < 4; i++) cm_{name}[4 * g + i] = (float)w[i];",
+                "    } else {",
+                "#pragma unroll",
+                "      for (int i = 0; i < 4; i++) {",
+                f"        const int kvi = kv + i < cust.{name}_kvlast ? kv + i : cust.{name}_kvlast;",
+                f"        cm_{name}[4 * g + i] = (float)cust.{name}_row[(int64_t)kvi * cust.{name}_kvstride];",
+                "      }",
+                "    }",
+                "  }"]
+            descs.append(CustomInput(name, dims, per_kv, in_dtype))
+            continue
         fields.append(f"float {name};")
         loads.append(f"c.{name} = ((const float*)p.custom[{slot}])[{index}];")
         leaves[id(sym)] = (f"cust.{name}", False)
         tdtype = torch.float32
         descs.append(CustomInput(name, dims, per_kv, tdtype))
-    return leaves, descs, loads, fields
+    return leaves, descs, loads, fields, preambles
 
 
 # threshold of the lazy running maximum, in the (natural-log) units of the user's exp():
@@ -192,7 +220,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
                    mask_value: str = "-inf") -> LoweredFunctors:
     """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
     custom_fwd_inputs = custom_fwd_inputs if custom_fwd_inputs is not None else CustomIO()
-    cust_leaves, customs, cust_loads, cust_fields = _custom_leaves(custom_fwd_inputs, in_dtype)
+    cust_leaves, customs, cust_loads, cust_fields, cust_preambles = _custom_leaves(custom_fwd_inputs, in_dtype)
 
     def index_leaves():
         b = SymbolScalar("b", Var("b"), shape_idx=[])
@@ -245,6 +273,9 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     if id(kv_idx) in em.done:
         body += ["  float kvf[N];", "#pragma unroll",
                  "  for (int e = 0; e < N; e++) kvf[e] = (float)(ctx.kv_base + ae_kv_off(e));"]
+    for sid, lines in cust_preambles.items():
+        if sid in em.done:
+            body += lines
     body.append(em.code())
     if sval[0] != "s":
         src = f"{sval[0]}[e]" if sval[1] else sval[0]
@@ -272,6 +303,8 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     em = Emitter(leaves, {}, ["dimv"], n="N", prefix="ep")
     oval = em.value(o_new)
     fvals = [(k, em.value(v)) for k, v in final_rowscales.items()]
+    if any(sid in em.done for sid in cust_preambles):
+        raise NotImplementedError("a custom input with a seq_len_kv dimension cannot be used in the epilogue")
     body = [em.code()]
     if oval[0] != "o":
         src = f"{oval[0]}[e]" if oval[1] else oval[0]

@@ -34,12 +34,14 @@ class PrefillOp:
             raise NotImplementedError(f"head dims (D={self.D}, DV={self.DV}) must be multiples of 16 / 32")
         self.mask_mod = mask_mod
         self.elementwise_mask = mask_mod is not None and mask_value == "-inf"
+        self.mask_value_zero = mask_value == "0"
         self.extern_block_mask = bool(extern_block_mask)
         self.mask_block = (int(infer_mask_block_M), int(infer_mask_block_N))
         self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
                                          self.dtype, mask_value)
         self.functor_src = L.render_functors(self.functors)
-        self.tiles = L.choose_prefill_tiles(self.D, self.DV, _dim(q_meta.shape[2], 0), self.functors.softmax,
+        self.tiles = L.choose_prefill_tiles(self.D, self.DV, _dim(q_meta.shape[2], 0),
+                                            None if self.mask_value_zero else self.functors.softmax,
                                             _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1))
         # Split-KV ("MHA decode": a few query tokens against a long KV, attn_engine.py:273-290 and
         # core/lower/lower_decode.py:287-313 of the reference): the kv axis is shared out over several
@@ -144,6 +146,8 @@ class PrefillOp:
             cfg_src = L.render_config(self.D, self.DV, self.dtype, self.tiles, mask_mode, has_mask_mod,
                                       self.n_rowscales, self.functors.o_scale_one, even_q, even_kv,
                                       self.functors.softmax if self.tiles.rows_per_wave == 64 else None)
+            if self.mask_value_zero:
+                cfg_src += "#define AE_MASK_VALUE_ZERO 1\n"
             if n_split > 1:
                 cfg_src += f"#define AE_NSPLIT {n_split}\n#define AE_COMBINE_THREADS {self.COMBINE_THREADS}\n"
             module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,

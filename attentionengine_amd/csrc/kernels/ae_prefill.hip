@@ -40,6 +40,14 @@
 #include "ae_device.h"
 #include "ae_functors.h"  // generated: the functor bodies
 
+// value given to score positions past seqlen_kv before the user functors run: -inf, or 0 for graphs
+// declared with mask_value="0" (no additive -inf mask anywhere, attn_tl.py:124-137 / lower.py:637)
+#if defined(AE_MASK_VALUE_ZERO) && AE_MASK_VALUE_ZERO
+#define AE_KV_PAD 0.f
+#else
+#define AE_KV_PAD AE_NEG_INF
+#endif
+
 #ifndef AE_RB
 #define AE_RB 1
 #endif
@@ -337,7 +345,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #if !AE_EVEN_KV
       if (kv0 + AE_BN > p.seqlen_kv) {
 #pragma unroll
-        for (int e = 0; e < AE_NS; e++) s[e] = (kvb + ae_kv_off(e) < p.seqlen_kv) ? s[e] : AE_NEG_INF;
+        for (int e = 0; e < AE_NS; e++) s[e] = (kvb + ae_kv_off(e) < p.seqlen_kv) ? s[e] : AE_KV_PAD;
       }
 #endif
 

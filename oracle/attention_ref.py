@@ -94,6 +94,20 @@ def relu_attention(q, k, v, scale=None, compute_dtype=torch.float32):
     return _apply_p(p, v, compute_dtype)
 
 
+def retention_attention(q, k, v, mask, compute_dtype=torch.float32):
+    """Retention with a decay mask: s = (QK^T) * mask, out = (s / max(sum_kv |s|, 1)) V, r = that
+    clamped row sum (restates ``ref_program`` of bench_utils.py:1062-1067; the running form of
+    attn_script/retention.py:32-58 telescopes to it).  mask [1|B, Hq, Sq, Skv]; returns
+    (out [B,Sq,Hq,DV], r [B,Hq,Sq])."""
+    B, Sq, Hq, _ = q.shape
+    Hkv = k.shape[2]
+    s = _grouped_scores(q, k, compute_dtype)                          # [B,Hkv,G,Sq,Skv]
+    m = mask.to(compute_dtype).expand(B, Hq, Sq, k.shape[1]).reshape(B, Hkv, Hq // Hkv, Sq, k.shape[1])
+    s = s * m
+    r = s.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
+    return _apply_p(s / r, v, compute_dtype), r.reshape(B, Hq, Sq)
+
+
 def mla_decode(q, q_pe, kv, k_pe, scale=None, compute_dtype=torch.float32):
     """MLA decode: K = [kv | k_pe], V = kv, one latent kv head shared by all q heads.
 

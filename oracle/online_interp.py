@@ -171,9 +171,12 @@ def online_attention(q, k, v, score_mod, mask_mod, online_func, custom_fwd_input
                                    torch.arange(j0, j1).view(1, -1))
                     vis = torch.as_tensor(vis, dtype=torch.bool).expand(Sq, j1 - j0)
                     s = s.masked_fill(~vis, float("-inf"))
-                env = {id(s_in): s, id(sb): float(b), id(sh): float(h), id(sq): qi, id(skv): kvi, **cenv}
+                # custom tensors with a kv dimension contribute their columns of this tile
+                tenv = {id(sym): (cenv[id(sym)][:, j0:j1] if "seq_len_kv" in sym.shape_idx else cenv[id(sym)])
+                        for sym in cust_syms}
+                env = {id(s_in): s, id(sb): float(b), id(sh): float(h), id(sq): qi, id(skv): kvi, **tenv}
                 s = _as_tensor(evaluate(s_out, env), s)
-                env = {id(o_in): s, id(ob): float(b), id(oh): float(h), id(oq): qi, **cenv}
+                env = {id(o_in): s, id(ob): float(b), id(oh): float(h), id(oq): qi, **tenv}
                 for n, r in rowscales.items():
                     env[id(r)] = state[n]
                 memo = {}

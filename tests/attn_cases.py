@@ -134,6 +134,15 @@ class OnlineAbsNorm(OnlineFunc):
         return o, {"r": online_rowscales["r"]}
 
 
+def retention_score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+    """attn_script/retention.py:14-16: the scores times a decay mask given as a [1,H,S,S] input."""
+    return score * custom_fwd_inputs.input_tensors["mask"]
+
+
+def retention_custom_inputs():
+    return CustomIO({"mask": (1, "heads", "seq_len", "seq_len_kv")})
+
+
 def make_inputs(B, Sq, Skv, Hq, Hkv, D, DV, dtype, seed=0):
     """Seeded inputs generated on the CPU in the order q, k, v (fp32 randn, then rounded to
     ``dtype``) so oracle, CPU baseline and GPU kernel see identical values."""

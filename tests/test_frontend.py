@@ -145,9 +145,31 @@ def test_unsupported_graphs_raise():
             super().__init__({"m": SymbolScalar("m", Var("banana"))}, {}, CustomIO())
     with pytest.raises(NotImplementedError):
         L.trace_functors(None, None, Bad(), CustomIO({}), torch.float16)
-    with pytest.raises(NotImplementedError):   # per-element custom tensors are not lowered yet
-        L.trace_functors(lambda s, c, b, h, q, kv: s * c.input_tensors["mask"], None, C.OnlineIdentity(),
-                         CustomIO({"mask": (1, "heads", "seq_len", "seq_len_kv")}), torch.float16)
+    with pytest.raises(NotImplementedError):   # an unknown dimension name in a custom input's shape
+        L.trace_functors(lambda s, c, b, h, q, kv: s * c.input_tensors["x"], None, C.OnlineIdentity(),
+                         CustomIO({"x": (1, "channels")}), torch.float16)
+
+
+def test_custom_input_with_a_kv_dimension_is_read_per_score():
+    """The retention decay mask (attn_script/retention.py:14-16, lower.py:590-597 of the reference):
+    a [1,H,S,S] input is indexed by the lane's row once and by kv position inside the tile loop."""
+    lf = L.trace_functors(C.retention_score_mod, C.causal_mask, C.OnlineAbsNorm(), C.retention_custom_inputs(),
+                          torch.float16, mask_value="0")
+    text = L.render_functors(lf)
+    assert lf.customs[0].per_kv and lf.customs[0].torch_dtype == torch.float16
+    assert "const ae_elem* mask_row;" in text and "p.custom[0]" in text
+    assert "(int64_t)(ctx.h) * (1 * (int64_t)p.seqlen_kv * (int64_t)p.seqlen_q)" in text   # [1, heads, seq_len, seq_len_kv]
+    assert "*(const ae_elem4*)src" in text and "ctx.kv_base + ae_kv_off(4 * g)" in text
+    assert "(s[e] * cm_mask[e])" in text and "ae_row_abssum<N>" in text
+    with pytest.raises(NotImplementedError):   # ... but not in the epilogue, which has no kv position
+        class Epi(C.OnlineIdentity):
+            @staticmethod
+            def online_fwd_epilogue(o, rs, b, h, q_idx):
+                return o, {}
+        bad = Epi()
+        cio = C.retention_custom_inputs()
+        bad.online_fwd_epilogue = staticmethod(lambda o, rs, b, h, q_idx: (o * cio.input_tensors["mask"], {}))
+        L.trace_functors(None, None, bad, cio, torch.float16)
 
 
 def test_combine_lowering_finds_the_merged_lse():

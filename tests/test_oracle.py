@@ -197,3 +197,30 @@ def test_block_classes_brute_force():
             blk = dense[0, 0, i * 16:(i + 1) * 16, j * 8:(j + 1) * 8]
             want = 0 if not blk.any() else (2 if blk.all() else 1)
             assert cls[0, 0, i, j] == want
+
+
+def test_retention_closed_form_loops_and_running_form():
+    """Retention with a decay mask (bench_utils.py:1062-1067): python loops on a tiny case, and the
+    running form of attn_script/retention.py:32-58 (abs-sum, clamp at 1, o_scale = r / r_new) run
+    tile by tile through the DAG interpreter telescopes to the same result for any tile width."""
+    B, S, H, D, DV = 1, 9, 2, 8, 4
+    q, k, v = C.make_inputs(B, S, S, H, H, D, DV, torch.float32, seed=8)
+    g = torch.Generator().manual_seed(9)
+    # rows both below and above the clamp
+    mask = torch.rand(1, H, S, S, generator=g).tril() * torch.linspace(0.01, 3.0, S).view(1, 1, S, 1)
+    out, r = R.retention_attention(q, k, v, mask, compute_dtype=torch.float64)
+    for h in range(H):
+        for i in range(S):
+            s = [sum(float(q[0, i, h, d]) * float(k[0, j, h, d]) for d in range(D)) * float(mask[0, h, i, j])
+                 for j in range(S)]
+            rr = max(sum(abs(x) for x in s), 1.0)
+            assert abs(float(r[0, h, i]) - rr) < 1e-9
+            for c in range(DV):
+                ref = sum(s[j] / rr * float(v[0, j, h, c]) for j in range(S))
+                assert abs(float(out[0, i, h, c]) - ref) < 1e-9
+    assert (r > 1.0).any() and (r == 1.0).any()
+    for bn in (2, 4, 16):
+        o2, fin = online_attention(q, k, v, C.retention_score_mod, C.causal_mask, C.OnlineAbsNorm(),
+                                   custom_fwd_inputs=C.retention_custom_inputs(), custom_tensors=(mask,),
+                                   block_n=bn, mask_value="0")
+        assert torch.allclose(o2, out, atol=1e-12) and torch.allclose(fin["r"], r, atol=1e-12)

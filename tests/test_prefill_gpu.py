@@ -245,3 +245,27 @@ def test_pipelined_kernel(cuda_device, monkeypatch, case):
     if (~visible).any():
         assert out[~visible.permute(0, 2, 1)].abs().max().item() == 0.0
         assert torch.isinf(lse[~visible]).all()
+
+
+@pytest.mark.parametrize("B,H,S,D,DV,dtype", [
+    (1, 2, 256, 64, 64, torch.float16),
+    (2, 3, 200, 128, 128, torch.bfloat16),     # ragged q and kv tiles, batch > 1 against a [1,H,S,S] mask
+    (1, 2, 512, 256, 512, torch.float16),      # head dims of attn_script/retention.py
+])
+def test_retention_with_decay_mask_input(cuda_device, B, H, S, D, DV, dtype):
+    """attn_script/retention.py: score * mask with the mask a [1,H,S,S] input tensor (one element
+    per score, read inside the tile loop), abs-sum normalisation clamped at 1, mask_value="0"."""
+    print(f"case retention B{B} H{H} S{S} D{D} DV{DV} {dtype}", flush=True)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, DV, dtype)
+    q = (q.float() * (1 / D) ** 0.5).to(dtype)                       # bench_utils.py:1034-1036
+    g = torch.Generator().manual_seed(5)
+    mask = (torch.rand(1, H, S, S, generator=g) * 4.0).tril().to(dtype).contiguous()
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, H, S, D, dtype=dtype),
+            meta_tensor(B, H, S, DV, dtype=dtype))
+    mod = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
+                          mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0")
+    out = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).float().cpu()
+    ref, r = R.retention_attention(q, k, v, mask)
+    assert (r > 1.0).any()
+    assert (mod.final_rowscales["r"].cpu() - r).abs().max().item() <= 2e-3 * r.max().item()
+    assert (out - ref).abs().max().item() <= OUT_TOL
