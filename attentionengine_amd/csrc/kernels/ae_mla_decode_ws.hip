@@ -174,15 +174,20 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         const bool tail = kv_begin + tn * AE_BN + AE_BN > kv_end;
         float mx = AE_NEG_INF;
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-          x[e] = (sacc[0][e] + sacc[1][e]) * (AE_SM_SCALE * AE_LOG2E);
-          if (tail) x[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
-          mx = __builtin_fmaxf(mx, x[e]);
+        for (int e = 0; e < 16; e++) x[e] = sacc[0][e] + sacc[1][e];   // raw scores: the scale is folded into the exponent
+        if (__builtin_expect(tail, 0)) {
+          // the empty asm keeps this a branch: flattened into selects it costs 5 instructions per score
+          // on every tile
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int e = 0; e < 16; e++) x[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
         }
+#pragma unroll
+        for (int e = 0; e < 16; e++) mx = __builtin_fmaxf(mx, x[e]);
         {
           float hi;
           const float lo = ae_swap32_lo_hi(mx, hi);
-          mx = __builtin_fmaxf(lo, hi);
+          mx = __builtin_fmaxf(lo, hi) * (AE_SM_SCALE * AE_LOG2E);   // the scale is positive
         }
         const bool need = (mx - m2) > AE_TAU2;
         const float mn = need ? mx : m2;
@@ -195,7 +200,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
           ae_elem4 w;
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            const float pv = ae_exp2(x[4 * rb + i] - mn);
+            const float pv = ae_exp2(__builtin_fmaf(x[4 * rb + i], AE_SM_SCALE * AE_LOG2E, -mn));
             rs += pv;
             w[i] = (ae_elem)pv;
           }
