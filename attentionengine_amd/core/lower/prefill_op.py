@@ -32,6 +32,13 @@ class PrefillOp:
             raise ValueError("q and k head dims differ")
         if self.D % 16 or self.DV % 32:
             raise NotImplementedError(f"head dims (D={self.D}, DV={self.DV}) must be multiples of 16 / 32")
+        # Value head dims above 256 (attn_script/retention.py: DV = 512) run as several launches over
+        # column slices of V and of the output: O for 512 columns would need 256 accumulator registers
+        # per lane, which spills (measured 8.0 ms against 2 x 1.2 ms at B1 H32 S4096 D256).  The scores
+        # are recomputed per slice; the row scales of every launch are the same.
+        self.DV_launch = self.DV
+        if self.DV > 256:
+            self.DV_launch = next(c for c in (256, 192, 128, 96, 64, 32) if self.DV % c == 0)
         self.mask_mod = mask_mod
         self.elementwise_mask = mask_mod is not None and mask_value == "-inf"
         self.mask_value_zero = mask_value == "0"
@@ -40,7 +47,7 @@ class PrefillOp:
         self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
                                          self.dtype, mask_value)
         self.functor_src = L.render_functors(self.functors)
-        self.tiles = L.choose_prefill_tiles(self.D, self.DV, _dim(q_meta.shape[2], 0),
+        self.tiles = L.choose_prefill_tiles(self.D, self.DV_launch, _dim(q_meta.shape[2], 0),
                                             None if self.mask_value_zero else self.functors.softmax,
                                             _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1))
         # Split-KV ("MHA decode": a few query tokens against a long KV, attn_engine.py:273-290 and
@@ -51,6 +58,8 @@ class PrefillOp:
         if self.split_kv:
             if self.tiles.template == "ae_prefill_simple.hip":
                 raise NotImplementedError("split-KV prefill needs head dims 64 or 128")
+            if self.DV_launch != self.DV:
+                raise NotImplementedError("split-KV prefill with a value head dim above 256")
             if not hasattr(online_func, "combine"):
                 raise NotImplementedError("split-KV needs OnlineFunc.combine to merge the partial results")
             from .lower_decode import lower_combine
@@ -143,7 +152,7 @@ class PrefillOp:
         v = self._variants.get(key)
         if v is None:
             has_mask_mod = self.elementwise_mask and mask_mode != 1
-            cfg_src = L.render_config(self.D, self.DV, self.dtype, self.tiles, mask_mode, has_mask_mod,
+            cfg_src = L.render_config(self.D, self.DV_launch, self.dtype, self.tiles, mask_mode, has_mask_mod,
                                       self.n_rowscales, self.functors.o_scale_one, even_q, even_kv,
                                       self.functors.softmax if self.tiles.rows_per_wave == 64 else None)
             if self.mask_value_zero:
@@ -154,8 +163,8 @@ class PrefillOp:
                                                           "ae_functors.h": self.functor_src})
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
                              threads=64 * self.tiles.n_waves,
-                             lds_bytes=self.tiles.lds_bytes(self.D, self.DV), head_dim=self.D,
-                             head_dim_v=self.DV, elem_bytes=2, n_rowscales=self.n_rowscales,
+                             lds_bytes=self.tiles.lds_bytes(self.D, self.DV_launch), head_dim=self.D,
+                             head_dim_v=self.DV_launch, elem_bytes=2, n_rowscales=self.n_rowscales,
                              mask_mode=mask_mode)
             v = self._variants[key] = (module, cfg, cfg_src)
         return v
@@ -237,7 +246,12 @@ class PrefillOp:
             rt.prefill_split_fwd(kern, module.kernel("ae_decode_combine_kernel"), p, cfg, ccfg, stream)
             rowscales = [r.transpose(1, 2).contiguous() for r in rowscales]
         else:
-            rt.prefill_fwd(kern, p, cfg, stream)
+            # one launch per slice of DV_launch value columns (a single one unless DV > 256)
+            esz = v.element_size()
+            for c0 in range(0, self.DV, self.DV_launch):
+                p.v = v.data_ptr() + c0 * esz
+                p.out = out.data_ptr() + c0 * esz
+                rt.prefill_fwd(kern, p, cfg, stream)
         self.final_rowscales = dict(zip(self.functors.final_rowscale_names, rowscales))
         self._keepalive = keep
         return out
