@@ -227,10 +227,90 @@ class Emitter:
             self._loop(f"{out}[e] = __builtin_fmaf({base}[e], {float_literal(mul)}, {add});")
         return (out, True)
 
+    # ---- a * tanh(x) + b ----------------------------------------------------------------
+    def _affine_of_tanh(self, sym: SymbolScalar):
+        """(tanh symbol, a, b) if ``sym`` is a*tanh(x) + b built from Mul/Div/Add/Sub/Neg with literal
+        constants, x an array; None otherwise."""
+        a, b = 1.0, 0.0
+        cur = sym
+        while True:
+            t = cur.code.type
+            if t == "Tanh":
+                return (cur, a, b) if self._is_array(cur.prev[0]) and cur is not sym else None
+            if id(cur) in self.done or id(cur) in self.leaves or not cur.prev:
+                return None
+            if t == "Neg":
+                a, cur = -a, cur.prev[0]
+                continue
+            if t not in ("Mul", "Div", "Add", "Sub") or len(cur.prev) != 2:
+                return None
+            x, y = cur.prev
+            cx = float(x.code.value) if x.code.type == "Const" else None
+            cy = float(y.code.value) if y.code.type == "Const" else None
+            if cy is not None and cx is None:
+                if t == "Mul":
+                    a, b = a, b          # out = a*(inner*cy)+b
+                    a *= cy
+                elif t == "Div":
+                    if cy == 0.0:
+                        return None
+                    a /= cy
+                elif t == "Add":
+                    b += a * cy
+                else:
+                    b -= a * cy
+                cur = x
+            elif cx is not None and cy is None:
+                if t == "Mul":
+                    a *= cx
+                elif t == "Add":
+                    b += a * cx
+                elif t == "Sub":     # cx - inner
+                    b += a * cx
+                    a = -a
+                else:
+                    return None
+                cur = y
+            else:
+                return None
+
+    def _emit_affine_of_tanh(self, sym, tanh_sym, a: float, b: float):
+        """a*tanh(x)+b = (a+b) - 2a / (exp(2x) + 1): one exponential and one reciprocal per element,
+        with x's own affine form folded into the exponent.  a = b = 1/2 is the logistic function
+        1 / (1 + exp(-2x)) (attn_script/sigmoidattn.py:14-18 writes sigmoid this way)."""
+        arg = tanh_sym.prev[0]
+        aff = self._as_affine(arg)
+        if aff is None:
+            base, mul, add = self.value(arg)[0], 1.0, None
+        else:
+            base, mul, add = aff
+        logistic = abs(a - 0.5) < 1e-12 and abs(b - 0.5) < 1e-12
+        k = (-2.0 if logistic else 2.0) * mul * LOG2E
+        if add is None:
+            ex = f"ae_exp2({base}[e] * {float_literal(k)})"
+        else:
+            hoist = self._tmp()
+            self.lines.append(f"const float {hoist} = ({add}) * {float_literal((-2.0 if logistic else 2.0) * LOG2E)};")
+            ex = f"ae_exp2(__builtin_fmaf({base}[e], {float_literal(k)}, {hoist}))"
+        out = self._tmp()
+        self.lines.append(f"float {out}[{self.n}];")
+        if logistic:
+            self._loop(f"{out}[e] = ae_rcp(1.0f + {ex});")
+        else:
+            self._loop(f"{out}[e] = __builtin_fmaf(ae_rcp({ex} + 1.0f), {float_literal(-2.0 * a)}, {float_literal(a + b)});")
+        return (out, True)
+
     def value(self, sym: SymbolScalar):  # noqa: F811  (affine-aware front end of the graph walk)
         key = id(sym)
         if key in self.done:
             return self.done[key]
+        if self._is_array(sym) and sym.code.type in ("Mul", "Div", "Add", "Sub", "Neg") and sym.prev:
+            ft = self._affine_of_tanh(sym)
+            if ft is not None:
+                val = self._emit_affine_of_tanh(sym, *ft)
+                self.done[key] = val
+                self._keep.append(sym)
+                return val
         if self._is_array(sym) and sym.code.type in ("Mul", "Div", "Add", "Sub", "Neg") and sym.prev:
             aff = self._as_affine(sym)
             if aff is not None and key in self.affine:

@@ -136,7 +136,26 @@ def test_emitted_identity_and_custom_scalar():
                           CustomIO({"softmax_bias": (1,)}), torch.float16)
     assert lf.o_scale_one and lf.rowstate_fields == [] and lf.final_rowscale_names == []
     assert lf.customs[0].name == "softmax_bias" and lf.customs[0].torch_dtype == torch.float32
-    assert "ae_tanh" in lf.online_fwd_body and "cust.softmax_bias" in lf.online_fwd_body
+    # ((x*0.5).tanh() + 1) * 0.5 is the logistic function: one exp2 and one reciprocal per score
+    assert "ae_rcp(1.0f + ae_exp2(__builtin_fmaf(s[e], -0.14426950" in lf.online_fwd_body
+    assert "ae_tanh" not in lf.online_fwd_body and "cust.softmax_bias" in lf.online_fwd_body
+
+
+def test_affine_of_tanh_forms():
+    """a*tanh(x)+b with literal constants: the logistic special case, the general case, and a bare
+    tanh (sigmoid script form attn_script/sigmoidattn.py:14-18; tanh semantics tl_gen.py:113-117)."""
+    def lower(f):
+        return L.trace_functors(f, None, C.OnlineIdentity(), CustomIO({}), torch.float16).online_fwd_body
+    gen = lower(lambda s, c, b, h, q, kv: 3.0 - (s * 0.25).tanh() * 2.0)           # a = -2, b = 3
+    assert "__builtin_fmaf(ae_rcp(ae_exp2(s[e] * 0.72134752" in gen and ", 4.0f, 1.0f)" in gen
+    bare = lower(lambda s, c, b, h, q, kv: (s * 0.25).tanh())
+    assert "ae_tanh" in bare
+    # the rewritten forms agree with the definition
+    import math
+    for x in (-30.0, -2.0, -0.1, 0.0, 0.3, 5.0, 40.0):
+        e = 2.0 ** (2 * 0.25 * x * 1.4426950408889634)
+        assert abs((1.0 / (e + 1.0)) * 4.0 + 1.0 - (3.0 - 2.0 * math.tanh(0.25 * x))) < 1e-12
+        assert abs(1.0 / (1.0 + 2.0 ** (-x * 1.4426950408889634)) - 0.5 * (math.tanh(0.5 * x) + 1)) < 1e-12
 
 
 def test_unsupported_graphs_raise():

@@ -269,3 +269,19 @@ def test_retention_with_decay_mask_input(cuda_device, B, H, S, D, DV, dtype):
     assert (r > 1.0).any()
     assert (mod.final_rowscales["r"].cpu() - r).abs().max().item() <= 2e-3 * r.max().item()
     assert (out - ref).abs().max().item() <= OUT_TOL
+
+
+def test_affine_of_tanh_score_mod(cuda_device):
+    """score_mod = 3 - 2*tanh(0.25*s): the emitter's a*tanh(x)+b rewrite against the DAG interpreter."""
+    from oracle.online_interp import online_attention
+    B, H, S, D = 1, 2, 192, 64
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+
+    def sm(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+        return 3.0 - (score * 0.25).tanh() * 2.0
+    mod = _engine(B, H, S, D, D, dtype, sm, None, C.OnlineIdentity())
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    ref, _ = online_attention(q, k, v, sm, None, C.OnlineIdentity(), block_n=64)
+    # sums of S terms of size up to 5: compare relative to the output scale
+    assert (out - ref.float()).abs().max().item() <= 5e-3 * ref.abs().max().item()
