@@ -48,8 +48,10 @@ WORKLOADS = {
 MEASURED_TRAFFIC_BYTES = {
     "c2_causal": 423.5e6 + 68.2e6,       # algorithmic Q+K+V+O+lse: 269.5e6 (K/V are fetched twice: the
                                          # heaviest-first causal order spreads a head's q tiles in time)
+    "c2_full": 201.7e6 + 84.7e6,         # Q+K+V read once: 201.3e6; O + lse written
+    "c3_sigmoid": 201.4e6 + 68.9e6,      # Q+K+V read once; O written (no row scales)
     "c4_gqa_decode": 2147.9e6 + 4.2e6,   # algorithmic K+V: 2147.5e6 (fp32 partials written: 4.2e6)
-    "c5_mla_decode": 623.2e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
+    "c5_mla_decode": 623.1e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
 }
 
 
