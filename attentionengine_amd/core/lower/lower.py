@@ -409,6 +409,15 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
     t = PrefillTiles(template="ae_prefill_simple.hip", k_pad=16)
     if max(d, dv) > 128:
         t.block_n, t.waves_per_eu = 32, 1
+    # the workgroup copies K and V tiles as 16-byte chunks, a whole number per thread: take the
+    # preferred kv tile if it divides, else the other one, else two waves instead of four
+    for n_waves, block_n in ((4, t.block_n), (4, 96 - t.block_n), (2, t.block_n), (2, 96 - t.block_n)):
+        nt = 64 * n_waves
+        if (block_n * d // 8) % nt == 0 and (block_n * dv // 8) % nt == 0:
+            t.n_waves, t.block_n = n_waves, block_n
+            break
+    else:
+        raise NotImplementedError(f"no tile shape for head dims D={d}, DV={dv}")
     # V rows must land on distinct LDS bank groups for the transpose reads: pitch = 64 mod 256
     t.v_pad = (64 - (2 * dv) % 256) % 256
     if t.v_pad == 0:

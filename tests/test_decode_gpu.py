@@ -178,3 +178,25 @@ def test_mha_decode_matches_unsplit(cuda_device):
     out1 = mod(q.cuda(), k.cuda(), v.cuda())
     assert (out.float() - out1.float()).abs().max().item() <= 2e-3
     assert (lse - mod.final_rowscales["lse"]).abs().max().item() <= 1e-4
+
+
+def test_decode_odd_shapes_against_oracle(cuda_device):
+    """Seeded sweep over decode shapes: one key, fewer keys than a tile, KV lengths no tile divides,
+    group sizes 2..24, head dims 64 / 128 / 256, both dtypes."""
+    import random
+    rng = random.Random(4321)
+    cases = [(1, 2, 1, 1, 64), (2, 4, 2, 31, 128), (1, 24, 1, 4097, 128), (1, 6, 3, 257, 256), (3, 16, 8, 95, 64)]
+    for _ in range(8):
+        hkv = rng.choice([1, 2, 4])
+        cases.append((rng.choice([1, 2, 5]), hkv * rng.choice([2, 3, 4, 8]), hkv, rng.randint(1, 3000),
+                      rng.choice([64, 128])))
+    for n, (B, Hq, Hkv, Skv, D) in enumerate(cases):
+        dtype = torch.float16 if n % 2 == 0 else torch.bfloat16
+        print(f"case odd decode B{B} Hq{Hq} Hkv{Hkv} Skv{Skv} D{D} {dtype}", flush=True)
+        q, k, v = C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, dtype, seed=100 + n)
+        mod = _decode_engine(B, Hq, Hkv, Skv, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.OnlineSoftmax())
+        out = mod(q.cuda(), k.cuda(), v.cuda())
+        ref, lse = R.softmax_attention(q, k, v, causal=False)
+        assert torch.isfinite(out).all()
+        assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL, (B, Hq, Hkv, Skv, D)
+        assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL, (B, Hq, Hkv, Skv, D)

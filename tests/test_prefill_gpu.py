@@ -285,3 +285,32 @@ def test_affine_of_tanh_score_mod(cuda_device):
     ref, _ = online_attention(q, k, v, sm, None, C.OnlineIdentity(), block_n=64)
     # sums of S terms of size up to 5: compare relative to the output scale
     assert (out - ref.float()).abs().max().item() <= 5e-3 * ref.abs().max().item()
+
+
+def test_small_and_odd_shapes_against_oracle(cuda_device):
+    """Seeded sweep over shapes the tiles do not divide: one token, fewer keys than a tile, odd head
+    counts, grouped heads, both dtypes, causal and unmasked - every one against the closed form."""
+    import random
+    rng = random.Random(1234)
+    cases = [(1, 1, 1, 1, 64), (1, 1, 1, 17, 128), (2, 3, 3, 33, 64), (1, 2, 1, 65, 128), (1, 5, 5, 129, 96)]
+    for _ in range(10):
+        hkv = rng.choice([1, 2, 3])
+        cases.append((rng.choice([1, 2]), hkv * rng.choice([1, 2, 4]), hkv, rng.randint(2, 300),
+                      rng.choice([64, 128, 96, 160])))
+    # head dims of every kernel template, K and V dims that differ, dims only two waves can tile
+    dims = {160: 160, 96: 96, 64: 64, 128: 128}
+    cases += [(1, 2, 2, 100, (80, 96)), (1, 2, 1, 70, (48, 32)), (1, 1, 1, 150, (112, 224)),
+              (2, 2, 2, 90, (192, 128)), (1, 3, 3, 40, (16, 32)), (1, 2, 2, 130, (256, 256))]
+    for n, (B, H, Hkv, S, D) in enumerate(cases):
+        D, DV = D if isinstance(D, tuple) else (D, dims[D])
+        dtype = torch.float16 if n % 2 == 0 else torch.bfloat16
+        causal = n % 3 != 0
+        print(f"case odd shape B{B} H{H} Hkv{Hkv} S{S} D{D} DV{DV} {dtype} causal={causal}", flush=True)
+        q, k, v = C.make_inputs(B, S, S, H, Hkv, D, DV, dtype, seed=n)
+        mod = _engine(B, H, S, D, DV, dtype, C.make_scale_score_mod(1 / math.sqrt(D)),
+                      C.causal_mask if causal else None, C.OnlineSoftmax(), Hkv=Hkv)
+        out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+        ref, lse = R.softmax_attention(q, k, v, causal=causal)
+        assert torch.isfinite(out).all()
+        assert (out - ref).abs().max().item() <= OUT_TOL, (B, H, Hkv, S, D)
+        assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL, (B, H, Hkv, S, D)
