@@ -200,3 +200,32 @@ def test_decode_odd_shapes_against_oracle(cuda_device):
         assert torch.isfinite(out).all()
         assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL, (B, Hq, Hkv, Skv, D)
         assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL, (B, Hq, Hkv, Skv, D)
+
+
+def test_mla_odd_shapes_against_oracle(cuda_device):
+    """Seeded sweep over MLA decode shapes: head counts below and above a workgroup's 64, several latent
+    heads, KV lengths from one token to lengths no tile divides, both dtypes, split and unsplit."""
+    import random
+    rng = random.Random(99)
+    D, DV = 576, 512
+    scale = 1 / math.sqrt(192)
+    cases = [(1, 1, 1, 1), (1, 7, 1, 33), (2, 96, 1, 1023), (1, 160, 2, 130), (5, 64, 1, 64)]
+    for _ in range(5):
+        g = rng.choice([1, 2])
+        cases.append((rng.choice([1, 3]), g * rng.choice([8, 40, 128]), g, rng.randint(1, 2500)))
+    for n, (B, H, G, S) in enumerate(cases):
+        dtype = torch.bfloat16 if n % 2 == 0 else torch.float16
+        print(f"case odd mla B{B} H{H} G{G} S{S} {dtype}", flush=True)
+        q, q_pe, kv, k_pe = _mla_inputs(B, H, G, S, DV, D - DV, dtype, seed=300 + n)
+        mod = _mla_engine(B, H, G, S, D, DV, dtype, scale)
+        out = mod(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda())
+        ref = torch.empty(B, H, DV)
+        lse = torch.empty(B, H)
+        hg = H // G
+        for g in range(G):      # the oracle takes one latent head at a time
+            r, l = R.mla_decode(q[:, 0, g * hg:(g + 1) * hg], q_pe[:, 0, g * hg:(g + 1) * hg], kv[:, :, g:g + 1],
+                                k_pe[:, :, g:g + 1], scale=scale)
+            ref[:, g * hg:(g + 1) * hg], lse[:, g * hg:(g + 1) * hg] = r, l
+        assert torch.isfinite(out).all()
+        assert (out[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL, (B, H, G, S)
+        assert (mod.final_rowscales["lse"][:, :, 0].cpu() - lse).abs().max().item() <= LSE_TOL, (B, H, G, S)

@@ -314,3 +314,33 @@ def test_small_and_odd_shapes_against_oracle(cuda_device):
         assert torch.isfinite(out).all()
         assert (out - ref).abs().max().item() <= OUT_TOL, (B, H, Hkv, S, D)
         assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL, (B, H, Hkv, S, D)
+
+
+def test_pipelined_kernel_odd_shapes_and_masks(cuda_device, monkeypatch):
+    """The software-pipelined kernel forced onto ragged shapes with elementwise masks (sliding window,
+    shifted causal, head dependent), grouped heads and both head dims, against the closed form with
+    the dense mask."""
+    import random
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    rng = random.Random(77)
+    masks = [None, C.causal_mask, C.make_sliding_window_mask(37), C.causal_shifted_mask, C.head_dependent_mask,
+             C.causal_plus_one_mask]
+    for n in range(12):
+        hkv = rng.choice([1, 2])
+        B, H, S, D = rng.choice([1, 2]), hkv * rng.choice([1, 2, 4]), rng.randint(1, 700), rng.choice([64, 128])
+        dtype = torch.float16 if n % 2 == 0 else torch.bfloat16
+        mask_mod = masks[n % len(masks)]
+        print(f"case pipelined odd B{B} H{H} Hkv{hkv} S{S} D{D} {dtype} mask {n % len(masks)}", flush=True)
+        q, k, v = C.make_inputs(B, S, S, H, hkv, D, D, dtype, seed=200 + n)
+        mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod, C.OnlineSoftmax(),
+                      Hkv=hkv)
+        assert mod._op.tiles.template == "ae_prefill_pipe.hip"
+        out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+        dense = _dense(mask_mod, B, H, S, S) if mask_mod is not None else None
+        ref, lse = R.softmax_attention(q, k, v, mask=dense)
+        got = mod.final_rowscales["lse"].cpu()
+        assert torch.isfinite(out).all()
+        assert (out - ref).abs().max().item() <= OUT_TOL, (B, H, S, D, n)
+        vis = torch.isfinite(lse)
+        assert torch.equal(torch.isfinite(got), vis)           # rows without a visible key: lse = -inf
+        assert (got[vis] - lse[vis]).abs().max().item() <= LSE_TOL, (B, H, S, D, n)
