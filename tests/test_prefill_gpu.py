@@ -344,3 +344,42 @@ def test_pipelined_kernel_odd_shapes_and_masks(cuda_device, monkeypatch):
         vis = torch.isfinite(lse)
         assert torch.equal(torch.isfinite(got), vis)           # rows without a visible key: lse = -inf
         assert (got[vis] - lse[vis]).abs().max().item() <= LSE_TOL, (B, H, S, D, n)
+
+
+def test_pipelined_kernel_scores_far_above_the_first_tiles(cuda_device, monkeypatch):
+    """Running maxima that keep moving: later keys score far above the first tiles' (for all rows, for the
+    rows of one wave only, growing slowly, and in one jump of three keys), so the lazy refresh of the
+    reference and the rescale of O outside the hot loop are taken many times, by some waves of a
+    workgroup and not by others.  (bf16 only where |out| stays small enough for the 2e-2 bar: a one-hot
+    softmax returns single rows of V, and bf16 rounds a value of 4 by 8e-3.)"""
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    B, H, S, D = 1, 2, 1536, 128
+    for dtype in (torch.float16, torch.bfloat16):
+        for case in ("all_rows", "one_wave", "slow_growth", "late_jump"):
+            if dtype == torch.bfloat16 and case in ("all_rows", "slow_growth"):
+                continue
+            for causal in (False, True):
+                print(f"case far-above {dtype} {case} causal={causal}", flush=True)
+                q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=31)
+                q, k = q.float(), k.float()
+                if case == "all_rows":
+                    k[:, S // 2:] *= 12.0
+                elif case == "one_wave":
+                    k[:, 700:] *= 3.0
+                    q[:, 832:896] *= 6.0              # rows of one wave of the q tile 768..1023
+                elif case == "slow_growth":
+                    k *= torch.linspace(1.0, 14.0, S).view(1, S, 1, 1)
+                else:
+                    k[:, 64 * 11: 64 * 11 + 3] *= 25.0
+                q, k = q.to(dtype), k.to(dtype)
+                mask_mod = C.causal_mask if causal else None
+                mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod,
+                              C.OnlineSoftmax())
+                assert mod._op.tiles.template == "ae_prefill_pipe.hip"
+                out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+                dense = _dense(mask_mod, B, H, S, S) if causal else None
+                ref, lse = R.softmax_attention(q, k, v, mask=dense)
+                got = mod.final_rowscales["lse"].cpu()
+                assert torch.isfinite(out).all(), (dtype, case, causal)
+                assert (out - ref).abs().max().item() <= OUT_TOL, (dtype, case, causal)
+                assert ((got - lse).abs() <= LSE_TOL + 2e-6 * lse.abs()).all(), (dtype, case, causal)
