@@ -171,6 +171,19 @@ class PrefillOp:
 
     # ---- launch ----------------------------------------------------------------------------
     def __call__(self, q, k, v, *extra):
+        """Forward; records the autograd edge when a gradient of q, k or v is wanted (the reference's
+        generated ``_attention`` autograd function, attn_tl.py:530-640)."""
+        if torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in (q, k, v)):
+            return _PrefillFunction.apply(self, q, k, v, *extra)
+        return self._forward(q, k, v, *extra)
+
+    def backward_op(self):
+        if getattr(self, "_bwd", None) is None:
+            from .prefill_bwd_op import PrefillBwdOp
+            self._bwd = PrefillBwdOp(self)
+        return self._bwd
+
+    def _forward(self, q, k, v, *extra):
         n_custom = len(self.functors.customs)
         extern_mask = None
         if len(extra) == n_custom + 1:
@@ -255,3 +268,23 @@ class PrefillOp:
         self.final_rowscales = dict(zip(self.functors.final_rowscale_names, rowscales))
         self._keepalive = keep
         return out
+
+
+class _PrefillFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, op, q, k, v, *extra):
+        # `extra`: the block mask the engine inferred from mask_mod, which it appends to every call (the
+        # backward applies mask_mod per element instead); custom inputs and external masks are refused
+        bwd = op.backward_op()                 # raises now if this graph has no backward
+        with torch.no_grad():
+            out = op._forward(q.detach(), k.detach(), v.detach(), *extra)
+        ctx.op = op
+        ctx.n_extra = len(extra)
+        ctx.save_for_backward(q, k, v, out, op.final_rowscales[bwd.lse_name])
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        dq, dk, dv = ctx.op.backward_op()(q, k, v, out, lse, dout)
+        return (None, dq, dk, dv) + (None,) * ctx.n_extra

@@ -65,6 +65,16 @@ class AttnParams(C.Structure):
     ]
 
 
+class AttnBwdParams(C.Structure):
+    """Mirror of ``ae_attn_bwd_params``."""
+    _fields_ = (
+        [(n, C.c_void_p) for n in ("q", "k", "v", "out", "dout", "lse", "delta", "dq", "dk", "dv")]
+        + [(f"{t}_stride_{a}", C.c_int64) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for a in "bsh"]
+        + [("batch", C.c_int32), ("heads_q", C.c_int32), ("heads_kv", C.c_int32),
+           ("seqlen_q", C.c_int32), ("seqlen_kv", C.c_int32), ("reserved", C.c_int32 * 3)]
+    )
+
+
 class TileCfg(C.Structure):
     """Mirror of ``ae_tile_cfg``."""
     _fields_ = [
@@ -110,6 +120,7 @@ _SIGNATURES = {
                                     C.POINTER(TileCfg), _VP]),
     "ae_prefill_split_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
                                        C.POINTER(TileCfg), _VP]),
+    "ae_prefill_bwd": (C.c_int, [_VP, _VP, _VP, C.POINTER(AttnBwdParams), C.POINTER(TileCfg), _VP]),
     "ae_event_create": (C.c_int, [C.POINTER(_VP)]),
     "ae_event_record": (C.c_int, [_VP, _VP]),
     "ae_event_elapsed_ms": (C.c_int, [_VP, _VP, C.POINTER(C.c_float)]),
@@ -326,3 +337,7 @@ def mla_decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: Tile
                    combine_cfg: TileCfg, stream: int = 0):
     _check(lib().ae_mla_decode_fwd(split.handle, combine.handle, C.byref(params), C.byref(cfg),
                                    C.byref(combine_cfg), _VP(stream)))
+
+
+def prefill_bwd(delta: Kernel, dkv: Kernel, dq: Kernel, params: AttnBwdParams, cfg: TileCfg, stream: int = 0):
+    _check(lib().ae_prefill_bwd(delta.handle, dkv.handle, dq.handle, C.byref(params), C.byref(cfg), _VP(stream)))

@@ -470,6 +470,41 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
   return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
 }
 
+int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
+                   const ae_tile_cfg* cfg, void* stream) {
+  if (!delta || !dkv || !dq) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: kernel is NULL");
+  if (!p || !cfg) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: params/cfg is NULL");
+  if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk ||
+      !p->dv)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: a tensor pointer is NULL");
+  if (p->batch <= 0 || p->heads_q <= 0 || p->heads_kv <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: non-positive extent (B=%d Hq=%d Hkv=%d Sq=%d Skv=%d)",
+                p->batch, p->heads_q, p->heads_kv, p->seqlen_q, p->seqlen_kv);
+  if (p->heads_q % p->heads_kv != 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: Hq=%d is not a multiple of Hkv=%d", p->heads_q,
+                p->heads_kv);
+  if (cfg->block_m != 128 || cfg->block_n != 64 || cfg->threads != 256 || cfg->lds_bytes <= 0 ||
+      cfg->lds_bytes > 160 * 1024 || cfg->head_dim_v <= 0 || cfg->head_dim_v % 8 != 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: bad tile configuration (bm=%d bn=%d threads=%d lds=%d dv=%d)",
+                cfg->block_m, cfg->block_n, cfg->threads, cfg->lds_bytes, cfg->head_dim_v);
+  const uint64_t rows = (uint64_t)p->batch * p->seqlen_q * p->heads_q;
+  const uint64_t rows_per_wg = 256u / (uint32_t)(cfg->head_dim_v / 8);
+  const uint64_t g_delta = (rows + rows_per_wg - 1) / rows_per_wg;
+  const uint64_t g_dkv = (((uint64_t)p->seqlen_kv + 127) / 128) * p->batch * p->heads_kv;
+  const uint64_t g_dq = (((uint64_t)p->seqlen_q + 127) / 128) * p->batch * p->heads_q;
+  if (g_delta > 0x7fffffffull || g_dkv > 0x7fffffffull || g_dq > 0x7fffffffull)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: grid too large");
+  uint32_t block[3] = {256, 1, 1};
+  uint32_t grid[3] = {(uint32_t)g_delta, 1, 1};
+  int rc = ae_launch(delta, p, sizeof *p, grid, block, 0, stream);
+  if (rc) return rc;
+  grid[0] = (uint32_t)g_dkv;
+  rc = ae_launch(dkv, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+  if (rc) return rc;
+  grid[0] = (uint32_t)g_dq;
+  return ae_launch(dq, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+}
+
 int ae_event_create(ae_event** out) {
   if (!out) return fail(AE_ERR_INVALID_ARG, "ae_event_create: out is NULL");
   *out = nullptr;

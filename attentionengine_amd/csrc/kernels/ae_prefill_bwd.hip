@@ -1,0 +1,390 @@
+// Backward of softmax attention (prefill shapes) for gfx950 / CDNA4: dQ, dK, dV from dO.
+//
+// Role of the reference's backward kernels for attn_script/mha.py
+// (attention_engine/core/template/tl_template/attn/attn_tl.py: flashattn_bwd_preprocess 196-221,
+// flashattn_bwd 238-420, flashattn_bwd_postprocess 422-455), for the graphs the lowering has proven
+// to be the online softmax of `score * constant`:
+//     p = exp(s*c - lse)                      (OnlineSoftmax.forward,  mha.py:75-78)
+//     dv = p^T do,  dp = do v^T
+//     ds = p * (dp - rowsum(do * o)) * c      (OnlineSoftmax.backward, mha.py:80-84; d score_mod = c)
+//     dq = ds k,  dk = ds^T q
+// The reference accumulates dq with fp32 atomics from the kernel that owns a kv tile and converts it
+// in a third kernel.  Here the work is split by OUTPUT instead, with no atomics and a fixed summation
+// order: one launch owns q rows and produces dq, one owns kv rows and produces dk and dv; both
+// recompute s and dp (7 tile products per tile pair instead of 5).  They are the same code with the
+// operands exchanged (AE_BWD_ROLE):
+//     role 0 (dq):      resident rows = q  (Q, dO in registers), streamed tiles = K, V
+//     role 1 (dk, dv):  resident rows = kv (K, V in registers),  streamed tiles = Q, dO of every q head
+//                       of the kv head's group, with their lse and rowsum(do * o)
+// A wave owns 32 resident rows as the B operand (n = row) of v_mfma_f32_32x32x16, so a lane owns ONE
+// resident row: S[streamed, resident] = X1 R1^T and dP = X2 R2^T come out with the streamed rows in
+// a lane's 16 accumulator registers, which makes the packed p and ds the B operand of the second
+// set of products, OUT^T[d, resident] += X^T[d, streamed] ds[streamed, resident], with X^T read from
+// the same LDS tile through ds_read_b64_tr_b16.  Streamed tiles (64 rows) are staged through LDS,
+// double buffered, with the pair swizzle of the forward kernels' V tile (transposed reads conflict
+// free, row reads two-way).
+//
+// Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0 none, 1 causal)
+// AE_HAS_MASK_MOD AE_SM_SCALE AE_BWD_ROLE.  Functors used ("ae_functors.h"): ae_mask_mod.
+
+#include "ae_hip.h"
+#include "ae_config.h"
+#include "ae_device.h"
+#include "ae_functors.h"
+
+#define AE_NWAVES 4
+#define AE_NT (AE_NWAVES * 64)
+#define AE_BR (AE_NWAVES * 32)     // resident rows per workgroup
+#define AE_BS 64                   // streamed rows per tile
+#define AE_STR1 (AE_D * 2)         // LDS row pitch of the first streamed tensor (K or Q), bytes
+#define AE_STR2 (AE_DV * 2)        // ... of the second (V or dO)
+#define AE_CPR1 (AE_D / 8)         // 16-byte chunks per row
+#define AE_CPR2 (AE_DV / 8)
+#define AE_T1_BYTES (AE_BS * AE_STR1)
+#define AE_T2_BYTES (AE_BS * AE_STR2)
+#define AE_STAGE_BYTES (AE_T1_BYTES + AE_T2_BYTES + 2 * AE_BS * 4)   // + lse, rowsum(do*o) of the streamed rows
+#define AE_NKS1 (AE_D / 16)        // k-steps of S
+#define AE_NKS2 (AE_DV / 16)       // k-steps of dP
+#define AE_NDB1 (AE_D / 32)        // 32-wide output blocks of dQ / dK
+#define AE_NDB2 (AE_DV / 32)       // ... of dV
+#define AE_L1 ((AE_BS * AE_CPR1) / AE_NT)   // 16-byte chunks a thread moves per tile
+#define AE_L2 ((AE_BS * AE_CPR2) / AE_NT)
+
+static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
+static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
+static_assert(AE_BWD_ROLE == 0 || AE_BWD_ROLE == 1, "role");
+static_assert(AE_MASK_MODE == 0 || AE_MASK_MODE == 1, "none or causal (an elementwise mask_mod on top)");
+
+typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
+typedef __attribute__((address_space(3))) float ae_lds_f32;
+
+// LDS position of 16-byte chunk c of row r: pairs of chunks are exchanged by the row's low bits
+template <int CPR>
+AE_DEV int ae_bwd_chunk_pos(int r, int c) {
+  return ((((c >> 1) ^ (r & (CPR / 2 - 1))) << 1) | (c & 1));
+}
+
+#if AE_BWD_ROLE == 0
+#define AE_BWD_KERNEL ae_bwd_dq_kernel
+#else
+#define AE_BWD_KERNEL ae_bwd_dkv_kernel
+#endif
+
+extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
+  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // two stages of [tile 1][tile 2][lse][delta]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int hf = lane >> 5;
+  const int group = p.heads_q / p.heads_kv;
+
+  // ---- which (resident tile, head, batch) --------------------------------------------------------
+#if AE_BWD_ROLE == 0
+  const int n_res = p.seqlen_q, n_str = p.seqlen_kv, heads = p.heads_q;
+#else
+  const int n_res = p.seqlen_kv, n_str = p.seqlen_q, heads = p.heads_kv;
+#endif
+  const int n_rt = (n_res + AE_BR - 1) / AE_BR;
+  const int rt = (int)(blockIdx.x % (unsigned)n_rt);
+  const int bh = (int)(blockIdx.x / (unsigned)n_rt);
+  if (bh >= p.batch * heads) return;
+  const int h = bh % heads;            // role 0: q head; role 1: kv head
+  const int b = bh / heads;
+  const int r0 = rt * AE_BR;
+  const int rrow = r0 + wave * 32 + l32;            // this lane's resident row
+  const bool r_ok = rrow < n_res;
+  const int rrow_c = r_ok ? rrow : n_res - 1;
+
+  // ---- resident operands: B[k = 16*ks + 8*hf + j][n = row] ---------------------------------------
+#if AE_BWD_ROLE == 0
+  const int hk = h / group;
+  const ae_elem* r1p = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)rrow_c * p.q_stride_s + (int64_t)h * p.q_stride_h;
+  const ae_elem* r2p = (const ae_elem*)p.dout + (int64_t)b * p.do_stride_b + (int64_t)rrow_c * p.do_stride_s + (int64_t)h * p.do_stride_h;
+#else
+  const int hk = h;
+  const ae_elem* r1p = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)rrow_c * p.k_stride_s + (int64_t)h * p.k_stride_h;
+  const ae_elem* r2p = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)rrow_c * p.v_stride_s + (int64_t)h * p.v_stride_h;
+#endif
+  ae_elem8 rf1[AE_NKS1], rf2[AE_NKS2];
+#pragma unroll
+  for (int ks = 0; ks < AE_NKS1; ks++) rf1[ks] = *(const ae_elem8*)(r1p + ks * 16 + hf * 8);
+#pragma unroll
+  for (int ks = 0; ks < AE_NKS2; ks++) rf2[ks] = *(const ae_elem8*)(r2p + ks * 16 + hf * 8);
+
+#if AE_BWD_ROLE == 0
+  // row scales of the lane's q row: lse in log2 units (+inf for a row without a visible key: p = 0)
+  float lse2_r, delta_r;
+  {
+    const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + rrow_c;
+    const float l = p.lse[ri];
+    lse2_r = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
+    delta_r = p.delta[ri];
+  }
+#endif
+
+  // ---- the streamed items --------------------------------------------------------------------------
+  // role 0: kv tiles 0 .. (causal: up to the diagonal); role 1: for every q head of the group, q tiles
+  // (causal: from the diagonal) .. last
+  const int n_st = (n_str + AE_BS - 1) / AE_BS;
+  int t_lo = 0, t_hi = n_st;
+#if AE_MASK_MODE == 1
+#if AE_BWD_ROLE == 0
+  {
+    const int lim = (r0 + AE_BR - 1) / AE_BS + 1;
+    t_hi = lim < n_st ? lim : n_st;
+  }
+#else
+  t_lo = r0 / AE_BS;
+  t_lo = t_lo < n_st ? t_lo : n_st;
+#endif
+#endif
+  const int n_t = t_hi - t_lo;
+#if AE_BWD_ROLE == 0
+  const int n_items = n_t;
+#else
+  const int n_items = n_t * group;
+#endif
+
+  // global -> register -> LDS staging: thread moves chunks ci = tid + 256*i of each tile
+  ae_elem8 buf1[AE_L1], buf2[AE_L2];
+  float buf_rs = 0.f;
+  auto item_tile = [&](int it) { return t_lo + (AE_BWD_ROLE == 0 ? it : it % n_t); };
+  auto item_head = [&](int it) { return AE_BWD_ROLE == 0 ? h : h * group + it / n_t; };   // q head of the item
+  auto load_item = [&](int it) {
+    const int s0 = item_tile(it) * AE_BS;
+#if AE_BWD_ROLE == 0
+    const ae_elem* x1 = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
+    const ae_elem* x2 = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
+    const int64_t st1 = p.k_stride_s, st2 = p.v_stride_s;
+#else
+    const int hq = item_head(it);
+    const ae_elem* x1 = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)hq * p.q_stride_h;
+    const ae_elem* x2 = (const ae_elem*)p.dout + (int64_t)b * p.do_stride_b + (int64_t)hq * p.do_stride_h;
+    const int64_t st1 = p.q_stride_s, st2 = p.do_stride_s;
+#endif
+#pragma unroll
+    for (int i = 0; i < AE_L1; i++) {
+      const int ci = tid + AE_NT * i;
+      int row = s0 + ci / AE_CPR1;
+      row = row < n_str ? row : n_str - 1;            // rows past the end re-read the last row (masked)
+      buf1[i] = *(const ae_elem8*)(x1 + (int64_t)row * st1 + (ci % AE_CPR1) * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < AE_L2; i++) {
+      const int ci = tid + AE_NT * i;
+      int row = s0 + ci / AE_CPR2;
+      row = row < n_str ? row : n_str - 1;
+      buf2[i] = *(const ae_elem8*)(x2 + (int64_t)row * st2 + (ci % AE_CPR2) * 8);
+    }
+#if AE_BWD_ROLE == 1
+    if (tid < 2 * AE_BS) {
+      int row = s0 + (tid & (AE_BS - 1));
+      row = row < n_str ? row : n_str - 1;
+      const int64_t ri = ((int64_t)b * p.heads_q + hq) * p.seqlen_q + row;
+      if (tid < AE_BS) {
+        const float l = p.lse[ri];
+        buf_rs = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
+      } else {
+        buf_rs = p.delta[ri];
+      }
+    }
+#endif
+  };
+  auto store_item = [&](int stage) {
+    ae_lds_byte* t1 = lds + stage * AE_STAGE_BYTES;
+    ae_lds_byte* t2 = t1 + AE_T1_BYTES;
+#pragma unroll
+    for (int i = 0; i < AE_L1; i++) {
+      const int ci = tid + AE_NT * i;
+      const int r = ci / AE_CPR1;
+      *(__attribute__((address_space(3))) ae_elem8*)(t1 + r * AE_STR1 + ae_bwd_chunk_pos<AE_CPR1>(r, ci % AE_CPR1) * 16) = buf1[i];
+    }
+#pragma unroll
+    for (int i = 0; i < AE_L2; i++) {
+      const int ci = tid + AE_NT * i;
+      const int r = ci / AE_CPR2;
+      *(__attribute__((address_space(3))) ae_elem8*)(t2 + r * AE_STR2 + ae_bwd_chunk_pos<AE_CPR2>(r, ci % AE_CPR2) * 16) = buf2[i];
+    }
+#if AE_BWD_ROLE == 1
+    if (tid < 2 * AE_BS) ((ae_lds_f32*)(t2 + AE_T2_BYTES))[tid] = buf_rs;
+#endif
+  };
+
+  // A operands out of a staged tile.  Row fragment: A[m = row 32*nb + lane%32][k = 16*ks + 8*hf + j].
+  auto row_frag1 = [&](const ae_lds_byte* t, int nb, int ks) -> ae_elem8 {
+    const int r = nb * 32 + l32;
+    return *(const __attribute__((address_space(3))) ae_elem8*)(t + r * AE_STR1 + ae_bwd_chunk_pos<AE_CPR1>(r, 2 * ks + hf) * 16);
+  };
+  auto row_frag2 = [&](const ae_lds_byte* t, int nb, int ks) -> ae_elem8 {
+    const int r = nb * 32 + l32;
+    return *(const __attribute__((address_space(3))) ae_elem8*)(t + r * AE_STR2 + ae_bwd_chunk_pos<AE_CPR2>(r, 2 * ks + hf) * 16);
+  };
+  // Transposed fragment: A[m = column 32*db + ..][k = the 16 rows of k-step kk], in the row order in which
+  // a lane's accumulator registers hold the rows (see the forward kernels' V^T fragment).
+  const int t_row = 4 * hf + ((lane & 15) >> 2);
+  const int t_g = l32 >> 4;
+  auto tr_frag = [&](const ae_lds_byte* t, int str, int ppr, int kk, int db) -> ae_elem8 {
+    const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
+    const int r_lo = rb0 + t_row;
+    const ae_lds_byte* a0 = t + r_lo * str + (lane & 3) * 8 + (((2 * db + t_g) ^ (t_row & (ppr - 1))) << 5);
+    ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)a0);
+    ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)(a0 + 8 * str));
+    return __builtin_bit_cast(ae_elem8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  ae_f32x16 acc1[AE_NDB1];            // dQ^T (role 0) / dK^T (role 1): [d][resident row]
+#pragma unroll
+  for (int db = 0; db < AE_NDB1; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc1[db][r] = 0.f;
+#if AE_BWD_ROLE == 1
+  ae_f32x16 acc2[AE_NDB2];            // dV^T
+#pragma unroll
+  for (int db = 0; db < AE_NDB2; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc2[db][r] = 0.f;
+#endif
+
+  if (n_items > 0) {
+    load_item(0);
+    store_item(0);
+  }
+  __syncthreads();
+
+  for (int it = 0; it < n_items; it++) {
+    const bool more = it + 1 < n_items;
+    if (more) load_item(it + 1);
+    const ae_lds_byte* t1 = lds + (it & 1) * AE_STAGE_BYTES;
+    const ae_lds_byte* t2 = t1 + AE_T1_BYTES;
+    const int s0 = item_tile(it) * AE_BS;
+
+    // S = X1 R1^T and dP = X2 R2^T: [streamed row][resident row]
+    ae_f32x16 sacc[2], pacc[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) sacc[nb][r] = pacc[nb][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS1; ks++) sacc[nb] = ae_mfma32(row_frag1(t1, nb, ks), rf1[ks], sacc[nb]);
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS2; ks++) pacc[nb] = ae_mfma32(row_frag2(t2, nb, ks), rf2[ks], pacc[nb]);
+    }
+
+    // p and ds, packed as B operands: k-step kk holds the lane's elements 8*kk .. 8*kk+7
+    ae_elem8 pf[4], dsf[4];
+#if AE_BWD_ROLE == 1
+    const ae_lds_f32* rs_l = (const ae_lds_f32*)(t2 + AE_T2_BYTES);
+    const int hq = item_head(it);
+#else
+    const int hq = h;
+#endif
+#pragma unroll
+    for (int e = 0; e < 32; e++) {
+      const int nb = e >> 4, r = e & 15;
+      const int sl = nb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);     // streamed row inside the tile
+      const int srow = s0 + sl;
+#if AE_BWD_ROLE == 0
+      const int qi = rrow, ki = srow;
+      const float l2 = lse2_r, dl = delta_r;
+#else
+      const int qi = srow, ki = rrow;
+      const float l2 = rs_l[sl], dl = rs_l[AE_BS + sl];
+#endif
+      bool vis = r_ok && srow < n_str;
+#if AE_MASK_MODE == 1
+      vis = vis && qi >= ki;
+#endif
+#if AE_HAS_MASK_MOD
+      vis = vis && ae_mask_mod(b, hq, qi, ki);
+#endif
+      const float pv = vis ? ae_exp2(__builtin_fmaf(sacc[nb][r], AE_SM_SCALE * AE_LOG2E, -l2)) : 0.f;
+      const float dsv = pv * (pacc[nb][r] - dl) * AE_SM_SCALE;
+      pf[e >> 3][e & 7] = (ae_elem)pv;
+      dsf[e >> 3][e & 7] = (ae_elem)dsv;
+    }
+    (void)hq;
+
+    // OUT^T[d][resident] += X^T[d][streamed] ds[streamed][resident]
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) {
+#pragma unroll
+      for (int db = 0; db < AE_NDB1; db++)
+        acc1[db] = ae_mfma32(tr_frag(t1, AE_STR1, AE_CPR1 / 2, kk, db), dsf[kk], acc1[db]);
+#if AE_BWD_ROLE == 1
+#pragma unroll
+      for (int db = 0; db < AE_NDB2; db++)
+        acc2[db] = ae_mfma32(tr_frag(t2, AE_STR2, AE_CPR2 / 2, kk, db), pf[kk], acc2[db]);
+#endif
+    }
+    (void)pf;
+
+    if (more) store_item((it + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- results: lane owns its resident row, columns 32*db + 8*(r/4) + 4*hf + r%4 ------------------
+  if (r_ok) {
+#if AE_BWD_ROLE == 0
+    ae_elem* o1 = (ae_elem*)p.dq + (int64_t)b * p.dq_stride_b + (int64_t)rrow * p.dq_stride_s + (int64_t)h * p.dq_stride_h;
+#else
+    ae_elem* o1 = (ae_elem*)p.dk + (int64_t)b * p.dk_stride_b + (int64_t)rrow * p.dk_stride_s + (int64_t)h * p.dk_stride_h;
+    ae_elem* o2 = (ae_elem*)p.dv + (int64_t)b * p.dv_stride_b + (int64_t)rrow * p.dv_stride_s + (int64_t)h * p.dv_stride_h;
+#endif
+#pragma unroll
+    for (int db = 0; db < AE_NDB1; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        ae_elem4 w;
+#pragma unroll
+        for (int t = 0; t < 4; t++) w[t] = (ae_elem)acc1[db][rg * 4 + t];
+        *(ae_elem4*)(o1 + db * 32 + rg * 8 + hf * 4) = w;
+      }
+#if AE_BWD_ROLE == 1
+#pragma unroll
+    for (int db = 0; db < AE_NDB2; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        ae_elem4 w;
+#pragma unroll
+        for (int t = 0; t < 4; t++) w[t] = (ae_elem)acc2[db][rg * 4 + t];
+        *(ae_elem4*)(o2 + db * 32 + rg * 8 + hf * 4) = w;
+      }
+#endif
+  }
+}
+
+#if AE_BWD_ROLE == 0
+// rowsum(do * o), fp32 [B,Hq,Sq]: the `doosum` row scale of the reference's backward
+// (flashattn_bwd_preprocess, attn_tl.py:196-221).  DV/8 lanes share a row, 16 bytes each.
+extern "C" __global__ __launch_bounds__(256)
+void ae_bwd_delta_kernel(const ae_attn_bwd_params p) {
+  constexpr int LPR = AE_DV / 8;                   // lanes per row
+  constexpr int RPB = 256 / LPR;                   // rows per workgroup
+  const int tid = threadIdx.x;
+  const int64_t n_rows = (int64_t)p.batch * p.seqlen_q * p.heads_q;
+  const int64_t row = (int64_t)blockIdx.x * RPB + tid / LPR;
+  const int c = tid % LPR;
+  float acc = 0.f;
+  int b = 0, s = 0, h = 0;
+  if (row < n_rows) {
+    h = (int)(row % p.heads_q);
+    s = (int)((row / p.heads_q) % p.seqlen_q);
+    b = (int)(row / ((int64_t)p.heads_q * p.seqlen_q));
+    const ae_elem8 o = *(const ae_elem8*)((const ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)s * p.o_stride_s + (int64_t)h * p.o_stride_h + c * 8);
+    const ae_elem8 d = *(const ae_elem8*)((const ae_elem*)p.dout + (int64_t)b * p.do_stride_b + (int64_t)s * p.do_stride_s + (int64_t)h * p.do_stride_h + c * 8);
+#pragma unroll
+    for (int j = 0; j < 8; j++) acc += (float)o[j] * (float)d[j];
+  }
+  // the LPR lanes of a row are consecutive and aligned: butterfly inside the group
+#pragma unroll
+  for (int m = 1; m < LPR; m <<= 1) {
+    const int lane = tid & 63;
+    acc += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ m) << 2, __builtin_bit_cast(int, acc)));
+  }
+  if (row < n_rows && c == 0) p.delta[((int64_t)b * p.heads_q + h) * p.seqlen_q + s] = acc;
+}
+#endif

@@ -49,7 +49,7 @@ using __hip_internal::uint64_t;
 extern "C" {
 #endif
 
-#define AE_ABI_VERSION 1
+#define AE_ABI_VERSION 2
 
 typedef enum ae_status {
   AE_OK = 0,
@@ -113,6 +113,36 @@ typedef struct ae_tile_cfg {
   int32_t mask_mode;   /* 0 none, 1 analytic causal, 2 block table                        */
   int32_t reserved[3];
 } ae_tile_cfg;
+
+/*
+ * Kernel argument block of the backward kernels (softmax attention, prefill shapes). Same layouts as
+ * ae_attn_params; dout [B,Sq,Hq,DV] is the gradient of `out`, dq/dk/dv have the shapes of q/k/v, lse
+ * is the forward's natural-log row scale fp32 [B,Hq,Sq], delta a caller-allocated fp32 [B,Hq,Sq]
+ * work buffer that receives rowsum(dout * out). Stands where the reference passes Q, K, V, dO, lse
+ * and Delta to flashattn_bwd (core/template/tl_template/attn/attn_tl.py:271-295).
+ */
+typedef struct ae_attn_bwd_params {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const void* dout;
+  const float* lse;
+  float* delta;
+  void* dq;
+  void* dk;
+  void* dv;
+  int64_t q_stride_b, q_stride_s, q_stride_h;
+  int64_t k_stride_b, k_stride_s, k_stride_h;
+  int64_t v_stride_b, v_stride_s, v_stride_h;
+  int64_t o_stride_b, o_stride_s, o_stride_h;
+  int64_t do_stride_b, do_stride_s, do_stride_h;
+  int64_t dq_stride_b, dq_stride_s, dq_stride_h;
+  int64_t dk_stride_b, dk_stride_s, dk_stride_h;
+  int64_t dv_stride_b, dv_stride_s, dv_stride_h;
+  int32_t batch, heads_q, heads_kv, seqlen_q, seqlen_kv;
+  int32_t reserved[3];
+} ae_attn_bwd_params;
 
 typedef struct ae_devinfo {
   char name[128];
@@ -208,6 +238,18 @@ int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_par
  */
 int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                       const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
+
+/*
+ * ae_prefill_bwd: backward of softmax attention. Three launches on `stream`: `delta`
+ *   (rowsum(dout*out), the reference's flashattn_bwd_preprocess, attn_tl.py:196-221), `dkv` (one
+ *   workgroup per 128 kv rows of a (batch, kv head): dk and dv, summed over the q heads of the group)
+ *   and `dq` (one workgroup per 128 q rows of a (batch, q head)). The reference's single backward
+ *   kernel with fp32 atomics on dq and its postprocess (attn_tl.py:238-455) are replaced by these two
+ *   atomic-free launches. cfg: block_m = 128, block_n = 64, threads = 256 and the dynamic LDS of the
+ *   compiled kernels; head dims as compiled. All gradients are written in full (no accumulation).
+ */
+int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
+                   const ae_tile_cfg* cfg, void* stream);
 
 /* ---- timing on the launch stream ------------------------------------------------- */
 int ae_event_create(ae_event** out);

@@ -68,6 +68,40 @@ def softmax_attention(q, k, v, scale=None, causal=False, mask=None, compute_dtyp
     return out, lse.reshape(B, Hq, Sq)
 
 
+def softmax_attention_grads(q, k, v, do, scale=None, causal=False, mask=None, compute_dtype=torch.float32):
+    """Gradients (dq, dk, dv) of ``softmax_attention`` for the output gradient ``do`` [B,Sq,Hq,DV].
+
+    Restates the backward the reference generates for attn_script/mha.py: recompute
+    p = exp(s*scale - lse) (OnlineSoftmax.forward, mha.py:75-78), dv = p^T do, dp = do v^T,
+    ds = p * (dp - rowsum(do * o)) (OnlineSoftmax.backward, mha.py:80-84, with the
+    ``doosum`` row scale of flashattn_bwd_preprocess, attn_tl.py:196-221), score_mod's derivative
+    (the constant ``scale``), dq = ds k, dk = ds^T q (attn_tl.py:330-420); grouped heads sum into their
+    kv head.  Pinned in tests/test_oracle.py against torch.autograd through ``softmax_attention``.
+    """
+    B, Sq, Hq, D = q.shape
+    Skv, Hkv = k.shape[1], k.shape[2]
+    G = Hq // Hkv
+    scale = 1.0 / math.sqrt(D) if scale is None else scale
+    s = _grouped_scores(q, k, compute_dtype)
+    vis = torch.ones(B, Hkv, G, Sq, Skv, dtype=torch.bool)
+    if causal:
+        vis = vis & torch.ones(Sq, Skv, dtype=torch.bool).tril()
+    if mask is not None:
+        vis = vis & _mask_to_grouped(mask, B, Hkv, G, Sq, Skv)
+    s = s.masked_fill(~vis, float("-inf")) * scale
+    lse = torch.logsumexp(s, dim=-1, keepdim=True)
+    p = torch.where(torch.isfinite(lse), torch.exp(s - lse.clamp(min=-3.0e38)), torch.zeros_like(s))
+    dog = do.to(compute_dtype).reshape(B, Sq, Hkv, G, -1)                 # [B,Sq,Hkv,G,DV]
+    vf = v.to(compute_dtype)
+    dv = torch.einsum("bhgst,bshgd->bthd", p, dog)
+    dp = torch.einsum("bshgd,bthd->bhgst", dog, vf)
+    delta = (dp * p).sum(-1, keepdim=True)                                 # = rowsum(do * o)
+    ds = p * (dp - delta) * scale
+    dq = torch.einsum("bhgst,bthd->bshgd", ds, k.to(compute_dtype)).reshape(B, Sq, Hq, D)
+    dk = torch.einsum("bhgst,bshgd->bthd", ds, q.to(compute_dtype).reshape(B, Sq, Hkv, G, D))
+    return dq, dk, dv
+
+
 def sigmoid_attention(q, k, v, scale=None, bias=0.0, causal=False, compute_dtype=torch.float32):
     """out = sum_kv sigmoid(QK^T * scale + bias) V, no normalisation.
 

@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in ae_hip.h but not exported"
     assert sorted(rt.EXPORTED_SYMBOLS) == names
-    assert rt.lib().ae_abi_version() == 1
+    assert rt.lib().ae_abi_version() == 2
 
 
 def test_struct_layout_matches_the_header():
@@ -41,6 +41,8 @@ def test_struct_layout_matches_the_header():
     # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints
     assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16
     assert ctypes.sizeof(rt.TileCfg) == 4 * 12
+    # backward: 10 pointers, 8 tensors x 3 strides, 5 + 3 ints
+    assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 10 + 8 * 24 + 4 * 8
 
 
 def _compile(src, opts=()):

@@ -224,3 +224,23 @@ def test_retention_closed_form_loops_and_running_form():
                                    custom_fwd_inputs=C.retention_custom_inputs(), custom_tensors=(mask,),
                                    block_n=bn, mask_value="0")
         assert torch.allclose(o2, out, atol=1e-12) and torch.allclose(fin["r"], r, atol=1e-12)
+
+
+def test_softmax_gradients_match_autograd():
+    """The closed-form backward against torch.autograd through the closed-form forward (fp64), with
+    grouped heads, causal and an arbitrary mask with one fully masked row."""
+    g = torch.Generator().manual_seed(5)
+    B, Sq, Skv, Hq, Hkv, D, DV = 2, 9, 13, 4, 2, 8, 6
+    q = torch.randn(B, Sq, Hq, D, generator=g, dtype=torch.float64, requires_grad=True)
+    k = torch.randn(B, Skv, Hkv, D, generator=g, dtype=torch.float64, requires_grad=True)
+    v = torch.randn(B, Skv, Hkv, DV, generator=g, dtype=torch.float64, requires_grad=True)
+    do = torch.randn(B, Sq, Hq, DV, generator=g, dtype=torch.float64)
+    mask = torch.rand(B, Hq, Sq, Skv, generator=g) > 0.3
+    mask[0, 1, 4] = False
+    for kw in (dict(), dict(causal=True), dict(mask=mask), dict(scale=0.37, causal=True)):
+        out, _ = R.softmax_attention(q, k, v, compute_dtype=torch.float64, **kw)
+        gq, gk, gv = torch.autograd.grad(out, (q, k, v), do)
+        dq, dk, dv = R.softmax_attention_grads(q.detach(), k.detach(), v.detach(), do,
+                                               compute_dtype=torch.float64, **kw)
+        for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+            assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)

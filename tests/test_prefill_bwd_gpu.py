@@ -1,0 +1,88 @@
+"""GPU parity of the backward of softmax attention: dq, dk, dv from libae_hip.so (through
+AttentionEngine and torch.autograd) against the CPU oracle's closed-form gradients on the same seeded
+inputs.  The oracle consumes the fp16/bf16-rounded inputs and computes in fp32; a gradient element may
+differ by 2e-2 + 1% of the largest magnitude of that gradient (the kernels round p and ds to the input
+type before the second products and the results to the input type)."""
+import math
+
+import pytest
+import torch
+
+import attn_cases as C
+from attn_engine import AttentionEngine
+from core import CustomIO, meta_tensor
+from oracle import attention_ref as R
+from oracle import masks as M
+
+pytestmark = pytest.mark.gpu
+
+
+def _engine(B, H, Hkv, S, D, DV, dtype, mask_mod, scale):
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+            meta_tensor(B, Hkv, S, DV, dtype=dtype))
+    return AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(scale), mask_mod=mask_mod,
+                           online_func=C.OnlineSoftmax())
+
+
+def _check(got, ref, what, case):
+    tol = 2e-2 + 1e-2 * ref.abs().max().item()
+    err = (got.float().cpu() - ref).abs().max().item()
+    assert math.isfinite(err) and err <= tol, (what, case, err, tol)
+
+
+def _run(B, H, Hkv, Sq, Skv, D, DV, dtype, mask_mod, causal, seed=3):
+    scale = 1 / math.sqrt(D)
+    q, k, v = C.make_inputs(B, Sq, Skv, H, Hkv, D, DV, dtype, seed=seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    do = torch.randn(B, Sq, H, DV, generator=g).to(dtype)
+    mod = _engine(B, H, Hkv, Sq, D, DV, dtype, mask_mod, scale)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = mod(qd, kd, vd)
+    out.backward(do.cuda())
+    dense = None
+    if mask_mod is not None and not causal:
+        dense = torch.from_numpy(M.dense_mask_grid(mask_mod, B, H, Sq, Skv))
+    ref_out, _ = R.softmax_attention(q, k, v, scale=scale, causal=causal, mask=dense)
+    assert (out.detach().float().cpu() - ref_out).abs().max().item() <= 2e-2
+    dq, dk, dv = R.softmax_attention_grads(q, k, v, do, scale=scale, causal=causal, mask=dense)
+    case = (B, H, Hkv, Sq, Skv, D, DV, dtype, causal)
+    _check(qd.grad, dq, "dq", case)
+    _check(kd.grad, dk, "dk", case)
+    _check(vd.grad, dv, "dv", case)
+    assert qd.grad.dtype == dtype and kd.grad.shape == k.shape and vd.grad.shape == v.shape
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,Hkv,S,D,dtype", [
+    (1, 2, 2, 256, 128, torch.float16),
+    (2, 4, 4, 512, 64, torch.float16),
+    (1, 2, 2, 384, 128, torch.bfloat16),
+    (1, 4, 2, 320, 128, torch.float16),      # grouped heads: dk, dv sum over the group
+    (1, 2, 1, 200, 64, torch.bfloat16),      # ragged: S not a multiple of any tile
+    (1, 1, 1, 77, 128, torch.float16),
+])
+def test_softmax_backward(cuda_device, B, H, Hkv, S, D, dtype, causal):
+    print(f"case bwd B{B} H{H} Hkv{Hkv} S{S} D{D} {dtype} causal={causal}", flush=True)
+    _run(B, H, Hkv, S, S, D, D, dtype, C.causal_mask if causal else None, causal)
+
+
+def test_softmax_backward_elementwise_mask_and_dv(cuda_device):
+    """A mask that is not causal is applied per element (sliding window: rows see 37 keys), and the
+    value head dim may differ from the key head dim."""
+    print("case bwd sliding window", flush=True)
+    _run(1, 2, 2, 300, 300, 128, 128, torch.float16, C.make_sliding_window_mask(37), False)
+    print("case bwd D128 DV64", flush=True)
+    _run(1, 2, 1, 256, 256, 128, 64, torch.float16, C.causal_mask, True)
+    print("case bwd D64 DV128", flush=True)
+    _run(2, 2, 2, 130, 130, 64, 128, torch.bfloat16, None, False)
+
+
+def test_backward_of_other_graphs_is_refused(cuda_device):
+    """Only graphs proven to be softmax attention have a backward; the others say so."""
+    B, H, S, D = 1, 2, 128, 64
+    meta = (meta_tensor(B, H, S, D, dtype=torch.float16),) * 3
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(0.125), mask_mod=None,
+                          online_func=C.OnlineIdentity())
+    q, k, v = (t.cuda().requires_grad_(True) for t in C.make_inputs(B, S, S, H, H, D, D, torch.float16))
+    with pytest.raises(NotImplementedError):
+        mod(q, k, v)
