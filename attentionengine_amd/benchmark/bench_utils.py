@@ -10,7 +10,7 @@ is the reference's own eager fallback (1250-1275: grouped einsum, ``tril`` mask 
 ``softmax(scores * scale)``, einsum), run on the GPU with torch.
 
 Not carried over: the external-library baselines (flash_attn, FA3, flash_sigmoid, flashinfer) --
-not installable here -- and everything backward: ``require_grad=True`` is accepted, the backward
+not installable here.  Backward exists for softmax attention (``do_bench_attention``); for the other graphs ``require_grad=True`` is accepted, the backward
 timing is skipped with a note.
 """
 from __future__ import annotations
@@ -129,29 +129,56 @@ def _report(name, latency_ms, flops):
 def do_bench_attention(attn, B, H, S, D, DV, mod=None, dtype=torch.float16, seqlenq=None,
                        require_grad=False, causal=True, groupnum=None):
     """Softmax attention (MHA / GQA / decode): correctness print-out against the eager reference,
-    then forward timing.  Returns (latency_ms, tflops, latency_ref_ms, tflops_ref)."""
+    then forward timing; with ``require_grad`` also dq/dk/dv against autograd through the eager
+    reference and backward timing (bench_utils.py:1179-1360; backward flops 4*B*H*S^2*DV + 6*B*H*S^2*D,
+    halved when causal, 1199-1201).  Returns (latency_ms, tflops, latency_ref_ms, tflops_ref)."""
     seqlenq = S if seqlenq is None else seqlenq
     groupnum = H if groupnum is None else groupnum
     tflops = 2 * B * H * seqlenq * S * D + 2 * B * H * seqlenq * S * DV
     tflops = tflops * 0.5 if causal else tflops
+    bwd_tflops = (4 * B * H * seqlenq * S * DV + 6 * B * H * seqlenq * S * D) * (0.5 if causal else 1.0)
     torch.cuda.manual_seed(0)
     device = "cuda"
-    query = torch.randn(B, seqlenq, H, D, device=device, dtype=dtype)
-    key = torch.randn(B, S, groupnum, D, device=device, dtype=dtype)
-    value = torch.randn(B, S, groupnum, DV, device=device, dtype=dtype)
-    torch.randn(B, seqlenq, H, DV, device=device, dtype=dtype)  # `do` of the reference: keeps the RNG stream aligned
+    query = torch.randn(B, seqlenq, H, D, device=device, dtype=dtype, requires_grad=require_grad)
+    key = torch.randn(B, S, groupnum, D, device=device, dtype=dtype, requires_grad=require_grad)
+    value = torch.randn(B, S, groupnum, DV, device=device, dtype=dtype, requires_grad=require_grad)
+    do = torch.randn(B, seqlenq, H, DV, device=device, dtype=dtype)
 
     o = attn(query, key, value)
-    if require_grad:
-        print("forward-only build: backward check and timing skipped")
     scale = (1 / D) ** 0.5
-    o_ref = _eager_attention(query, key, value, scale, causal)
+    if require_grad:
+        o.backward(do, retain_graph=True)
+        dQ, dK, dV = query.grad.clone(), key.grad.clone(), value.grad.clone()
+        query.grad = key.grad = value.grad = None
+    with torch.no_grad():
+        o_ref = _eager_attention(query, key, value, scale, causal)
     print_debug(o, o_ref)
+    if require_grad:
+        # autograd through the eager reference, one (batch, head) group at a time (the full score
+        # tensor of the headline shape does not fit twice)
+        gq, gk, gv = torch.zeros_like(query), torch.zeros_like(key), torch.zeros_like(value)
+        g = H // groupnum
+        for b0 in range(B):
+            for h0 in range(groupnum):
+                qs = query[b0:b0 + 1, :, h0 * g:(h0 + 1) * g].detach().float().requires_grad_(True)
+                ks = key[b0:b0 + 1, :, h0:h0 + 1].detach().float().requires_grad_(True)
+                vs = value[b0:b0 + 1, :, h0:h0 + 1].detach().float().requires_grad_(True)
+                _eager_attention(qs, ks, vs, scale, causal).backward(do[b0:b0 + 1, :, h0 * g:(h0 + 1) * g].float())
+                gq[b0:b0 + 1, :, h0 * g:(h0 + 1) * g] = qs.grad.to(dtype)
+                gk[b0:b0 + 1, :, h0:h0 + 1] = ks.grad.to(dtype)
+                gv[b0:b0 + 1, :, h0:h0 + 1] = vs.grad.to(dtype)
+        print_debug(dQ, gq)
+        print_debug(dK, gk)
+        print_debug(dV, gv)
 
-    latency = do_bench(lambda: attn(query, key, value), warmup=50, rep=100)
-    _report("hip", latency, tflops)
-    latency_ref = do_bench(lambda: _eager_attention(query, key, value, scale, causal), warmup=50, rep=100)
-    _report("eager torch", latency_ref, tflops)
+    with torch.no_grad():
+        latency = do_bench(lambda: attn(query, key, value), warmup=50, rep=100)
+        _report("hip", latency, tflops)
+        latency_ref = do_bench(lambda: _eager_attention(query, key, value, scale, causal), warmup=50, rep=100)
+        _report("eager torch", latency_ref, tflops)
+    if require_grad:
+        latency_bwd = do_bench(lambda: o.backward(do, retain_graph=True), warmup=50, rep=100)
+        _report("hip bwd", latency_bwd, bwd_tflops)
     return latency, tflops / latency * 1e-9, latency_ref, tflops / latency_ref * 1e-9
 
 

@@ -490,8 +490,9 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
   const uint64_t rows = (uint64_t)p->batch * p->seqlen_q * p->heads_q;
   const uint64_t rows_per_wg = 256u / (uint32_t)(cfg->head_dim_v / 8);
   const uint64_t g_delta = (rows + rows_per_wg - 1) / rows_per_wg;
-  const uint64_t g_dkv = (((uint64_t)p->seqlen_kv + 127) / 128) * p->batch * p->heads_kv;
-  const uint64_t g_dq = (((uint64_t)p->seqlen_q + 127) / 128) * p->batch * p->heads_q;
+  // ids are 8*slot + xcd, slot = tile*ceil(batch*heads/8) + head group (see ae_prefill_bwd.hip)
+  const uint64_t g_dkv = (((uint64_t)p->seqlen_kv + 127) / 128) * ((((uint64_t)p->batch * p->heads_kv) + 7) / 8) * 8;
+  const uint64_t g_dq = (((uint64_t)p->seqlen_q + 127) / 128) * ((((uint64_t)p->batch * p->heads_q) + 7) / 8) * 8;
   if (g_delta > 0x7fffffffull || g_dkv > 0x7fffffffull || g_dq > 0x7fffffffull)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: grid too large");
   uint32_t block[3] = {256, 1, 1};

@@ -88,10 +88,21 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #else
   const int n_res = p.seqlen_kv, n_str = p.seqlen_q, heads = p.heads_kv;
 #endif
+  // ids are dealt round-robin to the 8 XCDs (each with its own L2): id = 8*slot + xcd keeps all resident
+  // tiles of one (batch, head) on ONE XCD, where they share the streamed tiles, and the slots go tile by
+  // tile across the heads, under a causal mask the tile with the most work first (the last q rows for
+  // dq, the first kv rows for dk/dv).  The grid is padded to 8*ceil(batch*heads/8)*tiles ids.
   const int n_rt = (n_res + AE_BR - 1) / AE_BR;
-  const int rt = (int)(blockIdx.x % (unsigned)n_rt);
-  const int bh = (int)(blockIdx.x / (unsigned)n_rt);
-  if (bh >= p.batch * heads) return;
+  const int n_bh = p.batch * heads;
+  const int n_bg = (n_bh + 7) >> 3;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int bh = (slot % n_bg) * 8 + xcd;
+#if AE_BWD_ROLE == 0 && AE_MASK_MODE == 1
+  const int rt = n_rt - 1 - slot / n_bg;
+#else
+  const int rt = slot / n_bg;
+#endif
+  if (bh >= n_bh) return;
   const int h = bh % heads;            // role 0: q head; role 1: kv head
   const int b = bh / heads;
   const int r0 = rt * AE_BR;
@@ -149,12 +160,19 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   const int n_items = n_t * group;
 #endif
 
-  // global -> register -> LDS staging: thread moves chunks ci = tid + 256*i of each tile
-  ae_elem8 buf1[AE_L1], buf2[AE_L2];
-  float buf_rs = 0.f;
+  // global -> register -> LDS staging: thread moves chunks ci = tid + 256*i of each tile.  Two register
+  // sets: a tile is requested three iterations before it is multiplied and written to LDS one iteration
+  // before, so a request has two iterations to land (one was not enough once the workgroups of a head
+  // had drifted apart and their tiles came from beyond the L2).
+  struct ae_stage_regs {
+    ae_elem8 b1[AE_L1], b2[AE_L2];
+    float rs;
+  };
+  ae_stage_regs sa, sb;
+  sa.rs = sb.rs = 0.f;
   auto item_tile = [&](int it) { return t_lo + (AE_BWD_ROLE == 0 ? it : it % n_t); };
   auto item_head = [&](int it) { return AE_BWD_ROLE == 0 ? h : h * group + it / n_t; };   // q head of the item
-  auto load_item = [&](int it) {
+  auto load_item = [&](int it, ae_stage_regs& sr) {
     const int s0 = item_tile(it) * AE_BS;
 #if AE_BWD_ROLE == 0
     const ae_elem* x1 = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
@@ -171,14 +189,14 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       const int ci = tid + AE_NT * i;
       int row = s0 + ci / AE_CPR1;
       row = row < n_str ? row : n_str - 1;            // rows past the end re-read the last row (masked)
-      buf1[i] = *(const ae_elem8*)(x1 + (int64_t)row * st1 + (ci % AE_CPR1) * 8);
+      sr.b1[i] = *(const ae_elem8*)(x1 + (int64_t)row * st1 + (ci % AE_CPR1) * 8);
     }
 #pragma unroll
     for (int i = 0; i < AE_L2; i++) {
       const int ci = tid + AE_NT * i;
       int row = s0 + ci / AE_CPR2;
       row = row < n_str ? row : n_str - 1;
-      buf2[i] = *(const ae_elem8*)(x2 + (int64_t)row * st2 + (ci % AE_CPR2) * 8);
+      sr.b2[i] = *(const ae_elem8*)(x2 + (int64_t)row * st2 + (ci % AE_CPR2) * 8);
     }
 #if AE_BWD_ROLE == 1
     if (tid < 2 * AE_BS) {
@@ -187,30 +205,30 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       const int64_t ri = ((int64_t)b * p.heads_q + hq) * p.seqlen_q + row;
       if (tid < AE_BS) {
         const float l = p.lse[ri];
-        buf_rs = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
+        sr.rs = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
       } else {
-        buf_rs = p.delta[ri];
+        sr.rs = p.delta[ri];
       }
     }
 #endif
   };
-  auto store_item = [&](int stage) {
+  auto store_item = [&](int stage, const ae_stage_regs& sr) {
     ae_lds_byte* t1 = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* t2 = t1 + AE_T1_BYTES;
 #pragma unroll
     for (int i = 0; i < AE_L1; i++) {
       const int ci = tid + AE_NT * i;
       const int r = ci / AE_CPR1;
-      *(__attribute__((address_space(3))) ae_elem8*)(t1 + r * AE_STR1 + ae_bwd_chunk_pos<AE_CPR1>(r, ci % AE_CPR1) * 16) = buf1[i];
+      *(__attribute__((address_space(3))) ae_elem8*)(t1 + r * AE_STR1 + ae_bwd_chunk_pos<AE_CPR1>(r, ci % AE_CPR1) * 16) = sr.b1[i];
     }
 #pragma unroll
     for (int i = 0; i < AE_L2; i++) {
       const int ci = tid + AE_NT * i;
       const int r = ci / AE_CPR2;
-      *(__attribute__((address_space(3))) ae_elem8*)(t2 + r * AE_STR2 + ae_bwd_chunk_pos<AE_CPR2>(r, ci % AE_CPR2) * 16) = buf2[i];
+      *(__attribute__((address_space(3))) ae_elem8*)(t2 + r * AE_STR2 + ae_bwd_chunk_pos<AE_CPR2>(r, ci % AE_CPR2) * 16) = sr.b2[i];
     }
 #if AE_BWD_ROLE == 1
-    if (tid < 2 * AE_BS) ((ae_lds_f32*)(t2 + AE_T2_BYTES))[tid] = buf_rs;
+    if (tid < 2 * AE_BS) ((ae_lds_f32*)(t2 + AE_T2_BYTES))[tid] = sr.rs;
 #endif
   };
 
@@ -249,32 +267,23 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     for (int r = 0; r < 16; r++) acc2[db][r] = 0.f;
 #endif
 
+  // item `it` is multiplied out of LDS stage it % 2; at its end item it + 1 goes from its register set
+  // (sa for odd items, sb for even ones) to the other stage and the set takes the request for item it + 3
   if (n_items > 0) {
-    load_item(0);
-    store_item(0);
+    load_item(0, sb);
+    store_item(0, sb);
+    if (n_items > 1) load_item(1, sa);
+    if (n_items > 2) load_item(2, sb);
   }
   __syncthreads();
 
-  for (int it = 0; it < n_items; it++) {
-    const bool more = it + 1 < n_items;
-    if (more) load_item(it + 1);
+  auto iteration = [&](int it, ae_stage_regs& next) {
     const ae_lds_byte* t1 = lds + (it & 1) * AE_STAGE_BYTES;
     const ae_lds_byte* t2 = t1 + AE_T1_BYTES;
     const int s0 = item_tile(it) * AE_BS;
 
-    // S = X1 R1^T and dP = X2 R2^T: [streamed row][resident row]
-    ae_f32x16 sacc[2], pacc[2];
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) sacc[nb][r] = pacc[nb][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < AE_NKS1; ks++) sacc[nb] = ae_mfma32(row_frag1(t1, nb, ks), rf1[ks], sacc[nb]);
-#pragma unroll
-      for (int ks = 0; ks < AE_NKS2; ks++) pacc[nb] = ae_mfma32(row_frag2(t2, nb, ks), rf2[ks], pacc[nb]);
-    }
-
-    // p and ds, packed as B operands: k-step kk holds the lane's elements 8*kk .. 8*kk+7
+    // S = X1 R1^T and dP = X2 R2^T, [streamed row][resident row], one 32-row block of the tile at a
+    // time; p and ds are packed as B operands: k-step kk holds the lane's elements 8*kk .. 8*kk+7
     ae_elem8 pf[4], dsf[4];
 #if AE_BWD_ROLE == 1
     const ae_lds_f32* rs_l = (const ae_lds_f32*)(t2 + AE_T2_BYTES);
@@ -282,31 +291,41 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #else
     const int hq = h;
 #endif
+    (void)hq;
 #pragma unroll
-    for (int e = 0; e < 32; e++) {
-      const int nb = e >> 4, r = e & 15;
-      const int sl = nb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);     // streamed row inside the tile
-      const int srow = s0 + sl;
+    for (int nb = 0; nb < 2; nb++) {
+      ae_f32x16 sacc, pacc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) sacc[r] = pacc[r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS1; ks++) sacc = ae_mfma32(row_frag1(t1, nb, ks), rf1[ks], sacc);
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS2; ks++) pacc = ae_mfma32(row_frag2(t2, nb, ks), rf2[ks], pacc);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int e = nb * 16 + r;
+        const int sl = nb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);     // streamed row inside the tile
+        const int srow = s0 + sl;
 #if AE_BWD_ROLE == 0
-      const int qi = rrow, ki = srow;
-      const float l2 = lse2_r, dl = delta_r;
+        const int qi = rrow, ki = srow;
+        const float l2 = lse2_r, dl = delta_r;
 #else
-      const int qi = srow, ki = rrow;
-      const float l2 = rs_l[sl], dl = rs_l[AE_BS + sl];
+        const int qi = srow, ki = rrow;
+        const float l2 = rs_l[sl], dl = rs_l[AE_BS + sl];
 #endif
-      bool vis = r_ok && srow < n_str;
+        bool vis = r_ok && srow < n_str;
 #if AE_MASK_MODE == 1
-      vis = vis && qi >= ki;
+        vis = vis && qi >= ki;
 #endif
 #if AE_HAS_MASK_MOD
-      vis = vis && ae_mask_mod(b, hq, qi, ki);
+        vis = vis && ae_mask_mod(b, hq, qi, ki);
 #endif
-      const float pv = vis ? ae_exp2(__builtin_fmaf(sacc[nb][r], AE_SM_SCALE * AE_LOG2E, -l2)) : 0.f;
-      const float dsv = pv * (pacc[nb][r] - dl) * AE_SM_SCALE;
-      pf[e >> 3][e & 7] = (ae_elem)pv;
-      dsf[e >> 3][e & 7] = (ae_elem)dsv;
+        const float pv = vis ? ae_exp2(__builtin_fmaf(sacc[r], AE_SM_SCALE * AE_LOG2E, -l2)) : 0.f;
+        const float dsv = pv * (pacc[r] - dl) * AE_SM_SCALE;
+        pf[e >> 3][e & 7] = (ae_elem)pv;
+        dsf[e >> 3][e & 7] = (ae_elem)dsv;
+      }
     }
-    (void)hq;
 
     // OUT^T[d][resident] += X^T[d][streamed] ds[streamed][resident]
 #pragma unroll
@@ -322,8 +341,13 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     }
     (void)pf;
 
-    if (more) store_item((it + 1) & 1);
+    if (it + 1 < n_items) store_item((it + 1) & 1, next);
+    if (it + 3 < n_items) load_item(it + 3, next);
     __syncthreads();
+  };
+  for (int it = 0; it < n_items; it += 2) {
+    iteration(it, sa);
+    if (it + 1 < n_items) iteration(it + 1, sb);
   }
 
   // ---- results: lane owns its resident row, columns 32*db + 8*(r/4) + 4*hf + r%4 ------------------
