@@ -21,8 +21,8 @@
 // a lane's 16 accumulator registers, which makes the packed p and ds the B operand of the second
 // set of products, OUT^T[d, resident] += X^T[d, streamed] ds[streamed, resident], with X^T read from
 // the same LDS tile through ds_read_b64_tr_b16.  Streamed tiles (64 rows) are staged through LDS,
-// double buffered, with the pair swizzle of the forward kernels' V tile (transposed reads conflict
-// free, row reads two-way).
+// double buffered, with the pair swizzle of the forward kernels' V tile plus a flip of the two halves of
+// a pair (see ae_bwd_chunk_pos): one layout serves the row reads and the transposed reads.
 //
 // Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0 none, 1 causal)
 // AE_HAS_MASK_MOD AE_SM_SCALE AE_BWD_ROLE.  Functors used ("ae_functors.h"): ae_mask_mod.
@@ -57,11 +57,17 @@ static_assert(AE_MASK_MODE == 0 || AE_MASK_MODE == 1, "none or causal (an elemen
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 typedef __attribute__((address_space(3))) float ae_lds_f32;
+struct ae_bwd_true { static constexpr bool value = true; };
+struct ae_bwd_false { static constexpr bool value = false; };
 
-// LDS position of 16-byte chunk c of row r: pairs of chunks are exchanged by the row's low bits
+// LDS position of 16-byte chunk c of row r: the 32-byte pairs of a row are exchanged by the row's low
+// bits (transposed reads of a column group then spread over the banks), and the two chunks of a pair by
+// the next row bit (so do the row reads of 16 consecutive rows, which all ask for the same chunk).
+template <int CPR>
+AE_DEV int ae_bwd_half_flip(int r) { return (r >> (CPR == 16 ? 3 : 2)) & 1; }
 template <int CPR>
 AE_DEV int ae_bwd_chunk_pos(int r, int c) {
-  return ((((c >> 1) ^ (r & (CPR / 2 - 1))) << 1) | (c & 1));
+  return ((((c >> 1) ^ (r & (CPR / 2 - 1))) << 1) | ((c ^ ae_bwd_half_flip<CPR>(r)) & 1));
 }
 
 #if AE_BWD_ROLE == 0
@@ -245,12 +251,15 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   // a lane's accumulator registers hold the rows (see the forward kernels' V^T fragment).
   const int t_row = 4 * hf + ((lane & 15) >> 2);
   const int t_g = l32 >> 4;
-  auto tr_frag = [&](const ae_lds_byte* t, int str, int ppr, int kk, int db) -> ae_elem8 {
+  auto tr_frag = [&](const ae_lds_byte* t, int str, int cpr, int kk, int db) -> ae_elem8 {
     const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
-    const int r_lo = rb0 + t_row;
-    const ae_lds_byte* a0 = t + r_lo * str + (lane & 3) * 8 + (((2 * db + t_g) ^ (t_row & (ppr - 1))) << 5);
-    ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)a0);
-    ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)(a0 + 8 * str));
+    const int r_lo = rb0 + t_row, r_hi = r_lo + 8;
+    const int sh = cpr == 16 ? 3 : 2;
+    const int pair = ((2 * db + t_g) ^ (t_row & (cpr / 2 - 1))) << 5;
+    const ae_lds_byte* a_lo = t + r_lo * str + pair + (((lane & 3) * 8) ^ (((r_lo >> sh) & 1) * 16));
+    const ae_lds_byte* a_hi = t + r_hi * str + pair + (((lane & 3) * 8) ^ (((r_hi >> sh) & 1) * 16));
+    ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)a_lo);
+    ae_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)a_hi);
     return __builtin_bit_cast(ae_elem8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
@@ -292,8 +301,13 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     const int hq = h;
 #endif
     (void)hq;
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+    // only tiles that touch the diagonal, the end of a sequence or an elementwise mask test visibility
+    const int r0w = r0 + wave * 32;
+    bool need_vis = (AE_HAS_MASK_MOD != 0) || s0 + AE_BS > n_str || r0w + 32 > n_res;
+#if AE_MASK_MODE == 1
+    need_vis = need_vis || (AE_BWD_ROLE == 0 ? s0 + AE_BS - 1 > r0w : s0 < r0w + 31);
+#endif
+    auto block = [&](int nb, auto masked) {
       ae_f32x16 sacc, pacc;
 #pragma unroll
       for (int r = 0; r < 16; r++) sacc[r] = pacc[r] = 0.f;
@@ -313,18 +327,29 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
         const int qi = srow, ki = rrow;
         const float l2 = rs_l[sl], dl = rs_l[AE_BS + sl];
 #endif
-        bool vis = r_ok && srow < n_str;
+        float pv = ae_exp2(__builtin_fmaf(sacc[r], AE_SM_SCALE * AE_LOG2E, -l2));
+        if (decltype(masked)::value) {
+          bool vis = r_ok && srow < n_str;
 #if AE_MASK_MODE == 1
-        vis = vis && qi >= ki;
+          vis = vis && qi >= ki;
 #endif
 #if AE_HAS_MASK_MOD
-        vis = vis && ae_mask_mod(b, hq, qi, ki);
+          vis = vis && ae_mask_mod(b, hq, qi, ki);
 #endif
-        const float pv = vis ? ae_exp2(__builtin_fmaf(sacc[r], AE_SM_SCALE * AE_LOG2E, -l2)) : 0.f;
-        const float dsv = pv * (pacc[r] - dl) * AE_SM_SCALE;
+          pv = vis ? pv : 0.f;
+        }
+        (void)qi; (void)ki;
+        const float dsv = pv * (pacc[r] - dl);                 // score_mod's derivative (the scale) is applied to the sums
         pf[e >> 3][e & 7] = (ae_elem)pv;
         dsf[e >> 3][e & 7] = (ae_elem)dsv;
       }
+    };
+    if (need_vis) {
+      block(0, ae_bwd_true{});
+      block(1, ae_bwd_true{});
+    } else {
+      block(0, ae_bwd_false{});
+      block(1, ae_bwd_false{});
     }
 
     // OUT^T[d][resident] += X^T[d][streamed] ds[streamed][resident]
@@ -332,11 +357,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     for (int kk = 0; kk < 4; kk++) {
 #pragma unroll
       for (int db = 0; db < AE_NDB1; db++)
-        acc1[db] = ae_mfma32(tr_frag(t1, AE_STR1, AE_CPR1 / 2, kk, db), dsf[kk], acc1[db]);
+        acc1[db] = ae_mfma32(tr_frag(t1, AE_STR1, AE_CPR1, kk, db), dsf[kk], acc1[db]);
 #if AE_BWD_ROLE == 1
 #pragma unroll
       for (int db = 0; db < AE_NDB2; db++)
-        acc2[db] = ae_mfma32(tr_frag(t2, AE_STR2, AE_CPR2 / 2, kk, db), pf[kk], acc2[db]);
+        acc2[db] = ae_mfma32(tr_frag(t2, AE_STR2, AE_CPR2, kk, db), pf[kk], acc2[db]);
 #endif
     }
     (void)pf;
@@ -364,7 +389,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       for (int rg = 0; rg < 4; rg++) {
         ae_elem4 w;
 #pragma unroll
-        for (int t = 0; t < 4; t++) w[t] = (ae_elem)acc1[db][rg * 4 + t];
+        for (int t = 0; t < 4; t++) w[t] = (ae_elem)(acc1[db][rg * 4 + t] * AE_SM_SCALE);
         *(ae_elem4*)(o1 + db * 32 + rg * 8 + hf * 4) = w;
       }
 #if AE_BWD_ROLE == 1
