@@ -65,6 +65,12 @@ AE_DEV void ae_load_lds16(const void* gptr, ae_lds_u8* lds_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(m0v) : "memory");
 }
 
+// The 4-byte form: lane i's dword lands at lds_base + 4*i.
+AE_DEV void ae_load_lds4(const void* gptr, ae_lds_u8* lds_base) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(unsigned long)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(gptr), "s"(m0v) : "memory");
+}
+
 // N (1..8) such loads behind ONE write of M0.  Every write of M0 makes the wave wait for its LDS reads
 // in flight, which costs a kernel that keeps its LDS pipe busy about 40 ns per load; a burst pays that
 // once.  Load i lands at lds_mid + (i - N/2) KiB + lane*16.  The instruction's immediate offset moves

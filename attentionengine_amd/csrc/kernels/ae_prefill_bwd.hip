@@ -20,8 +20,8 @@
 // resident row: S[streamed, resident] = X1 R1^T and dP = X2 R2^T come out with the streamed rows in
 // a lane's 16 accumulator registers, which makes the packed p and ds the B operand of the second
 // set of products, OUT^T[d, resident] += X^T[d, streamed] ds[streamed, resident], with X^T read from
-// the same LDS tile through ds_read_b64_tr_b16.  Streamed tiles (64 rows) are staged through LDS,
-// double buffered, with the pair swizzle of the forward kernels' V tile plus a flip of the two halves of
+// the same LDS tile through ds_read_b64_tr_b16.  Streamed tiles (64 rows) go HBM -> LDS directly
+// (global_load_lds, 16 B per lane), three stages deep, with the pair swizzle of the forward kernels' V tile plus a flip of the two halves of
 // a pair (see ae_bwd_chunk_pos): one layout serves the row reads and the transposed reads.
 //
 // Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0 none, 1 causal)
@@ -47,8 +47,11 @@
 #define AE_NKS2 (AE_DV / 16)       // k-steps of dP
 #define AE_NDB1 (AE_D / 32)        // 32-wide output blocks of dQ / dK
 #define AE_NDB2 (AE_DV / 32)       // ... of dV
-#define AE_L1 ((AE_BS * AE_CPR1) / AE_NT)   // 16-byte chunks a thread moves per tile
+#define AE_L1 ((AE_BS * AE_CPR1) / AE_NT)   // 1 KiB load instructions per wave and tile
 #define AE_L2 ((AE_BS * AE_CPR2) / AE_NT)
+#define AE_NSTAGE 3                // a tile is requested two iterations before it is multiplied
+#define AE_NLOADS (AE_L1 + AE_L2 + (AE_BWD_ROLE == 1 ? 1 : 0))   // load instructions per wave and tile
+#define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 
 static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
 static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
@@ -79,7 +82,7 @@ AE_DEV int ae_bwd_chunk_pos(int r, int c) {
 extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
-  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // two stages of [tile 1][tile 2][lse][delta]
+  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // AE_NSTAGE stages of [tile 1][tile 2][lse][delta]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -137,11 +140,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   float lse2_r, delta_r;
   {
     const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + rrow_c;
-    const float l = p.lse[ri];
-    lse2_r = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
     delta_r = p.delta[ri];
+    lse2_r = p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri];
   }
 #endif
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the resident operands are in registers before any tile request
 
   // ---- the streamed items --------------------------------------------------------------------------
   // role 0: kv tiles 0 .. (causal: up to the diagonal); role 1: for every q head of the group, q tiles
@@ -166,75 +169,79 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   const int n_items = n_t * group;
 #endif
 
-  // global -> register -> LDS staging: thread moves chunks ci = tid + 256*i of each tile.  Two register
-  // sets: a tile is requested three iterations before it is multiplied and written to LDS one iteration
-  // before, so a request has two iterations to land (one was not enough once the workgroups of a head
-  // had drifted apart and their tiles came from beyond the L2).
-  struct ae_stage_regs {
-    ae_elem8 b1[AE_L1], b2[AE_L2];
-    float rs;
+  // Direct HBM -> LDS tile requests.  Wave w fills the 1 KiB blocks w*L .. w*L+L-1 of each tile; a lane's
+  // 16 bytes land at block*1024 + lane*16, i.e. at chunk position cp of row r, so it fetches the global
+  // chunk that belongs there (the swizzle is its own inverse).  A tile's loads of one tensor go out as
+  // one burst behind a single write of M0 (wave-uniform base + per-lane offset + immediate, see
+  // ae_load_lds16_burst_base: bases are passed 4 KiB low and offsets 4 KiB high).  Rows past the end of
+  // the sequence re-read its last row (they are masked).
+  auto lane_off1 = [&](int i, int last_row, int64_t st) -> unsigned {
+    const int sidx = (wave * AE_L1 + i) * 64 + lane;
+    int r = sidx / AE_CPR1;
+    const int c = ae_bwd_chunk_pos<AE_CPR1>(r, sidx % AE_CPR1);
+    r = r < last_row ? r : last_row;
+    return (unsigned)((r * (int)st + c * 8) * 2 + 4096 - (i - AE_L1 / 2) * 1024);
   };
-  ae_stage_regs sa, sb;
-  sa.rs = sb.rs = 0.f;
+  auto lane_off2 = [&](int i, int last_row, int64_t st) -> unsigned {
+    const int sidx = (wave * AE_L2 + i) * 64 + lane;
+    int r = sidx / AE_CPR2;
+    const int c = ae_bwd_chunk_pos<AE_CPR2>(r, sidx % AE_CPR2);
+    r = r < last_row ? r : last_row;
+    return (unsigned)((r * (int)st + c * 8) * 2 + 4096 - (i - AE_L2 / 2) * 1024);
+  };
+#if AE_BWD_ROLE == 0
+  const int64_t st1 = p.k_stride_s, st2 = p.v_stride_s;
+#else
+  const int64_t st1 = p.q_stride_s, st2 = p.do_stride_s;
+#endif
+  unsigned off1[AE_L1], off2[AE_L2];
+#pragma unroll
+  for (int i = 0; i < AE_L1; i++) off1[i] = lane_off1(i, AE_BS, st1);
+#pragma unroll
+  for (int i = 0; i < AE_L2; i++) off2[i] = lane_off2(i, AE_BS, st2);
   auto item_tile = [&](int it) { return t_lo + (AE_BWD_ROLE == 0 ? it : it % n_t); };
   auto item_head = [&](int it) { return AE_BWD_ROLE == 0 ? h : h * group + it / n_t; };   // q head of the item
-  auto load_item = [&](int it, ae_stage_regs& sr) {
-    const int s0 = item_tile(it) * AE_BS;
+  // request item `it` (clamped to the last one: every call issues AE_NLOADS loads) into stage it % NSTAGE
+  auto request_item = [&](int it) {
+    const int itc = it < n_items ? it : n_items - 1;
+    const int s0 = item_tile(itc) * AE_BS;
+    ae_lds_byte* t1 = lds + (it % AE_NSTAGE) * AE_STAGE_BYTES;
+    ae_lds_byte* t2 = t1 + AE_T1_BYTES;
 #if AE_BWD_ROLE == 0
-    const ae_elem* x1 = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
-    const ae_elem* x2 = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
-    const int64_t st1 = p.k_stride_s, st2 = p.v_stride_s;
+    const char* x1 = (const char*)((const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h + (int64_t)s0 * st1);
+    const char* x2 = (const char*)((const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h + (int64_t)s0 * st2);
 #else
-    const int hq = item_head(it);
-    const ae_elem* x1 = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)hq * p.q_stride_h;
-    const ae_elem* x2 = (const ae_elem*)p.dout + (int64_t)b * p.do_stride_b + (int64_t)hq * p.do_stride_h;
-    const int64_t st1 = p.q_stride_s, st2 = p.do_stride_s;
+    const int hq = item_head(itc);
+    const char* x1 = (const char*)((const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)hq * p.q_stride_h + (int64_t)s0 * st1);
+    const char* x2 = (const char*)((const ae_elem*)p.dout + (int64_t)b * p.do_stride_b + (int64_t)hq * p.do_stride_h + (int64_t)s0 * st2);
 #endif
+    unsigned g1[8], g2[8];
+    const bool ragged = s0 + AE_BS > n_str;           // wave-uniform
 #pragma unroll
-    for (int i = 0; i < AE_L1; i++) {
-      const int ci = tid + AE_NT * i;
-      int row = s0 + ci / AE_CPR1;
-      row = row < n_str ? row : n_str - 1;            // rows past the end re-read the last row (masked)
-      sr.b1[i] = *(const ae_elem8*)(x1 + (int64_t)row * st1 + (ci % AE_CPR1) * 8);
+    for (int i = 0; i < 8; i++) {
+      g1[i] = off1[i < AE_L1 ? i : 0];
+      g2[i] = off2[i < AE_L2 ? i : 0];
     }
+    if (__builtin_expect(ragged, 0)) {
+      asm volatile("" ::: "memory");                   // (keeps this one branch, out of the common path)
 #pragma unroll
-    for (int i = 0; i < AE_L2; i++) {
-      const int ci = tid + AE_NT * i;
-      int row = s0 + ci / AE_CPR2;
-      row = row < n_str ? row : n_str - 1;
-      sr.b2[i] = *(const ae_elem8*)(x2 + (int64_t)row * st2 + (ci % AE_CPR2) * 8);
-    }
-#if AE_BWD_ROLE == 1
-    if (tid < 2 * AE_BS) {
-      int row = s0 + (tid & (AE_BS - 1));
-      row = row < n_str ? row : n_str - 1;
-      const int64_t ri = ((int64_t)b * p.heads_q + hq) * p.seqlen_q + row;
-      if (tid < AE_BS) {
-        const float l = p.lse[ri];
-        sr.rs = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
-      } else {
-        sr.rs = p.delta[ri];
+      for (int i = 0; i < 8; i++) {
+        g1[i] = lane_off1(i < AE_L1 ? i : 0, n_str - 1 - s0, st1);
+        g2[i] = lane_off2(i < AE_L2 ? i : 0, n_str - 1 - s0, st2);
       }
     }
-#endif
-  };
-  auto store_item = [&](int stage, const ae_stage_regs& sr) {
-    ae_lds_byte* t1 = lds + stage * AE_STAGE_BYTES;
-    ae_lds_byte* t2 = t1 + AE_T1_BYTES;
-#pragma unroll
-    for (int i = 0; i < AE_L1; i++) {
-      const int ci = tid + AE_NT * i;
-      const int r = ci / AE_CPR1;
-      *(__attribute__((address_space(3))) ae_elem8*)(t1 + r * AE_STR1 + ae_bwd_chunk_pos<AE_CPR1>(r, ci % AE_CPR1) * 16) = sr.b1[i];
-    }
-#pragma unroll
-    for (int i = 0; i < AE_L2; i++) {
-      const int ci = tid + AE_NT * i;
-      const int r = ci / AE_CPR2;
-      *(__attribute__((address_space(3))) ae_elem8*)(t2 + r * AE_STR2 + ae_bwd_chunk_pos<AE_CPR2>(r, ci % AE_CPR2) * 16) = sr.b2[i];
-    }
+    ae_load_lds16_burst_base<AE_L1>(x1 - 4096, g1, t1 + (wave * AE_L1 + AE_L1 / 2) * 1024);
+    ae_load_lds16_burst_base<AE_L2>(x2 - 4096, g2, t2 + (wave * AE_L2 + AE_L2 / 2) * 1024);
 #if AE_BWD_ROLE == 1
-    if (tid < 2 * AE_BS) ((ae_lds_f32*)(t2 + AE_T2_BYTES))[tid] = sr.rs;
+    {
+      // lse (log2 units) and rowsum(do * o) of the tile's 64 q rows: even waves fetch the one, odd waves
+      // the other (twice each, so that every wave issues the same number of loads)
+      int row = s0 + lane;
+      row = row < n_str ? row : n_str - 1;
+      const int plane = (wave & 1) ^ 1;                // plane 0: rowsum(do * o), plane 1: lse
+      const float* src = p.delta + ((int64_t)plane * p.batch * p.heads_q + (int64_t)b * p.heads_q + hq) * p.seqlen_q + row;
+      ae_load_lds4(src, t2 + AE_T2_BYTES + (wave & 1) * AE_BS * 4);
+    }
 #endif
   };
 
@@ -276,18 +283,17 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     for (int r = 0; r < 16; r++) acc2[db][r] = 0.f;
 #endif
 
-  // item `it` is multiplied out of LDS stage it % 2; at its end item it + 1 goes from its register set
-  // (sa for odd items, sb for even ones) to the other stage and the set takes the request for item it + 3
+  // item `it` is multiplied out of stage it % NSTAGE while items it + 1 and it + 2 are on their way
   if (n_items > 0) {
-    load_item(0, sb);
-    store_item(0, sb);
-    if (n_items > 1) load_item(1, sa);
-    if (n_items > 2) load_item(2, sb);
+    request_item(0);
+    request_item(1);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // item 0 has landed
   }
   __syncthreads();
 
-  auto iteration = [&](int it, ae_stage_regs& next) {
-    const ae_lds_byte* t1 = lds + (it & 1) * AE_STAGE_BYTES;
+  for (int it = 0; it < n_items; it++) {
+    request_item(it + 2);             // into the stage of item it - 1, which everyone left at the last barrier
+    const ae_lds_byte* t1 = lds + (it % AE_NSTAGE) * AE_STAGE_BYTES;
     const ae_lds_byte* t2 = t1 + AE_T1_BYTES;
     const int s0 = item_tile(it) * AE_BS;
 
@@ -311,10 +317,18 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       ae_f32x16 sacc, pacc;
 #pragma unroll
       for (int r = 0; r < 16; r++) sacc[r] = pacc[r] = 0.f;
+      // (fences: without them the scheduler hoists every fragment read of the iteration to its top and
+      // the register allocator answers with spills)
 #pragma unroll
-      for (int ks = 0; ks < AE_NKS1; ks++) sacc = ae_mfma32(row_frag1(t1, nb, ks), rf1[ks], sacc);
+      for (int ks = 0; ks < AE_NKS1; ks++) {
+        sacc = ae_mfma32(row_frag1(t1, nb, ks), rf1[ks], sacc);
+        if ((ks & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
-      for (int ks = 0; ks < AE_NKS2; ks++) pacc = ae_mfma32(row_frag2(t2, nb, ks), rf2[ks], pacc);
+      for (int ks = 0; ks < AE_NKS2; ks++) {
+        pacc = ae_mfma32(row_frag2(t2, nb, ks), rf2[ks], pacc);
+        if ((ks & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int e = nb * 16 + r;
@@ -343,6 +357,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
         pf[e >> 3][e & 7] = (ae_elem)pv;
         dsf[e >> 3][e & 7] = (ae_elem)dsv;
       }
+      __builtin_amdgcn_sched_barrier(0);
     };
     if (need_vis) {
       block(0, ae_bwd_true{});
@@ -363,17 +378,14 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       for (int db = 0; db < AE_NDB2; db++)
         acc2[db] = ae_mfma32(tr_frag(t2, AE_STR2, AE_CPR2, kk, db), pf[kk], acc2[db]);
 #endif
+      __builtin_amdgcn_sched_barrier(0);
     }
     (void)pf;
 
-    if (it + 1 < n_items) store_item((it + 1) & 1, next);
-    if (it + 3 < n_items) load_item(it + 3, next);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // item it + 1 has landed (only it + 2 is outstanding)
     __syncthreads();
-  };
-  for (int it = 0; it < n_items; it += 2) {
-    iteration(it, sa);
-    if (it + 1 < n_items) iteration(it + 1, sb);
   }
+  __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));             // nothing may land in LDS after the workgroup has gone
 
   // ---- results: lane owns its resident row, columns 32*db + 8*(r/4) + 4*hf + r%4 ------------------
   if (r_ok) {
@@ -407,8 +419,9 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 }
 
 #if AE_BWD_ROLE == 0
-// rowsum(do * o), fp32 [B,Hq,Sq]: the `doosum` row scale of the reference's backward
-// (flashattn_bwd_preprocess, attn_tl.py:196-221).  DV/8 lanes share a row, 16 bytes each.
+// Work buffer fp32 [2,B,Hq,Sq]: plane 0 = rowsum(do * o), the `doosum` row scale of the reference's
+// backward (flashattn_bwd_preprocess, attn_tl.py:196-221); plane 1 = lse in log2 units, the form the two
+// other launches subtract inside exp2.  DV/8 lanes share a row, 16 bytes each.
 extern "C" __global__ __launch_bounds__(256)
 void ae_bwd_delta_kernel(const ae_attn_bwd_params p) {
   constexpr int LPR = AE_DV / 8;                   // lanes per row
@@ -434,6 +447,12 @@ void ae_bwd_delta_kernel(const ae_attn_bwd_params p) {
     const int lane = tid & 63;
     acc += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ m) << 2, __builtin_bit_cast(int, acc)));
   }
-  if (row < n_rows && c == 0) p.delta[((int64_t)b * p.heads_q + h) * p.seqlen_q + s] = acc;
+  if (row < n_rows && c == 0) {
+    const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + s;
+    const float l = p.lse[ri];
+    p.delta[ri] = acc;
+    // second plane: lse in log2 units, +inf for a row without a visible key (its p is 0 everywhere)
+    p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
+  }
 }
 #endif

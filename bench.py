@@ -38,6 +38,8 @@ WORKLOADS = {
     "c3_sigmoid": ("c3_sigmoid", "prefill"),
     "c4_gqa_decode": ("c4_gqa_decode", "gqa_decode"),
     "c5_mla_decode": ("c5_mla_decode", "mla_decode"),
+    # not a BASELINE configuration: the backward of c2_causal (dq, dk, dv from dout; three launches)
+    "c2_causal_bwd": ("c2_softmax_causal", "prefill_bwd"),
 }
 
 
@@ -64,12 +66,16 @@ def _inputs(name, device):
     def rn(*shape, dtype):
         return torch.randn(*shape, generator=g, dtype=torch.float32).to(dtype).to(device)
     f16, bf16 = torch.float16, torch.bfloat16
-    if name in ("c2_causal", "c2_full", "c3_sigmoid"):
+    if name in ("c2_causal", "c2_full", "c3_sigmoid", "c2_causal_bwd"):
         B, H, S, D = 2, 32, 4096, 128
         args = [rn(B, S, H, D, dtype=f16), rn(B, S, H, D, dtype=f16), rn(B, S, H, D, dtype=f16)]
         if name == "c3_sigmoid":
             args.append(torch.tensor([-math.log(S)], dtype=torch.float32, device=device))
-        flops = 4.0 * B * H * S * S * D * (0.5 if name == "c2_causal" else 1.0)
+        if name == "c2_causal_bwd":
+            args.append(rn(B, S, H, D, dtype=f16))          # dout
+        flops = 4.0 * B * H * S * S * D * (1.0 if name in ("c2_full", "c3_sigmoid") else 0.5)
+        if name == "c2_causal_bwd":
+            flops *= 2.5     # the reference's count: 4*B*H*S^2*DV + 6*B*H*S^2*D, halved (bench_utils.py:1199-1201)
         return args, {"flops": flops, "bytes": 4.0 * B * S * H * D * 2,
                       "shape": {"B": B, "H": H, "S": S, "D": D, "DV": D}, "dtype": "fp16"}
     if name == "c4_gqa_decode":
@@ -98,6 +104,13 @@ def measure(name, steps, warmup):
     key, kind = WORKLOADS[name]
     mod = G.benchmark_engines({key})[key]
     args, info = _inputs(name, dev)
+    if kind == "prefill_bwd":
+        # the timed step is the backward alone: dq, dk, dv from (q, k, v, out, lse, dout)
+        q, k, v, dout = args
+        with torch.no_grad():
+            out = mod(q, k, v)
+        lse = mod.final_rowscales["lse"]
+        mod, args = mod._op.backward_op(), [q, k, v, out, lse, dout]
     # Untimed warm-up: the W steps asked for, continued until the launches have covered CLOCK_RAMP_MS.
     # The shader clock of an idle MI355X takes some tens of milliseconds of load to reach its working
     # point (measured: 0.335 ms per step after 10 warm-up steps, 0.29 ms after 50 or more), and the
@@ -123,7 +136,7 @@ def measure(name, steps, warmup):
            **info}
     res["tflops"] = info["flops"] / (wall_ms * 1e-3) / 1e12
     res["gbs"] = info["bytes"] / (wall_ms * 1e-3) / 1e9
-    if kind == "prefill":
+    if kind in ("prefill", "prefill_bwd"):
         ach = info["flops"] / (ev_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                            "frac": ach / PEAK_MFMA_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
@@ -166,6 +179,17 @@ def cpu_baseline(name):
     from oracle import attention_ref as R
     threads = torch.get_num_threads()
     g = torch.Generator().manual_seed(0)
+    if name == "c2_causal_bwd":
+        H, S, D, chunk = 32, 4096, 128, 2
+        q, k, v, do = (torch.randn(1, S, H, D, generator=g).half().float() for _ in range(4))
+        t0 = time.perf_counter()
+        for h0 in range(0, H, chunk):
+            sl = slice(h0, h0 + chunk)
+            R.softmax_attention_grads(q[:, :, sl], k[:, :, sl], v[:, :, sl], do[:, :, sl], causal=True)
+        dt = time.perf_counter() - t0
+        return {"value": 10.0 * H * S * S * D * 0.5 / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": f"oracle gradients on 1 of 2 batch entries (32 heads, S=4096, D=128, fp32), {dt:.2f} s, "
+                          "reference flop convention"}
     if name in ("c2_causal", "c2_full", "c3_sigmoid"):
         H, S, D, chunk = 32, 4096, 128, 4
         q = torch.randn(1, S, H, D, generator=g).half().float()

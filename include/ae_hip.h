@@ -117,8 +117,8 @@ typedef struct ae_tile_cfg {
 /*
  * Kernel argument block of the backward kernels (softmax attention, prefill shapes). Same layouts as
  * ae_attn_params; dout [B,Sq,Hq,DV] is the gradient of `out`, dq/dk/dv have the shapes of q/k/v, lse
- * is the forward's natural-log row scale fp32 [B,Hq,Sq], delta a caller-allocated fp32 [B,Hq,Sq]
- * work buffer that receives rowsum(dout * out). Stands where the reference passes Q, K, V, dO, lse
+ * is the forward's natural-log row scale fp32 [B,Hq,Sq], delta a caller-allocated fp32 [2,B,Hq,Sq]
+ * work buffer (the first launch fills it: rowsum(dout * out), and lse in log2 units). Stands where the reference passes Q, K, V, dO, lse
  * and Delta to flashattn_bwd (core/template/tl_template/attn/attn_tl.py:271-295).
  */
 typedef struct ae_attn_bwd_params {
