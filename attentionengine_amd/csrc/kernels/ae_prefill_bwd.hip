@@ -52,6 +52,10 @@
 #define AE_NSTAGE 3                // a tile is requested two iterations before it is multiplied
 #define AE_NLOADS (AE_L1 + AE_L2 + (AE_BWD_ROLE == 1 ? 1 : 0))   // load instructions per wave and tile
 #define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+#ifndef AE_AHEAD
+#define AE_AHEAD 4                 // LDS fragments in flight ahead of the MFMA that uses them
+#endif
+#define AE_RING (AE_AHEAD + 1)
 
 static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
 static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
@@ -317,17 +321,29 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       ae_f32x16 sacc, pacc;
 #pragma unroll
       for (int r = 0; r < 16; r++) sacc[r] = pacc[r] = 0.f;
-      // (fences: without them the scheduler hoists every fragment read of the iteration to its top and
-      // the register allocator answers with spills)
+      // fragment stream of the block: S and dP k-steps alternate (two independent accumulation chains);
+      // fragments are read AE_AHEAD MFMAs ahead of their use into a small ring, one fence per MFMA (left to
+      // itself the scheduler either exposes the LDS latency or hoists every read and spills)
+      constexpr int NF = AE_NKS1 + AE_NKS2;
+      auto frag = [&](int f) -> ae_elem8 {
+        // f even and S still has k-steps: S; else dP (the dims may differ)
+        const int pairs = AE_NKS1 < AE_NKS2 ? AE_NKS1 : AE_NKS2;
+        if (f < 2 * pairs) return (f & 1) ? row_frag2(t2, nb, f >> 1) : row_frag1(t1, nb, f >> 1);
+        return AE_NKS1 > AE_NKS2 ? row_frag1(t1, nb, f - pairs) : row_frag2(t2, nb, f - pairs);
+      };
+      ae_elem8 ring[AE_RING];
 #pragma unroll
-      for (int ks = 0; ks < AE_NKS1; ks++) {
-        sacc = ae_mfma32(row_frag1(t1, nb, ks), rf1[ks], sacc);
-        if ((ks & 3) == 3) __builtin_amdgcn_sched_barrier(0);
-      }
+      for (int f = 0; f < AE_AHEAD && f < NF; f++) ring[f] = frag(f);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 0; ks < AE_NKS2; ks++) {
-        pacc = ae_mfma32(row_frag2(t2, nb, ks), rf2[ks], pacc);
-        if ((ks & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+      for (int f = 0; f < NF; f++) {
+        if (f + AE_AHEAD < NF) ring[(f + AE_AHEAD) % AE_RING] = frag(f + AE_AHEAD);
+        const int pairs = AE_NKS1 < AE_NKS2 ? AE_NKS1 : AE_NKS2;
+        const bool is_s = f < 2 * pairs ? !(f & 1) : AE_NKS1 > AE_NKS2;
+        const int ks = f < 2 * pairs ? f >> 1 : f - pairs;
+        if (is_s) sacc = ae_mfma32(ring[f % AE_RING], rf1[ks], sacc);
+        else pacc = ae_mfma32(ring[f % AE_RING], rf2[ks], pacc);
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) {
@@ -367,18 +383,32 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       block(1, ae_bwd_false{});
     }
 
-    // OUT^T[d][resident] += X^T[d][streamed] ds[streamed][resident]
+    // OUT^T[d][resident] += X^T[d][streamed] ds[streamed][resident]: fragment f = (k-step kk, output block
+    // j of dQ/dK, then of dV), read ahead through the same kind of ring
+    {
+      constexpr int NB_OUT = AE_NDB1 + (AE_BWD_ROLE == 1 ? AE_NDB2 : 0);
+      constexpr int NF = 4 * NB_OUT;
+      auto frag = [&](int f) -> ae_elem8 {
+        const int kk = f / NB_OUT, j = f % NB_OUT;
+        return j < AE_NDB1 ? tr_frag(t1, AE_STR1, AE_CPR1, kk, j) : tr_frag(t2, AE_STR2, AE_CPR2, kk, j - AE_NDB1);
+      };
+      ae_elem8 ring[AE_RING];
 #pragma unroll
-    for (int kk = 0; kk < 4; kk++) {
-#pragma unroll
-      for (int db = 0; db < AE_NDB1; db++)
-        acc1[db] = ae_mfma32(tr_frag(t1, AE_STR1, AE_CPR1, kk, db), dsf[kk], acc1[db]);
-#if AE_BWD_ROLE == 1
-#pragma unroll
-      for (int db = 0; db < AE_NDB2; db++)
-        acc2[db] = ae_mfma32(tr_frag(t2, AE_STR2, AE_CPR2, kk, db), pf[kk], acc2[db]);
-#endif
+      for (int f = 0; f < AE_AHEAD && f < NF; f++) ring[f] = frag(f);
       __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int f = 0; f < NF; f++) {
+        if (f + AE_AHEAD < NF) ring[(f + AE_AHEAD) % AE_RING] = frag(f + AE_AHEAD);
+        const int kk = f / NB_OUT, j = f % NB_OUT;
+        if (j < AE_NDB1) {
+          acc1[j] = ae_mfma32(ring[f % AE_RING], dsf[kk], acc1[j]);
+        } else {
+#if AE_BWD_ROLE == 1
+          acc2[j - AE_NDB1] = ae_mfma32(ring[f % AE_RING], pf[kk], acc2[j - AE_NDB1]);
+#endif
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     (void)pf;
 
