@@ -54,6 +54,8 @@ MEASURED_TRAFFIC_BYTES = {
     "c3_sigmoid": 201.4e6 + 68.9e6,      # Q+K+V read once; O written (no row scales)
     "c4_gqa_decode": 2147.9e6 + 4.2e6,   # algorithmic K+V: 2147.5e6 (fp32 partials written: 4.2e6)
     "c5_mla_decode": 623.1e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
+    "c2_causal_bwd": 748.0e6 + 134.9e6,      # the dk/dv launch (the longest of the three): q, k, v, dout read
+                                         # about three times over (algorithmic 268e6), dk + dv written once
 }
 
 
