@@ -68,10 +68,12 @@ class AttnParams(C.Structure):
 class AttnBwdParams(C.Structure):
     """Mirror of ``ae_attn_bwd_params``."""
     _fields_ = (
-        [(n, C.c_void_p) for n in ("q", "k", "v", "out", "dout", "lse", "delta", "dq", "dk", "dv")]
+        [(n, C.c_void_p) for n in ("q", "k", "v", "out", "dout", "lse", "delta", "dq", "dk", "dv",
+                                   "mask_dq", "mask_dkv")]
         + [(f"{t}_stride_{a}", C.c_int64) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for a in "bsh"]
         + [("batch", C.c_int32), ("heads_q", C.c_int32), ("heads_kv", C.c_int32),
-           ("seqlen_q", C.c_int32), ("seqlen_kv", C.c_int32), ("reserved", C.c_int32 * 3)]
+           ("seqlen_q", C.c_int32), ("seqlen_kv", C.c_int32), ("mask_b", C.c_int32), ("mask_h", C.c_int32),
+           ("reserved", C.c_int32 * 1)]
     )
 
 

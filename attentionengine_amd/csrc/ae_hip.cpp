@@ -487,6 +487,13 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
       cfg->lds_bytes > 160 * 1024 || cfg->head_dim_v <= 0 || cfg->head_dim_v % 8 != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: bad tile configuration (bm=%d bn=%d threads=%d lds=%d dv=%d)",
                 cfg->block_m, cfg->block_n, cfg->threads, cfg->lds_bytes, cfg->head_dim_v);
+  if (cfg->mask_mode == 2) {
+    if (!p->mask_dq || !p->mask_dkv)
+      return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: tile-class kernels without their tables");
+    if ((p->mask_b != 1 && p->mask_b != p->batch) || (p->mask_h != 1 && p->mask_h != p->heads_q))
+      return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: table batch/head extent (%d,%d) must be 1 or (B,Hq)",
+                  p->mask_b, p->mask_h);
+  }
   const uint64_t rows = (uint64_t)p->batch * p->seqlen_q * p->heads_q;
   const uint64_t rows_per_wg = 256u / (uint32_t)(cfg->head_dim_v / 8);
   const uint64_t g_delta = (rows + rows_per_wg - 1) / rows_per_wg;

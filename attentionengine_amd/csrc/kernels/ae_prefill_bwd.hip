@@ -24,8 +24,13 @@
 // (global_load_lds, 16 B per lane), three stages deep, with the pair swizzle of the forward kernels' V tile plus a flip of the two halves of
 // a pair (see ae_bwd_chunk_pos): one layout serves the row reads and the transposed reads.
 //
-// Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0 none, 1 causal)
-// AE_HAS_MASK_MOD AE_SM_SCALE AE_BWD_ROLE.  Functors used ("ae_functors.h"): ae_mask_mod.
+// Masks: mode 0 none; mode 1 analytic causal (tiles beyond the diagonal never visited); mode 2 two
+// tile-class tables built on the host from mask_mod (0 skip, 1 test per element, 2 fully visible), one
+// per launch because the two tile shapes differ: [q tiles of 128][kv tiles of 64] for dq,
+// [q tiles of 64][kv tiles of 128] for dk/dv (role of blockattn_tl.py's block mask in the backward).
+//
+// Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0, 1, 2) AE_HAS_MASK_MOD
+// AE_SM_SCALE AE_BWD_ROLE.  Functors used ("ae_functors.h"): ae_mask_mod.
 
 #include "ae_hip.h"
 #include "ae_config.h"
@@ -60,7 +65,7 @@
 static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
 static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
 static_assert(AE_BWD_ROLE == 0 || AE_BWD_ROLE == 1, "role");
-static_assert(AE_MASK_MODE == 0 || AE_MASK_MODE == 1, "none or causal (an elementwise mask_mod on top)");
+static_assert(AE_MASK_MODE >= 0 && AE_MASK_MODE <= 2, "none, causal, or tile-class tables");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 typedef __attribute__((address_space(3))) float ae_lds_f32;
@@ -167,11 +172,33 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #endif
 #endif
   const int n_t = t_hi - t_lo;
+  // item x: tile t_lo + x % n_t of q head x / n_t of the group (role 0: one head)
 #if AE_BWD_ROLE == 0
   const int n_items = n_t;
 #else
   const int n_items = n_t * group;
 #endif
+  auto item_tile = [&](int x) { return t_lo + (AE_BWD_ROLE == 0 ? x : x % n_t); };
+  auto item_head = [&](int x) { return AE_BWD_ROLE == 0 ? h : h * group + x / n_t; };   // q head of the item
+#if AE_MASK_MODE == 2
+  // class of item x for this workgroup's resident tile
+  auto item_class = [&](int x) -> int {
+    const int hq = item_head(x), t = item_tile(x);
+    const int64_t mbh = (int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : hq);
+#if AE_BWD_ROLE == 0
+    return p.mask_dq[(mbh * n_rt + rt) * n_st + t];            // [q tiles of 128][kv tiles of 64]
+#else
+    return p.mask_dkv[(mbh * n_st + t) * n_rt + rt];           // [q tiles of 64][kv tiles of 128]
+#endif
+  };
+#endif
+  // first item at or after x that has anything visible (n_items if none)
+  auto next_item = [&](int x) {
+#if AE_MASK_MODE == 2
+    while (x < n_items && item_class(x) == 0) x++;
+#endif
+    return x < n_items ? x : n_items;
+  };
 
   // Direct HBM -> LDS tile requests.  Wave w fills the 1 KiB blocks w*L .. w*L+L-1 of each tile; a lane's
   // 16 bytes land at block*1024 + lane*16, i.e. at chunk position cp of row r, so it fetches the global
@@ -203,13 +230,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   for (int i = 0; i < AE_L1; i++) off1[i] = lane_off1(i, AE_BS, st1);
 #pragma unroll
   for (int i = 0; i < AE_L2; i++) off2[i] = lane_off2(i, AE_BS, st2);
-  auto item_tile = [&](int it) { return t_lo + (AE_BWD_ROLE == 0 ? it : it % n_t); };
-  auto item_head = [&](int it) { return AE_BWD_ROLE == 0 ? h : h * group + it / n_t; };   // q head of the item
-  // request item `it` (clamped to the last one: every call issues AE_NLOADS loads) into stage it % NSTAGE
-  auto request_item = [&](int it) {
-    const int itc = it < n_items ? it : n_items - 1;
+  // request item x (past the end: the last item again, so that every call issues AE_NLOADS loads) into `stage`
+  auto request_item = [&](int x, int stage) {
+    const int itc = x < n_items ? x : n_items - 1;
     const int s0 = item_tile(itc) * AE_BS;
-    ae_lds_byte* t1 = lds + (it % AE_NSTAGE) * AE_STAGE_BYTES;
+    ae_lds_byte* t1 = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* t2 = t1 + AE_T1_BYTES;
 #if AE_BWD_ROLE == 0
     const char* x1 = (const char*)((const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h + (int64_t)s0 * st1);
@@ -287,17 +312,19 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     for (int r = 0; r < 16; r++) acc2[db][r] = 0.f;
 #endif
 
-  // item `it` is multiplied out of stage it % NSTAGE while items it + 1 and it + 2 are on their way
-  if (n_items > 0) {
-    request_item(0);
-    request_item(1);
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // item 0 has landed
+  // the n-th visited item is multiplied out of stage n % NSTAGE while the next two are on their way
+  int x0 = next_item(0), x1 = next_item(x0 + 1), x2 = next_item(x1 + 1);
+  if (x0 < n_items) {
+    request_item(x0, 0);
+    request_item(x1, 1);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // the first item has landed
   }
   __syncthreads();
 
-  for (int it = 0; it < n_items; it++) {
-    request_item(it + 2);             // into the stage of item it - 1, which everyone left at the last barrier
-    const ae_lds_byte* t1 = lds + (it % AE_NSTAGE) * AE_STAGE_BYTES;
+  for (int n = 0; x0 < n_items; n++) {
+    const int it = x0;
+    request_item(x2, (n + 2) % AE_NSTAGE);   // into the stage everyone left at the last barrier
+    const ae_lds_byte* t1 = lds + (n % AE_NSTAGE) * AE_STAGE_BYTES;
     const ae_lds_byte* t2 = t1 + AE_T1_BYTES;
     const int s0 = item_tile(it) * AE_BS;
 
@@ -313,7 +340,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     (void)hq;
     // only tiles that touch the diagonal, the end of a sequence or an elementwise mask test visibility
     const int r0w = r0 + wave * 32;
+#if AE_MASK_MODE == 2
+    bool need_vis = item_class(it) != 2 || s0 + AE_BS > n_str || r0w + 32 > n_res;
+#else
     bool need_vis = (AE_HAS_MASK_MOD != 0) || s0 + AE_BS > n_str || r0w + 32 > n_res;
+#endif
 #if AE_MASK_MODE == 1
     need_vis = need_vis || (AE_BWD_ROLE == 0 ? s0 + AE_BS - 1 > r0w : s0 < r0w + 31);
 #endif
@@ -412,8 +443,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     }
     (void)pf;
 
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // item it + 1 has landed (only it + 2 is outstanding)
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // the next item has landed (only the one after it is outstanding)
     __syncthreads();
+    x0 = x1;
+    x1 = x2;
+    x2 = next_item(x2 + 1);
   }
   __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));             // nothing may land in LDS after the workgroup has gone
 

@@ -132,6 +132,8 @@ typedef struct ae_attn_bwd_params {
   void* dq;
   void* dk;
   void* dv;
+  const int8_t* mask_dq;   /* mask mode 2: tile classes [mask_b,mask_h,ceil(Sq/128),ceil(Skv/64)], else NULL */
+  const int8_t* mask_dkv;  /* mask mode 2: tile classes [mask_b,mask_h,ceil(Sq/64),ceil(Skv/128)], else NULL */
   int64_t q_stride_b, q_stride_s, q_stride_h;
   int64_t k_stride_b, k_stride_s, k_stride_h;
   int64_t v_stride_b, v_stride_s, v_stride_h;
@@ -141,7 +143,8 @@ typedef struct ae_attn_bwd_params {
   int64_t dk_stride_b, dk_stride_s, dk_stride_h;
   int64_t dv_stride_b, dv_stride_s, dv_stride_h;
   int32_t batch, heads_q, heads_kv, seqlen_q, seqlen_kv;
-  int32_t reserved[3];
+  int32_t mask_b, mask_h;  /* batch / head extents of the two tables: 1 or (B, Hq) */
+  int32_t reserved[1];
 } ae_attn_bwd_params;
 
 typedef struct ae_devinfo {
@@ -246,7 +249,8 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
  *   and `dq` (one workgroup per 128 q rows of a (batch, q head)). The reference's single backward
  *   kernel with fp32 atomics on dq and its postprocess (attn_tl.py:238-455) are replaced by these two
  *   atomic-free launches. cfg: block_m = 128, block_n = 64, threads = 256 and the dynamic LDS of the
- *   compiled kernels; head dims as compiled. All gradients are written in full (no accumulation).
+ *   compiled kernels, mask_mode as compiled (2 needs the two tile-class tables: 0 skip, 1 test per
+ *   element, 2 fully visible); head dims as compiled. All gradients are written in full (no accumulation).
  */
 int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
                    const ae_tile_cfg* cfg, void* stream);

@@ -77,6 +77,20 @@ def test_softmax_backward_elementwise_mask_and_dv(cuda_device):
     _run(2, 2, 2, 130, 130, 64, 128, torch.bfloat16, None, False)
 
 
+def test_softmax_backward_skips_masked_tiles(cuda_device):
+    """Masks that are not causal come with two tile-class tables (one per launch): tiles without a
+    visible element are skipped, partly visible ones test mask_mod per element.  A narrow sliding window
+    over a long sequence (most tiles skipped), a mask that depends on the head (one table per head), a
+    shifted causal mask with grouped heads."""
+    for name, mask_mod, H, Hkv, S in (("window", C.make_sliding_window_mask(100), 2, 2, 700),
+                                      ("head", C.head_dependent_mask, 4, 4, 520),
+                                      ("shifted", C.causal_shifted_mask, 4, 2, 333)):
+        print(f"case bwd tile classes {name}", flush=True)
+        _run(1, H, Hkv, S, S, 128, 128, torch.float16, mask_mod, False, seed=11)
+        eng = _engine(1, H, Hkv, S, 128, 128, torch.float16, mask_mod, 1 / math.sqrt(128))
+        assert eng._op._plan(1, H, S, S, None).mode == 2
+
+
 def test_backward_of_other_graphs_is_refused(cuda_device):
     """Only graphs proven to be softmax attention have a backward; the others say so."""
     B, H, S, D = 1, 2, 128, 64
