@@ -377,7 +377,15 @@ class Emitter:
             self.lines.append(f"const float {out} = {fn}<{self.n}>({src});")
             return (out, False)
         if t == "MaxBwd":
-            raise NotImplementedError("MaxBwd belongs to the backward pass")
+            # gradient g of max(x, y) with respect to x: passes where x won (zero at a tie)
+            is_arr = any(a for _, a in ins)
+            expr = f"({self._at(ins[1])} > {self._at(ins[2])} ? {self._at(ins[0])} : 0.0f)"
+            if is_arr:
+                self.lines.append(f"float {out}[{self.n}];")
+                self._loop(f"{out}[e] = {expr};")
+            else:
+                self.lines.append(f"const float {out} = {expr};")
+            return (out, is_arr)
         if t not in ELEMENTWISE_UNARY and t not in ELEMENTWISE_BINARY:
             raise NotImplementedError(str(t))
 

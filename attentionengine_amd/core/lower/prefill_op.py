@@ -46,6 +46,7 @@ class PrefillOp:
         self.mask_block = (int(infer_mask_block_M), int(infer_mask_block_N))
         self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
                                          self.dtype, mask_value)
+        self._graph = (score_mod, online_func, custom_fwd_inputs)     # the backward traces score_mod again
         self.functor_src = L.render_functors(self.functors)
         self.tiles = L.choose_prefill_tiles(self.D, self.DV_launch, _dim(q_meta.shape[2], 0),
                                             None if self.mask_value_zero else self.functors.softmax,
@@ -180,7 +181,7 @@ class PrefillOp:
     def backward_op(self):
         if getattr(self, "_bwd", None) is None:
             from .prefill_bwd_op import PrefillBwdOp
-            self._bwd = PrefillBwdOp(self)
+            self._bwd = PrefillBwdOp(self, *self._graph)
         return self._bwd
 
     def _forward(self, q, k, v, *extra):
@@ -280,11 +281,13 @@ class _PrefillFunction(torch.autograd.Function):
             out = op._forward(q.detach(), k.detach(), v.detach(), *extra)
         ctx.op = op
         ctx.n_extra = len(extra)
-        ctx.save_for_backward(q, k, v, out, op.final_rowscales[bwd.lse_name])
+        ctx.customs = tuple(extra[:len(op.functors.customs)])       # scalar CustomIO tensors of score_mod
+        lse = op.final_rowscales[bwd.lse_name] if bwd.lse_name is not None else q.new_empty(0)
+        ctx.save_for_backward(q, k, v, out, lse)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         q, k, v, out, lse = ctx.saved_tensors
-        dq, dk, dv = ctx.op.backward_op()(q, k, v, out, lse, dout)
+        dq, dk, dv = ctx.op.backward_op()(q, k, v, out, lse, dout, ctx.customs)
         return (None, dq, dk, dv) + (None,) * ctx.n_extra

@@ -70,6 +70,7 @@ class AttnBwdParams(C.Structure):
     _fields_ = (
         [(n, C.c_void_p) for n in ("q", "k", "v", "out", "dout", "lse", "delta", "dq", "dk", "dv",
                                    "mask_dq", "mask_dkv")]
+        + [("custom", C.c_void_p * AE_MAX_CUSTOM)]
         + [(f"{t}_stride_{a}", C.c_int64) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for a in "bsh"]
         + [("batch", C.c_int32), ("heads_q", C.c_int32), ("heads_kv", C.c_int32),
            ("seqlen_q", C.c_int32), ("seqlen_kv", C.c_int32), ("mask_b", C.c_int32), ("mask_h", C.c_int32),

@@ -8,7 +8,7 @@ API-compatible with attention_engine/core/transform/core.py:
 
 User callables (score_mod, OnlineFunc.online_fwd, ...) are traced by calling them on these
 objects; every operation appends a node and returns a new symbol whose ``prev`` are its
-operands.  The forward-only build leaves out the symbolic differentiation (119-199).
+operands.  The symbolic differentiation (119-199) lives in autodiff.py (``derivative``).
 """
 from __future__ import annotations
 
@@ -114,7 +114,7 @@ class SymbolScalar:
         return out
 
     def backward(self, grad=None):
-        raise NotImplementedError("symbolic differentiation is outside the forward-only build")
+        raise NotImplementedError("use core.transform.autodiff.derivative(out, wrt): the derivative as a traced expression")
 
     def __add__(self, other):
         return self.op(Add, [other])

@@ -474,8 +474,7 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
                    const ae_tile_cfg* cfg, void* stream) {
   if (!delta || !dkv || !dq) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: kernel is NULL");
   if (!p || !cfg) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: params/cfg is NULL");
-  if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->lse || !p->delta || !p->dq || !p->dk ||
-      !p->dv)
+  if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->delta || !p->dq || !p->dk || !p->dv)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: a tensor pointer is NULL");
   if (p->batch <= 0 || p->heads_q <= 0 || p->heads_kv <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: non-positive extent (B=%d Hq=%d Hkv=%d Sq=%d Skv=%d)",

@@ -29,8 +29,13 @@
 // per launch because the two tile shapes differ: [q tiles of 128][kv tiles of 64] for dq,
 // [q tiles of 64][kv tiles of 128] for dk/dv (role of blockattn_tl.py's block mask in the backward).
 //
+// AE_BWD_KIND 1: graphs whose online function does nothing, out = sum_kv f(s) v with f = score_mod (sigmoid
+// and relu attention, attn_script/sigmoidattn.py, reluattn.py): p = f(s), ds = dp * f'(s), both from the
+// generated ae_bwd_pd (f' by symbolic differentiation of the traced score_mod); no row scales, scale 1.
+//
 // Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0, 1, 2) AE_HAS_MASK_MOD
-// AE_SM_SCALE AE_BWD_ROLE.  Functors used ("ae_functors.h"): ae_mask_mod.
+// AE_SM_SCALE AE_BWD_ROLE AE_BWD_KIND.  Functors used ("ae_functors.h"): ae_mask_mod; kind 1: ae_bwd_pd,
+// ae_bwd_load_custom.
 
 #include "ae_hip.h"
 #include "ae_config.h"
@@ -65,6 +70,9 @@
 static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
 static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
 static_assert(AE_BWD_ROLE == 0 || AE_BWD_ROLE == 1, "role");
+#ifndef AE_BWD_KIND
+#define AE_BWD_KIND 0
+#endif
 static_assert(AE_MASK_MODE >= 0 && AE_MASK_MODE <= 2, "none, causal, or tile-class tables");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
@@ -137,6 +145,10 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   const int hk = h;
   const ae_elem* r1p = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)rrow_c * p.k_stride_s + (int64_t)h * p.k_stride_h;
   const ae_elem* r2p = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)rrow_c * p.v_stride_s + (int64_t)h * p.v_stride_h;
+#endif
+#if AE_BWD_KIND == 1
+  ae_custom cust;
+  ae_bwd_load_custom(cust, p);
 #endif
   ae_elem8 rf1[AE_NKS1], rf2[AE_NKS2];
 #pragma unroll
@@ -388,9 +400,18 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
         const int qi = srow, ki = rrow;
         const float l2 = rs_l[sl], dl = rs_l[AE_BS + sl];
 #endif
+#if AE_BWD_KIND == 0
         float pv = ae_exp2(__builtin_fmaf(sacc[r], AE_SM_SCALE * AE_LOG2E, -l2));
+        const float dfac = pacc[r] - dl;
+#else
+        float pv, dfac;
+        ae_bwd_pd(sacc[r], (float)b, (float)hq, (float)qi, (float)ki, cust, pv, dfac);
+        dfac *= pacc[r];
+        (void)l2; (void)dl;
+#endif
+        bool vis = true;
         if (decltype(masked)::value) {
-          bool vis = r_ok && srow < n_str;
+          vis = r_ok && srow < n_str;
 #if AE_MASK_MODE == 1
           vis = vis && qi >= ki;
 #endif
@@ -400,7 +421,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
           pv = vis ? pv : 0.f;
         }
         (void)qi; (void)ki;
-        const float dsv = pv * (pacc[r] - dl);                 // score_mod's derivative (the scale) is applied to the sums
+#if AE_BWD_KIND == 0
+        const float dsv = pv * dfac;                           // score_mod's derivative (the scale) is applied to the sums
+#else
+        const float dsv = vis ? dfac : 0.f;                    // an invisible score contributes nothing and moves nothing
+#endif
         pf[e >> 3][e & 7] = (ae_elem)pv;
         dsf[e >> 3][e & 7] = (ae_elem)dsv;
       }
@@ -513,7 +538,7 @@ void ae_bwd_delta_kernel(const ae_attn_bwd_params p) {
   }
   if (row < n_rows && c == 0) {
     const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + s;
-    const float l = p.lse[ri];
+    const float l = p.lse ? p.lse[ri] : 0.f;
     p.delta[ri] = acc;
     // second plane: lse in log2 units, +inf for a row without a visible key (its p is 0 everywhere)
     p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;

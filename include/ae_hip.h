@@ -117,7 +117,7 @@ typedef struct ae_tile_cfg {
 /*
  * Kernel argument block of the backward kernels (softmax attention, prefill shapes). Same layouts as
  * ae_attn_params; dout [B,Sq,Hq,DV] is the gradient of `out`, dq/dk/dv have the shapes of q/k/v, lse
- * is the forward's natural-log row scale fp32 [B,Hq,Sq], delta a caller-allocated fp32 [2,B,Hq,Sq]
+ * is the forward's natural-log row scale fp32 [B,Hq,Sq] (NULL for graphs without row scales), delta a caller-allocated fp32 [2,B,Hq,Sq]
  * work buffer (the first launch fills it: rowsum(dout * out), and lse in log2 units). Stands where the reference passes Q, K, V, dO, lse
  * and Delta to flashattn_bwd (core/template/tl_template/attn/attn_tl.py:271-295).
  */
@@ -134,6 +134,7 @@ typedef struct ae_attn_bwd_params {
   void* dv;
   const int8_t* mask_dq;   /* mask mode 2: tile classes [mask_b,mask_h,ceil(Sq/128),ceil(Skv/64)], else NULL */
   const int8_t* mask_dkv;  /* mask mode 2: tile classes [mask_b,mask_h,ceil(Sq/64),ceil(Skv/128)], else NULL */
+  const void* custom[AE_MAX_CUSTOM]; /* scalar CustomIO tensors (fp32 [1]) of score_mod, in dict order   */
   int64_t q_stride_b, q_stride_s, q_stride_h;
   int64_t k_stride_b, k_stride_s, k_stride_h;
   int64_t v_stride_b, v_stride_s, v_stride_h;
@@ -251,6 +252,8 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
  *   atomic-free launches. cfg: block_m = 128, block_n = 64, threads = 256 and the dynamic LDS of the
  *   compiled kernels, mask_mode as compiled (2 needs the two tile-class tables: 0 skip, 1 test per
  *   element, 2 fully visible); head dims as compiled. All gradients are written in full (no accumulation).
+ *   The same three launches serve the graphs whose online function does nothing (sigmoid, relu attention:
+ *   kernels compiled with AE_BWD_KIND 1 and the generated derivative of score_mod; lse is NULL then).
  */
 int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
                    const ae_tile_cfg* cfg, void* stream);

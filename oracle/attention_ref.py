@@ -128,6 +128,39 @@ def relu_attention(q, k, v, scale=None, compute_dtype=torch.float32):
     return _apply_p(p, v, compute_dtype)
 
 
+def elementwise_attention_grads(q, k, v, do, kind, scale=None, bias=0.0, causal=False,
+                                compute_dtype=torch.float32):
+    """Gradients (dq, dk, dv) of ``sigmoid_attention`` (kind "sigmoid") and ``relu_attention`` (kind
+    "relu"): out = sum_kv f(s) v has dv = p^T do, ds = (do v^T) * f'(s), dq = ds k, dk = ds^T q -- what the
+    reference's backward computes for attn_script/sigmoidattn.py and reluattn.py, whose online function
+    passes scores and dp through (``OnlineIdentity.forward/backward``) and whose f' comes from the symbolic
+    derivative of score_mod (core/transform/core.py:119-199).  relu' is 0 at 0.  Pinned in
+    tests/test_oracle.py against torch.autograd through the two forward functions."""
+    B, Sq, Hq, D = q.shape
+    Skv, Hkv = k.shape[1], k.shape[2]
+    G = Hq // Hkv
+    scale = 1.0 / math.sqrt(D) if scale is None else scale
+    s = _grouped_scores(q, k, compute_dtype) * scale
+    if kind == "sigmoid":
+        p = torch.sigmoid(s + bias)
+        dpds = p * (1.0 - p) * scale
+    elif kind == "relu":
+        p = torch.relu(s)
+        dpds = (s > 0).to(compute_dtype) * scale
+    else:
+        raise ValueError(kind)
+    if causal:
+        tril = torch.ones(Sq, Skv, dtype=torch.bool).tril()
+        p = p.masked_fill(~tril, 0.0)
+        dpds = dpds.masked_fill(~tril, 0.0)
+    dog = do.to(compute_dtype).reshape(B, Sq, Hkv, G, -1)
+    dv = torch.einsum("bhgst,bshgd->bthd", p, dog)
+    ds = torch.einsum("bshgd,bthd->bhgst", dog, v.to(compute_dtype)) * dpds
+    dq = torch.einsum("bhgst,bthd->bshgd", ds, k.to(compute_dtype)).reshape(B, Sq, Hq, D)
+    dk = torch.einsum("bhgst,bshgd->bthd", ds, q.to(compute_dtype).reshape(B, Sq, Hkv, G, D))
+    return dq, dk, dv
+
+
 def retention_attention(q, k, v, mask, compute_dtype=torch.float32):
     """Retention with a decay mask: s = (QK^T) * mask, out = (s / max(sum_kv |s|, 1)) V, r = that
     clamped row sum (restates ``ref_program`` of bench_utils.py:1062-1067; the running form of

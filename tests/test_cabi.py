@@ -41,8 +41,8 @@ def test_struct_layout_matches_the_header():
     # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints
     assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16
     assert ctypes.sizeof(rt.TileCfg) == 4 * 12
-    # backward: 12 pointers, 8 tensors x 3 strides, 7 + 1 ints
-    assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 12 + 8 * 24 + 4 * 8
+    # backward: 12 + 4 pointers, 8 tensors x 3 strides, 7 + 1 ints
+    assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 16 + 8 * 24 + 4 * 8
 
 
 def _compile(src, opts=()):

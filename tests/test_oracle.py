@@ -244,3 +244,23 @@ def test_softmax_gradients_match_autograd():
                                                compute_dtype=torch.float64, **kw)
         for a, b in ((dq, gq), (dk, gk), (dv, gv)):
             assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)
+
+
+def test_elementwise_gradients_match_autograd():
+    """Closed-form backward of sigmoid and relu attention against torch.autograd through the closed-form
+    forwards (fp64)."""
+    g = torch.Generator().manual_seed(6)
+    B, Sq, Skv, Hq, Hkv, D, DV = 2, 7, 11, 4, 2, 8, 6
+    q = torch.randn(B, Sq, Hq, D, generator=g, dtype=torch.float64, requires_grad=True)
+    k = torch.randn(B, Skv, Hkv, D, generator=g, dtype=torch.float64, requires_grad=True)
+    v = torch.randn(B, Skv, Hkv, DV, generator=g, dtype=torch.float64, requires_grad=True)
+    do = torch.randn(B, Sq, Hq, DV, generator=g, dtype=torch.float64)
+    for kind, fwd, kw in (("sigmoid", R.sigmoid_attention, dict(bias=-0.7, causal=True, scale=0.4)),
+                          ("sigmoid", R.sigmoid_attention, dict(bias=0.3)),
+                          ("relu", R.relu_attention, dict(scale=0.3))):
+        out = fwd(q, k, v, compute_dtype=torch.float64, **kw)
+        gq, gk, gv = torch.autograd.grad(out, (q, k, v), do)
+        dq, dk, dv = R.elementwise_attention_grads(q.detach(), k.detach(), v.detach(), do, kind,
+                                                   compute_dtype=torch.float64, **kw)
+        for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+            assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)

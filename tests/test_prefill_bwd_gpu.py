@@ -91,12 +91,46 @@ def test_softmax_backward_skips_masked_tiles(cuda_device):
         assert eng._op._plan(1, H, S, S, None).mode == 2
 
 
+def test_sigmoid_and_relu_backward(cuda_device):
+    """Graphs whose online function does nothing (attn_script/sigmoidattn.py, reluattn.py): p = f(s),
+    ds = dp f'(s) with f' from the symbolic derivative of the traced score_mod; the sigmoid's bias is a
+    scalar CustomIO tensor.  Against the oracle's closed-form gradients."""
+    g = torch.Generator().manual_seed(9)
+    for kind, causal, B, H, Hkv, S, D, dtype in (("sigmoid", True, 1, 2, 2, 300, 128, torch.float16),
+                                                 ("sigmoid", False, 2, 4, 2, 256, 64, torch.bfloat16),
+                                                 ("relu", False, 1, 3, 3, 200, 64, torch.float16)):
+        print(f"case bwd {kind} causal={causal} B{B} H{H} Hkv{Hkv} S{S} D{D} {dtype}", flush=True)
+        scale = 1 / math.sqrt(D)
+        q, k, v = C.make_inputs(B, S, S, H, Hkv, D, D, dtype, seed=21)
+        do = torch.randn(B, S, H, D, generator=g).to(dtype)
+        meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+                meta_tensor(B, Hkv, S, D, dtype=dtype))
+        if kind == "sigmoid":
+            bias = torch.tensor([-math.log(S)], dtype=torch.float32)
+            mod = AttentionEngine(meta, CustomIO({"softmax_bias": (1,)}), score_mod=C.make_sigmoid_score_mod(scale),
+                                  mask_mod=C.causal_mask if causal else None, online_func=C.OnlineIdentity())
+            extra, kw = (bias.cuda(),), dict(bias=bias.item(), causal=causal)
+        else:
+            mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_relu_score_mod(scale), mask_mod=None,
+                                  online_func=C.OnlineIdentity())
+            extra, kw = (), dict()
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        out = mod(qd, kd, vd, *extra)
+        out.backward(do.cuda())
+        dq, dk, dv = R.elementwise_attention_grads(q, k, v, do, kind, scale=scale, **kw)
+        case = (kind, causal, B, H, Hkv, S, D, dtype)
+        _check(qd.grad, dq, "dq", case)
+        _check(kd.grad, dk, "dk", case)
+        _check(vd.grad, dv, "dv", case)
+
+
 def test_backward_of_other_graphs_is_refused(cuda_device):
-    """Only graphs proven to be softmax attention have a backward; the others say so."""
+    """Softmax attention and graphs whose online function does nothing have a backward; an online function
+    that keeps other row scales (here: the running sum of |s|) says it has none."""
     B, H, S, D = 1, 2, 128, 64
     meta = (meta_tensor(B, H, S, D, dtype=torch.float16),) * 3
     mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(0.125), mask_mod=None,
-                          online_func=C.OnlineIdentity())
+                          online_func=C.OnlineAbsNorm())
     q, k, v = (t.cuda().requires_grad_(True) for t in C.make_inputs(B, S, S, H, H, D, D, torch.float16))
     with pytest.raises(NotImplementedError):
         mod(q, k, v)
