@@ -78,6 +78,9 @@ def evaluate(sym, env, memo=None):
             val = torch.log(a[0])
         elif t == "Log2":
             val = torch.log2(a[0])
+        elif t == "MaxBwd":
+            # gradient a[0] of max(x, y) with respect to x: passes where x won (zero at a tie)
+            val = torch.where(a[1] > a[2], a[0], torch.zeros_like(a[0]))
         elif t == "ReduceSum":
             val = a[0].sum(dim=-1, keepdim=True)
         elif t == "ReduceMax":

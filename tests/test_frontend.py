@@ -284,3 +284,47 @@ def test_shapes_broadcast_by_name():
     s = SymbolicArray("s", Var("s"), shape_idx=["block_M", "block_N"])
     assert (s - q).shape_idx == ["block_M", "block_N"] and (q * 2).shape_idx == ["block_M"]
     assert s.get_reduce("max").shape_idx == ["block_M"]
+
+
+def test_symbolic_derivative_matches_autograd():
+    """core.transform.autodiff.derivative on traced elementwise graphs (every node type the tracer has),
+    evaluated by the oracle's graph interpreter, against torch.autograd of the same function."""
+    from core.transform.autodiff import derivative
+    from oracle.online_interp import evaluate
+    x = torch.linspace(-2.3, 2.7, 41, dtype=torch.float64)
+    cases = [
+        (lambda s: ((s * 0.125 + 0.3) * 0.5).tanh() * 0.5 + 0.5, lambda t: torch.sigmoid(t * 0.125 + 0.3)),
+        (lambda s: (s * 0.7).max(0), lambda t: torch.relu(t * 0.7)),
+        (lambda s: (s * s + 1.5).log() / (s.exp() + 2.0), lambda t: torch.log(t * t + 1.5) / (torch.exp(t) + 2.0)),
+        (lambda s: (s * 0.4).exp2() - (s * s + 1.0).log2() - s.abs() * 0.25 + (-s) * 0.1,
+         lambda t: torch.exp2(t * 0.4) - torch.log2(t * t + 1.0) - t.abs() * 0.25 - t * 0.1),
+        (lambda s: 3.0 / (s * s + 1.0) + (2.0 - s) * s, lambda t: 3.0 / (t * t + 1.0) + (2.0 - t) * t),
+    ]
+    for traced_fn, torch_fn in cases:
+        s = SymbolScalar("scores", Var("scores"), shape_idx=[])
+        y = traced_fn(s)
+        dy = derivative(y, s)
+        got = evaluate(dy, {id(s): x})
+        t = x.clone().requires_grad_(True)
+        (want,) = torch.autograd.grad(torch_fn(t).sum(), t)
+        got = got if isinstance(got, torch.Tensor) else torch.full_like(x, float(got))
+        assert torch.allclose(got.expand_as(want), want, atol=1e-12, rtol=1e-10)
+    # no dependence -> zero
+    s, c = SymbolScalar("scores", Var("scores"), shape_idx=[]), SymbolScalar("c", Var("c"), shape_idx=[])
+    assert float(evaluate(derivative(c * 2.0, s), {id(c): 1.0})) == 0.0
+
+
+def test_elementwise_backward_lowering():
+    """The backward functors of sigmoid / relu attention are emitted; online functions that keep row
+    scales, non-scalar custom inputs and non-identity forward/backward rules are refused."""
+    from core.lower.prefill_bwd_op import lower_elementwise_backward
+    src = lower_elementwise_backward(C.make_sigmoid_score_mod(0.125), C.OnlineIdentity(),
+                                     CustomIO({"softmax_bias": (1,)}), torch.float16)
+    assert "ae_bwd_pd" in src and "cust.softmax_bias" in src and "p.custom[0]" in src
+    src = lower_elementwise_backward(C.make_relu_score_mod(0.125), C.OnlineIdentity(), CustomIO({}), torch.float16)
+    assert "> 0.0f ?" in src
+    with pytest.raises(NotImplementedError):
+        lower_elementwise_backward(C.make_scale_score_mod(0.125), C.OnlineAbsNorm(), CustomIO({}), torch.float16)
+    with pytest.raises(NotImplementedError):
+        lower_elementwise_backward(C.retention_score_mod, C.OnlineIdentity(), C.retention_custom_inputs(),
+                                   torch.float16)
