@@ -10,8 +10,9 @@ is the reference's own eager fallback (1250-1275: grouped einsum, ``tril`` mask 
 ``softmax(scores * scale)``, einsum), run on the GPU with torch.
 
 Not carried over: the external-library baselines (flash_attn, FA3, flash_sigmoid, flashinfer) --
-not installable here.  Backward exists for softmax attention (``do_bench_attention``); for the other graphs ``require_grad=True`` is accepted, the backward
-timing is skipped with a note.
+not installable here.  ``require_grad=True`` checks dq, dk, dv against autograd through the eager
+reference and times the backward for softmax, sigmoid and relu attention; the retention harness accepts
+it and skips the backward with a note.
 """
 from __future__ import annotations
 
@@ -126,6 +127,34 @@ def _report(name, latency_ms, flops):
     print("tflops: {:.2f}".format(flops / latency_ms * 1e-9))
 
 
+def _check_and_time_backward(o, do, leaves, eager_one_head, bwd_flops, name="hip bwd"):
+    """``o.backward(do)`` against autograd through an eager fp32 reference evaluated one (batch, kv head)
+    group at a time (the full score tensor of the headline shapes does not fit twice), then its timing.
+    ``leaves`` = (query, key, value) with requires_grad; ``eager_one_head(q, k, v)`` -> out for slices
+    [1, S, g, D], [1, S, 1, D], [1, S, 1, DV] in fp32."""
+    query, key, value = leaves
+    o.backward(do, retain_graph=True)
+    got = [t.grad.clone() for t in leaves]
+    for t in leaves:
+        t.grad = None
+    want = [torch.zeros_like(t) for t in leaves]
+    g = query.shape[2] // key.shape[2]
+    for b0 in range(query.shape[0]):
+        for h0 in range(key.shape[2]):
+            qs = query[b0:b0 + 1, :, h0 * g:(h0 + 1) * g].detach().float().requires_grad_(True)
+            ks = key[b0:b0 + 1, :, h0:h0 + 1].detach().float().requires_grad_(True)
+            vs = value[b0:b0 + 1, :, h0:h0 + 1].detach().float().requires_grad_(True)
+            eager_one_head(qs, ks, vs).backward(do[b0:b0 + 1, :, h0 * g:(h0 + 1) * g].float())
+            want[0][b0:b0 + 1, :, h0 * g:(h0 + 1) * g] = qs.grad.to(query.dtype)
+            want[1][b0:b0 + 1, :, h0:h0 + 1] = ks.grad.to(key.dtype)
+            want[2][b0:b0 + 1, :, h0:h0 + 1] = vs.grad.to(value.dtype)
+    for a_, b_ in zip(got, want):
+        print_debug(a_, b_, rtol=1e-2, atol=1e-2)
+    latency = do_bench(lambda: o.backward(do, retain_graph=True), warmup=50, rep=100)
+    _report(name, latency, bwd_flops)
+    return latency
+
+
 def do_bench_attention(attn, B, H, S, D, DV, mod=None, dtype=torch.float16, seqlenq=None,
                        require_grad=False, causal=True, groupnum=None):
     """Softmax attention (MHA / GQA / decode): correctness print-out against the eager reference,
@@ -189,15 +218,22 @@ def do_bench_sigmoidattn(attn, B, H, S, D, DV, dtype=torch.float16, requires_gra
     tflops = (2 * B * H * S * S * D + 2 * B * H * S * S * DV) * (0.5 if causal else 1.0)
     torch.cuda.manual_seed(0)
     device = "cuda"
-    query = torch.randn(B, S, H, D, device=device, dtype=dtype)
-    key = torch.randn(B, S, H, D, device=device, dtype=dtype)
-    value = torch.randn(B, S, H, DV, device=device, dtype=dtype)
-    torch.randn(B, S, H, DV, device=device, dtype=dtype)
+    query = torch.randn(B, S, H, D, device=device, dtype=dtype, requires_grad=requires_grad)
+    key = torch.randn(B, S, H, D, device=device, dtype=dtype, requires_grad=requires_grad)
+    value = torch.randn(B, S, H, DV, device=device, dtype=dtype, requires_grad=requires_grad)
+    do = torch.randn(B, S, H, DV, device=device, dtype=dtype)
     softmax_bias = 0.1 * torch.randn(1, device=device, dtype=torch.float32)
 
     o = attn(query, key, value, softmax_bias)
     if requires_grad:
-        print("forward-only build: backward check and timing skipped")
+        def one_head(qs, ks, vs):
+            sc = torch.einsum("bqhd,bkhd->bhqk", qs, ks)
+            pr = torch.sigmoid(sc + softmax_bias)
+            if causal:
+                pr = pr.masked_fill(~torch.ones(S, S, device=device, dtype=torch.bool).tril(), 0.0)
+            return torch.einsum("bhqk,bkhd->bqhd", pr, vs)
+        _check_and_time_backward(o, do, (query, key, value), one_head, 2.5 * tflops)
+        query, key, value = query.detach(), key.detach(), value.detach()
 
     def ref():
         out = torch.empty_like(o)
@@ -222,14 +258,20 @@ def do_bench_reluattn(attn, B, H, S, D, DV, dtype=torch.float16, causal=False, r
     tflops = (2 * B * H * S * S * D + 2 * B * H * S * S * DV) * (0.5 if causal else 1.0)
     torch.cuda.manual_seed(0)
     device = "cuda"
-    query = torch.randn(B, S, H, D, device=device, dtype=dtype)
-    key = torch.randn(B, S, H, D, device=device, dtype=dtype)
-    value = torch.randn(B, S, H, DV, device=device, dtype=dtype)
-    torch.randn(B, S, H, DV, device=device, dtype=dtype)
+    query = torch.randn(B, S, H, D, device=device, dtype=dtype, requires_grad=requires_grad)
+    key = torch.randn(B, S, H, D, device=device, dtype=dtype, requires_grad=requires_grad)
+    value = torch.randn(B, S, H, DV, device=device, dtype=dtype, requires_grad=requires_grad)
+    do = torch.randn(B, S, H, DV, device=device, dtype=dtype)
 
     o = attn(query, key, value)
     if requires_grad:
-        print("forward-only build: backward check and timing skipped")
+        def one_head(qs, ks, vs):
+            pr = F.relu(torch.einsum("bqhd,bkhd->bhqk", qs, ks) / (D ** 0.5))
+            if causal:
+                pr = pr.masked_fill(~torch.ones(S, S, device=device, dtype=torch.bool).tril(), 0.0)
+            return torch.einsum("bhqk,bkhd->bqhd", pr, vs)
+        _check_and_time_backward(o, do, (query, key, value), one_head, 2.5 * tflops)
+        query, key, value = query.detach(), key.detach(), value.detach()
 
     def ref_program():
         qk = torch.einsum("bqhd,bkhd->bhqk", query, key) / (D ** 0.5)
