@@ -91,6 +91,25 @@ def test_softmax_backward_skips_masked_tiles(cuda_device):
         assert eng._op._plan(1, H, S, S, None).mode == 2
 
 
+def test_backward_odd_shapes_against_oracle(cuda_device):
+    """Seeded sweep: ragged sequence lengths (also Sq != Skv without a mask), grouped heads, both head
+    dims for keys and values, both dtypes, no mask / causal / sliding window / head-dependent masks."""
+    import random
+    rng = random.Random(2024)
+    masks = [(None, False), (C.causal_mask, True), (C.make_sliding_window_mask(53), False),
+             (C.head_dependent_mask, False)]
+    for n in range(14):
+        hkv = rng.choice([1, 2, 3])
+        B, H = rng.choice([1, 2]), hkv * rng.choice([1, 2, 4])
+        D, DV = rng.choice([64, 128]), rng.choice([64, 128])
+        dtype = torch.float16 if n % 2 == 0 else torch.bfloat16
+        mask_mod, causal = masks[n % len(masks)]
+        Sq = rng.randint(1, 450)
+        Skv = Sq if mask_mod is not None else rng.randint(1, 450)
+        print(f"case bwd odd B{B} H{H} Hkv{hkv} Sq{Sq} Skv{Skv} D{D} DV{DV} {dtype} mask {n % len(masks)}", flush=True)
+        _run(B, H, hkv, Sq, Skv, D, DV, dtype, mask_mod, causal, seed=300 + n)
+
+
 def test_sigmoid_and_relu_backward(cuda_device):
     """Graphs whose online function does nothing (attn_script/sigmoidattn.py, reluattn.py): p = f(s),
     ds = dp f'(s) with f' from the symbolic derivative of the traced score_mod; the sigmoid's bias is a
