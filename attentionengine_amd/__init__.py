@@ -1,4 +1,5 @@
-"""MI355X-native implementation of AttentionEngine's fused attention forward path.
+"""MI355X-native implementation of AttentionEngine's fused attention path (forward, and the backward of
+softmax, sigmoid and relu attention).
 
 The reference puts ``attention_engine/`` on PYTHONPATH so that ``attn_engine``, ``core`` and
 ``benchmark`` are top-level packages (README.md:50) and its scripts import them by those names

@@ -47,12 +47,14 @@ class OnlineFunc:
 
     @staticmethod
     def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
-        """Recompute rule for the backward pass (unused by this forward-only build)."""
+        """Recompute rule of the backward pass, p from the modified scores and the final row scales.  The
+        backward checks that it is the identity for online functions without row scales; for softmax
+        attention the gradient is fixed by the proven forward and the rule is not traced."""
         return scores
 
     @staticmethod
     def backward(dp, scores, final_rowscales, b, h, q_idx, kv_idx):
-        """Backward rule (unused by this forward-only build)."""
+        """Backward rule, dscores from dp (see ``forward``)."""
         return dp
 
     @staticmethod

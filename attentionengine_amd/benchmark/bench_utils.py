@@ -1,6 +1,6 @@
 """Benchmark / comparison harness the example scripts call.
 
-Drop-in counterpart of attention_engine/benchmark/bench_utils.py for the forward path: same
+Drop-in counterpart of attention_engine/benchmark/bench_utils.py: same
 function names, arguments and printed quantities for ``do_bench`` (14-99), ``check_close``
 (133-155), ``print_debug`` (158-192), ``do_bench_attention`` (1179-1360),
 ``do_bench_sigmoidattn`` (701-788) and ``do_bench_reluattn`` (949-1022).  Inputs are generated

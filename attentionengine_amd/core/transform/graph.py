@@ -18,7 +18,7 @@ class Node:
         self.grad = None
 
     def backward(self, grad=None):
-        raise NotImplementedError("symbolic differentiation is outside the forward-only build")
+        raise NotImplementedError("use core.transform.autodiff.derivative(out, wrt): the derivative as a traced expression")
 
     def __str__(self):
         return f"{self.type}(" + "".join(f"{n}, " for n in self.inputs) + ")"

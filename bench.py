@@ -1,4 +1,4 @@
-"""Benchmark of the fused attention forward path on one MI355X.
+"""Benchmark of the fused attention path (forward; one extra workload for the backward) on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extra] [--no-cpu]
 

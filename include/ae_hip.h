@@ -1,6 +1,6 @@
 /*
  * ae_hip.h -- C ABI of libae_hip.so, the native boundary of the MI355X (gfx950)
- * attention-forward path.
+ * attention path (forward launches and the backward of the prefill shapes).
  *
  * What it replaces in the reference (microsoft/AttentionEngine):
  *   - the TileLang JIT boundary `tl.compile(prim_func, out_idx=[...])` that turns a

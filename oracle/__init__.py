@@ -1,4 +1,4 @@
-"""CPU oracle for the attention-forward path.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle for the attention path (forward results and gradients).  TEST INFRASTRUCTURE ONLY.
 
 Nothing in the product (the ``attentionengine_amd`` package) imports this package; only
 ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` do, and only
