@@ -59,7 +59,12 @@
 #define AE_NDB2 (AE_DV / 32)       // ... of dV
 #define AE_L1 ((AE_BS * AE_CPR1) / AE_NT)   // 1 KiB load instructions per wave and tile
 #define AE_L2 ((AE_BS * AE_CPR2) / AE_NT)
-#define AE_NSTAGE 3                // a tile is requested two iterations before it is multiplied
+#ifndef AE_NSTAGE
+#define AE_NSTAGE 3                // LDS stages: a tile is requested AE_NSTAGE - 1 iterations before it is multiplied
+#endif
+#ifndef AE_BWD_WAVES_PER_EU
+#define AE_BWD_WAVES_PER_EU 1
+#endif
 #define AE_NLOADS (AE_L1 + AE_L2 + (AE_BWD_ROLE == 1 ? 1 : 0))   // load instructions per wave and tile
 #define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 #ifndef AE_AHEAD
@@ -96,7 +101,8 @@ AE_DEV int ae_bwd_chunk_pos(int r, int c) {
 #define AE_BWD_KERNEL ae_bwd_dkv_kernel
 #endif
 
-extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(1, 1)))
+static_assert(AE_NSTAGE == 2 || AE_NSTAGE == 3, "two or three stages");
+extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(AE_BWD_WAVES_PER_EU, AE_BWD_WAVES_PER_EU)))
 void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
   ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // AE_NSTAGE stages of [tile 1][tile 2][lse][delta]
@@ -328,14 +334,15 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   int x0 = next_item(0), x1 = next_item(x0 + 1), x2 = next_item(x1 + 1);
   if (x0 < n_items) {
     request_item(x0, 0);
-    request_item(x1, 1);
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // the first item has landed
+    if (AE_NSTAGE == 3) request_item(x1, 1);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT((AE_NSTAGE - 2) * AE_NLOADS));   // the first item has landed
   }
   __syncthreads();
 
   for (int n = 0; x0 < n_items; n++) {
     const int it = x0;
-    request_item(x2, (n + 2) % AE_NSTAGE);   // into the stage everyone left at the last barrier
+    // into the stage everyone left at the last barrier
+    request_item(AE_NSTAGE == 3 ? x2 : x1, (n + AE_NSTAGE - 1) % AE_NSTAGE);
     const ae_lds_byte* t1 = lds + (n % AE_NSTAGE) * AE_STAGE_BYTES;
     const ae_lds_byte* t2 = t1 + AE_T1_BYTES;
     const int s0 = item_tile(it) * AE_BS;
@@ -468,7 +475,8 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     }
     (void)pf;
 
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_NLOADS));   // the next item has landed (only the one after it is outstanding)
+    // the next item has landed (with three stages the one after it is still outstanding)
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT((AE_NSTAGE - 2) * AE_NLOADS));
     __syncthreads();
     x0 = x1;
     x1 = x2;
