@@ -138,9 +138,6 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // Q has landed
     __syncthreads();                           // tile 0 has landed
 
-#ifdef AE_SCORE_PRIO
-    __builtin_amdgcn_s_setprio(AE_SCORE_PRIO);
-#endif
     // K fragment of k-step ks: row lane%32, global chunk 2*ks + lane/32
     const int k_row_off = l32s * AE_KSTR;
     const int k_sw = AE_SWZ(l32s);
