@@ -482,7 +482,8 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
   if (p->heads_q % p->heads_kv != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: Hq=%d is not a multiple of Hkv=%d", p->heads_q,
                 p->heads_kv);
-  if (cfg->block_m != 128 || cfg->block_n != 64 || cfg->threads != 256 || cfg->lds_bytes <= 0 ||
+  // block_m / threads describe the dq launch (4 or 8 waves of 32 resident rows); dk/dv always runs 4 waves
+  if ((cfg->block_m != 128 && cfg->block_m != 256) || cfg->block_n != 64 || cfg->threads != 2 * cfg->block_m || cfg->lds_bytes <= 0 ||
       cfg->lds_bytes > 160 * 1024 || cfg->head_dim_v <= 0 || cfg->head_dim_v % 8 != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: bad tile configuration (bm=%d bn=%d threads=%d lds=%d dv=%d)",
                 cfg->block_m, cfg->block_n, cfg->threads, cfg->lds_bytes, cfg->head_dim_v);
@@ -498,7 +499,7 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
   const uint64_t g_delta = (rows + rows_per_wg - 1) / rows_per_wg;
   // ids are 8*slot + xcd, slot = tile*ceil(batch*heads/8) + head group (see ae_prefill_bwd.hip)
   const uint64_t g_dkv = (((uint64_t)p->seqlen_kv + 127) / 128) * ((((uint64_t)p->batch * p->heads_kv) + 7) / 8) * 8;
-  const uint64_t g_dq = (((uint64_t)p->seqlen_q + 127) / 128) * ((((uint64_t)p->batch * p->heads_q) + 7) / 8) * 8;
+  const uint64_t g_dq = (((uint64_t)p->seqlen_q + cfg->block_m - 1) / cfg->block_m) * ((((uint64_t)p->batch * p->heads_q) + 7) / 8) * 8;
   if (g_delta > 0x7fffffffull || g_dkv > 0x7fffffffull || g_dq > 0x7fffffffull)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: grid too large");
   uint32_t block[3] = {256, 1, 1};
@@ -509,6 +510,7 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
   rc = ae_launch(dkv, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
   if (rc) return rc;
   grid[0] = (uint32_t)g_dq;
+  block[0] = (uint32_t)cfg->threads;
   return ae_launch(dq, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
 }
 

@@ -247,10 +247,11 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
  * ae_prefill_bwd: backward of softmax attention. Three launches on `stream`: `delta`
  *   (rowsum(dout*out), the reference's flashattn_bwd_preprocess, attn_tl.py:196-221), `dkv` (one
  *   workgroup per 128 kv rows of a (batch, kv head): dk and dv, summed over the q heads of the group)
- *   and `dq` (one workgroup per 128 q rows of a (batch, q head)). The reference's single backward
+ *   and `dq` (one workgroup per cfg->block_m q rows of a (batch, q head)). The reference's single backward
  *   kernel with fp32 atomics on dq and its postprocess (attn_tl.py:238-455) are replaced by these two
- *   atomic-free launches. cfg: block_m = 128, block_n = 64, threads = 256 and the dynamic LDS of the
- *   compiled kernels, mask_mode as compiled (2 needs the two tile-class tables: 0 skip, 1 test per
+ *   atomic-free launches. cfg describes the dq launch: block_m = 128 with threads = 256, or block_m = 256
+ *   with threads = 512 for a dq kernel compiled with AE_BWD_NWAVES 8 (dkv always runs 256 threads);
+ *   block_n = 64 and the dynamic LDS of the compiled kernels, mask_mode as compiled (2 needs the two tile-class tables: 0 skip, 1 test per
  *   element, 2 fully visible); head dims as compiled. All gradients are written in full (no accumulation).
  *   The same three launches serve the graphs whose online function does nothing (sigmoid, relu attention:
  *   kernels compiled with AE_BWD_KIND 1 and the generated derivative of score_mod; lse is NULL then).
