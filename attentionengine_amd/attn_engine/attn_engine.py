@@ -102,10 +102,8 @@ class AttentionEngine:
         dtype_map[q_meta.dtype]  # KeyError for unsupported dtypes, as in the reference (225-228, 304)
         q_seqlen, kv_len = q_meta.shape[2], v_meta.shape[2]
         head, head_kv = q_meta.shape[1], v_meta.shape[1]
-        for dim in (q_meta.shape[0], head, head_kv, q_seqlen, kv_len):
-            if isinstance(dim, str):
-                # dynamic extents are runtime parameters of the kernels; the meta value is a hint
-                continue
+        # dynamic (string) extents are runtime parameters of the kernels; they only rule out the
+        # shape-dependent dispatch to the decode templates
         dynamic = any(isinstance(d, str) for m in qkv_meta for d in m.shape)
 
         if kv_shared:

@@ -127,6 +127,20 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
 LAZY_MAX_TAU = 8.0 * 0.6931471805599453
 
 
+def is_plain_softmax(m_new, new_scores, scores_mod) -> bool:
+    """True when the graph ``find_lazy_softmax`` accepted is exactly the online softmax OF scores_mod:
+    ``m_new = max(m, rowmax(scores_mod))`` and ``scores' = exp(scores_mod - m_new)``.  The wider class
+    (any per-row x inside the max, anything with a kv axis in front of ``- m_new``) is still
+    independent of the reference point, so it may use the lazy maximum, but only this case may run
+    the kernels that hard-code ``exp(c * S - m)`` or the softmax backward."""
+    try:
+        x = m_new.prev[1]
+        return (x.code.type == "ReduceMax" and x.prev[0] is scores_mod
+                and new_scores.prev[0].prev[0] is scores_mod)
+    except (IndexError, AttributeError):
+        return False
+
+
 def find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale):
     """Return the ``m_new = max(m, x)`` symbol if the traced online function is the online softmax
     (attn_script/mha.py:47-72), whose outputs do not depend on the reference point m:
@@ -257,8 +271,11 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     softmax = None
     if lazy is not None:
         em.lazy_max[id(lazy)] = LAZY_MAX_TAU
-        scale = _pure_scale(scores_mod, scores)
-        if scale is not None and scale > 0.0 and math.isfinite(scale):
+        scale = _pure_scale(scores_mod, scores) if is_plain_softmax(lazy, new_scores, scores_mod) else None
+        # the specialised kernels start every row from m = -inf (lower.py:23-29: -1e38) and r = 0
+        init = {k: float(init_literal(v.code.name).rstrip("f")) for k, v in rowscales.items()}
+        inits_ok = all((v <= -1e30) if new_rowscales[k] is lazy else (v == 0.0) for k, v in init.items())
+        if scale is not None and inits_ok and scale > 0.0 and math.isfinite(scale):
             (mk,) = [k for k, v in new_rowscales.items() if v is lazy]
             (rk,) = [k for k in new_rowscales if k != mk]
             softmax = (scale, mk, rk)
@@ -432,6 +449,11 @@ def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, h
     if softmax is not None:
         extra = [f"#define AE_SM_SCALE {float_literal(softmax[0])}", f"#define AE_SM_M {softmax[1]}",
                  f"#define AE_SM_R {softmax[2]}"]
+        # The pipelined kernel folds the score scale into its fp16 Q fragments (one rounding of q*c*log2e
+        # to fp16: a score moves by about 2^-12 of its size, i.e. lse by < 1e-3 while |score*c| stays below
+        # ~20).  AE_PREFILL_PRESCALE=0 keeps Q as it is and multiplies every score in fp32 instead.
+        if os.environ.get("AE_PREFILL_PRESCALE", "") in ("0", "1"):
+            extra.append(f"#define AE_PRESCALE {os.environ['AE_PREFILL_PRESCALE']}")
     return "\n".join([
         "// generated by core/lower/lower.py -- do not edit",
         f"#define AE_D {d}",

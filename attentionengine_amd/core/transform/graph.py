@@ -4,8 +4,9 @@ Same public names and ``type`` strings as the reference's
 attention_engine/core/transform/graph.py:2-243 (Var, Const, Add, Mul, Neg, Sub, Div, Exp, Exp2,
 Log, Log2, Tanh, Abs, Max, MaxBwd, ReduceSum, ReduceMax, ReduceAbsSum, ColReduceMax,
 ColReduceSum, ColReduceAbsSum).  The HIP functor emitter and the CPU interpreter dispatch on
-``Node.type``.  Only the forward vocabulary is implemented: the reference's per-node
-``_backward`` rules belong to the backward pass, which this build does not cover.
+``Node.type``.  The reference's per-node ``_backward`` rules (graph.py:2-243, driven by
+SymbolScalar.backward, core.py:119-199) are replaced by one function,
+core.transform.autodiff.derivative, which returns the derivative as a traced expression.
 """
 
 

@@ -16,17 +16,24 @@
 // 32x32x16 MFMA keeps the matrix pipe busy for 32 cycles but the wave's issue port for only about 16,
 // v_exp_f32 costs 8; so the rest of an MFMA's time is free for independent VALU work.  One loop
 // iteration therefore interleaves, MFMA by MFMA,
-//     phase 1:  S(j+1) = K(j+1) Q^T   with   p(j) = exp2(s(j)*c*log2e - m*log2e), row sums, fp16 cast
-//     phase 2:  O += V(j)^T p(j)^T     with   reading S(j+1) out of its accumulators, row maxima
-// with `sched_barrier` fences pinning the interleaving, the exponentiation split into stages (fma,
-// exp2, pack + sum) that run in different MFMA slots so no instruction waits for the one just
-// issued, A fragments read from LDS a few MFMAs ahead of their use into a small register ring, and
-// the tile loads (HBM -> LDS direct) issued as two bursts from phase-1 slots.
-// The rescale of O happens outside the hot loop (lazy running maximum: it is rare).
+//     phase 1:  x(j+1) = K(j+1) Q'^T - m2   with   p(j) = exp2(x(j)), row sums, fp16 cast
+//     phase 2:  O += V(j)^T p(j)^T          with   reading x(j+1) out of its accumulators, row maxima
+// with `sched_barrier` fences pinning the interleaving, the exponentiation split into stages (exp2,
+// pack + sum) that run in different MFMA slots so no instruction waits for the one just issued, A
+// fragments read from LDS a few MFMAs ahead of their use into a small register ring, and the tile
+// loads (HBM -> LDS direct) issued as two bursts from phase-1 slots.
+// The loop is bound by the number of instructions a wave issues per tile, so what can leave the loop
+// has left it: for fp16 the Q fragments are multiplied by c*log2e once (Q' above; the rounding of the
+// product to fp16 moves a score by about 2^-12 of its size, inside the 1e-3 bar on lse for scores up
+// to a few tens) and the row's reference -m2 enters as the C operand of the first k-step, so the MFMA
+// result IS the exponent; bf16 (8 significant bits) keeps one fma per score instead.  The reference is
+// lazy: it moves only when a tile exceeds it by more than 8 (p < 256), and then a cold path shifts the
+// tile, rescales the running sum and leaves the loop so that O is rescaled outside it.
 //
 // Configuration ("ae_config.h"): AE_D AE_DV AE_BN(=64) AE_NWAVES AE_DTYPE_BF16 AE_MASK_MODE
 // AE_HAS_MASK_MOD AE_N_ROWSCALES AE_EVEN_Q AE_EVEN_KV, plus AE_SM_SCALE (the constant c > 0) and
-// AE_SM_M / AE_SM_R (names of the running-max and running-sum fields of ae_rowstate).
+// AE_SM_M / AE_SM_R (names of the running-max and running-sum fields of ae_rowstate, which the
+// lowering has checked to start at -inf and 0).
 // Functors used ("ae_functors.h"): ae_rowstate, ae_rowstate_init, ae_mask_mod, ae_epilogue,
 // ae_load_custom.
 
@@ -68,18 +75,16 @@
 #define AE_VLOAD_SLOT (AE_NKF + 7)
 #endif
 #define AE_TAU 5.545177444479562f  // 8 ln 2: the running maximum is refreshed only when it moved by more
-
-static_assert(AE_BN == 64, "the pipelined kernel is written for 64-wide kv tiles");
-static_assert(AE_D == 64 || AE_D == 128, "head dim 64 or 128");
-static_assert(AE_DV == 64 || AE_DV == 128, "value head dim 64 or 128");
-static_assert((AE_BN * AE_KCPR) % AE_NT == 0 && (AE_BN * AE_VCPR) % AE_NT == 0, "tile / workgroup split");
-static_assert(AE_VPS2 >= 2, "work split");
-static_assert(AE_K_LOADS >= 1 && AE_K_LOADS <= 8 && AE_V_LOADS >= 1 && AE_V_LOADS <= 8, "one burst per tile and wave");
-// k-step kk of O^T += V^T P^T starts in slot 2*NKF + 2*NDB*kk; its last unit (8*kk+7) must be done
-static_assert(((7 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF, "exp units of k-step 0 finish in phase 1");
-static_assert(((31 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 6 * AE_NDB, "exp units of k-step 3 finish in time");
-static_assert(((23 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 4 * AE_NDB, "exp units of k-step 2 finish in time");
-static_assert(((15 * AE_EXP_SPAN) / 32) + 2 < 2 * AE_NKF + 2 * AE_NDB, "exp units of k-step 1 finish in time");
+// 1: an iteration ends by requesting the next one's first LDS fragments and compares the new tile's maxima
+// with the reference while they travel; 0: it starts with the requests.  Measured on B2 H32 S4096 D128:
+// 1 is 3.5 % faster without a mask, 0 is 2 % faster under a causal mask (set by the lowering).
+#ifndef AE_TOP_PREFETCH
+#define AE_TOP_PREFETCH (AE_MASK_MODE == 0)
+#endif
+// 1: Q carries c*log2e and the reference is the C operand of the first k-step (see above)
+#ifndef AE_PRESCALE
+#define AE_PRESCALE (!AE_DTYPE_BF16)
+#endif
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 #define AE_SB() __builtin_amdgcn_sched_barrier(0)
@@ -141,7 +146,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
     const ae_elem* qptr = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)qr * p.q_stride_s +
                           (int64_t)h * p.q_stride_h;
 #pragma unroll
-    for (int ks = 0; ks < AE_NKS; ks++) qf[qb][ks] = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
+    for (int ks = 0; ks < AE_NKS; ks++) {
+      ae_elem8 t = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
+#if AE_PRESCALE
+#pragma unroll
+      for (int i = 0; i < 8; i++) t[i] = (ae_elem)((float)t[i] * (AE_SM_SCALE * AE_LOG2E));
+#endif
+      qf[qb][ks] = t;
+    }
   }
 
   // ---- KV tile range and tile classes --------------------------------------------------------
@@ -263,7 +275,24 @@ void ae_prefill_kernel(const ae_attn_params p) {
   ae_custom cust[2];
   ae_rowstate st[2];
   ae_f32x16 oacc[2][AE_NDB];
-  float m_run[2], r_run[2], negm2[2], osc[2];
+  // Scores leave the MFMAs already as the exponent of p:  x = s*c*log2e - m2.  With AE_PRESCALE the Q
+  // fragments carry the factor c*log2e and -m2 is the C operand of the first k-step (16 equal registers
+  // per q block, `negc`, kept in the accumulator file and rewritten only when the reference moves), so no
+  // instruction touches a score between the MFMA and v_exp.  m2 is the row's reference in log2 units;
+  // thr is what a tile maximum (relative to the reference) must exceed before the reference moves: 8
+  // (p stays below 256), or -inf while the row has not seen a visible key and its reference is unset.
+  float m2[2], r_run[2], thr[2];
+  ae_f32x16 negc[2];
+  ae_elem8 zero8;
+#pragma unroll
+  for (int i = 0; i < 8; i++) zero8[i] = (ae_elem)0.f;
+  // a value DEFINED by an MFMA lives in the accumulator file: splat(v) + 0*0
+  auto acc_splat = [&](float v) -> ae_f32x16 {
+    ae_f32x16 t;
+#pragma unroll
+    for (int r = 0; r < 16; r++) t[r] = v;
+    return ae_mfma32(zero8, zero8, t);
+  };
 #pragma unroll
   for (int qb = 0; qb < 2; qb++) {
     ctx[qb].b = b;
@@ -272,10 +301,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
     ctx[qb].kv_base = 0;
     ae_load_custom(cust[qb], p, ctx[qb]);
     ae_rowstate_init(st[qb]);
-    m_run[qb] = st[qb].AE_SM_M;
-    r_run[qb] = st[qb].AE_SM_R;       // per-lane partial sum; the two halves of a row meet in the epilogue
-    negm2[qb] = 0.f;
-    osc[qb] = 1.f;
+    m2[qb] = 0.f;
+    thr[qb] = AE_NEG_INF;
+    r_run[qb] = 0.f;                  // per-lane partial sum; the two halves of a row meet in the epilogue
+    negc[qb] = acc_splat(0.f);
 #pragma unroll
     for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
@@ -307,13 +336,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
   };
 
   ae_f32x16 sacc[2][2];     // [kv block][q block] accumulators of the tile being multiplied
-  float sv[2][32];          // [q block][score]: the tile being exponentiated (raw scores, masked)
-  float mx[2];              // lane-local maxima of sv
-  ae_elem8 pf[2][4];        // [q block][k-step] P^T fragments (B operand of O^T += V^T P^T)
+  float sv[2][32];          // [q block][score]: exponents x of the tile being exponentiated (masked)
+  float mx[2];              // lane-local maxima of the tile being multiplied
+  ae_u32x4 pf[2][4];        // [q block][k-step] P^T fragments (B operand of O^T += V^T P^T), as packed pairs
   ae_elem8 ring[AE_RING];
   bool rescale = false;
+  float osc[2];             // factors of a pending rescale of O
 
-  // read S out of its accumulators (q block qb, scores e0 .. e0+n-1) and track the maximum
+  // read x out of its accumulators (q block qb, scores e0 .. e0+n-1) and track the maximum
   auto read_scores = [&](int qb, int e0, int n) {
 #pragma unroll
     for (int e = e0; e < e0 + n; e++) {
@@ -325,16 +355,23 @@ void ae_prefill_kernel(const ae_attn_params p) {
       mx[qb] = __builtin_fmaxf(mx[qb], x);
     }
   };
-  // p = exp2(s*c*log2e - m*log2e), two scores at a time ("unit" u: q block u%2, k-step u/8, pair
-  // (u/2)%4 of that k-step's 8 scores), in three stages that run in DIFFERENT MFMA slots so that no
-  // instruction waits for the one just issued: A = fma, B = exp2, C = convert + row sum.  Unit u
-  // starts in slot ae_unit_slot(u); units are ordered by k-step, the order O^T += V^T P^T needs them.
+  // p = exp2(x), two scores at a time ("unit" u: q block u%2, k-step u/8, pair (u/2)%4 of that k-step's 8
+  // scores), in stages that run in DIFFERENT MFMA slots so that no instruction waits for the one just
+  // issued: A = (without AE_PRESCALE) the fma that turns a raw score into x, B = exp2, C = convert + row
+  // sum.  Unit u starts in slot (u * AE_EXP_SPAN) / 32; units are ordered by k-step, the order
+  // O^T += V^T P^T needs them.
   float rsum[2];
   float xa[32][2];
+  float negm2[2] = {0.f, 0.f};
   auto stage_a = [&](int u) {
     const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
+#if AE_PRESCALE
+    xa[u][0] = sv[qb][e];
+    xa[u][1] = sv[qb][e + 1];
+#else
     xa[u][0] = __builtin_fmaf(sv[qb][e], AE_SM_SCALE * AE_LOG2E, negm2[qb]);
     xa[u][1] = __builtin_fmaf(sv[qb][e + 1], AE_SM_SCALE * AE_LOG2E, negm2[qb]);
+#endif
   };
   auto stage_b = [&](int u) {
     xa[u][0] = ae_exp2(xa[u][0]);
@@ -342,17 +379,16 @@ void ae_prefill_kernel(const ae_attn_params p) {
   };
   auto stage_c = [&](int u) {
     const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
-    const ae_elem h0 = (ae_elem)xa[u][0], h1 = (ae_elem)xa[u][1];
-    pf[qb][e >> 3][e & 7] = h0;
-    pf[qb][e >> 3][(e & 7) + 1] = h1;
+    typedef float ae_f32x2 __attribute__((ext_vector_type(2)));
+    const ae_f32x2 x2 = {xa[u][0], xa[u][1]};
+    const ae_elem2 hv = __builtin_convertvector(x2, ae_elem2);   // one packed conversion, round to nearest
+    pf[qb][e >> 3][(e & 7) >> 1] = __builtin_bit_cast(unsigned, hv);
 #if AE_DTYPE_BF16
     // bf16 keeps 8 significant bits: summing the rounded values would put ~1e-3 into lse for rows
     // with few visible keys, so the fp32 values are summed (fp16 sums the rounded pairs in one v_dot2)
     rsum[qb] += xa[u][0] + xa[u][1];
 #else
-    typedef _Float16 ae_h2 __attribute__((ext_vector_type(2)));
-    ae_h2 hv = {h0, h1};
-    ae_h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+    const ae_elem2 one = {(_Float16)1.0f, (_Float16)1.0f};
     rsum[qb] = __builtin_amdgcn_fdot2(hv, one, rsum[qb], false);
 #endif
   };
@@ -373,7 +409,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
     for (int u = 0; u < 32; u++) stage_c(u);
   };
-  // mask fix-up of sv for tile j, then the row maxima, the (lazy) running maximum and the factors
+  // Tile j sits in sv, its lane-local maxima in mx: mask fix-up where the tile needs it, then the
+  // row maxima against the (lazy) reference.  The common case ends after two exchanges and a ballot; a
+  // row whose maximum exceeds its threshold moves its reference (cold path): sv is shifted, the
+  // running sum rescaled here, O before the next iteration (rescale_o, outside the hot loop).
   auto finish_scores = [&](int j) {
     const int kvb = j * AE_BN + 4 * hf;
     if (needs_mask(j)) {
@@ -403,25 +442,45 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #if !AE_EVEN_KV
           vis = vis && (kv < p.seqlen_kv);
 #endif
-          sv[qb][e] = vis ? sv[qb][e] : AE_NEG_INF;
-          mx[qb] = __builtin_fmaxf(mx[qb], sv[qb][e]);
+          const float x = vis ? sv[qb][e] : AE_NEG_INF;
+          sv[qb][e] = x;
+          mx[qb] = __builtin_fmaxf(mx[qb], x);
         }
       }
     }
+    float tmax[2];
     bool any_need = false;
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) {
       float hi;
       const float lo = ae_swap32_lo_hi(mx[qb], hi);
-      const float sc = __builtin_fmaxf(lo, hi) * AE_SM_SCALE;
-      const bool need = (sc - m_run[qb]) > AE_TAU;
-      const float mn = need ? sc : m_run[qb];
-      osc[qb] = need ? ae_exp(m_run[qb] - mn) : 1.0f;
-      m_run[qb] = mn;
-      negm2[qb] = -mn * AE_LOG2E;
-      any_need = any_need || need;
+#if AE_PRESCALE
+      tmax[qb] = __builtin_fmaxf(lo, hi);                              // relative to the reference, log2 units
+#else
+      tmax[qb] = __builtin_fmaf(__builtin_fmaxf(lo, hi), AE_SM_SCALE * AE_LOG2E, negm2[qb]);
+#endif
+      any_need = any_need || (tmax[qb] > thr[qb]);
     }
     rescale = __builtin_amdgcn_ballot_w64(any_need) != 0;
+    if (__builtin_expect(rescale, 0)) {
+#pragma unroll
+      for (int qb = 0; qb < 2; qb++) {
+        const bool need = tmax[qb] > thr[qb];
+        const float d = need ? tmax[qb] : 0.f;
+        // a row whose reference was unset has O = 0 and r = 0: any finite factor will do
+        osc[qb] = (need && thr[qb] > AE_NEG_INF) ? ae_exp2(-d) : 1.0f;
+        thr[qb] = need ? AE_TAU * AE_LOG2E : thr[qb];
+        m2[qb] += d;
+        r_run[qb] *= osc[qb];
+#if AE_PRESCALE
+#pragma unroll
+        for (int e = 0; e < 32; e++) sv[qb][e] -= d;
+        negc[qb] = acc_splat(-m2[qb]);
+#else
+        negm2[qb] = -m2[qb];
+#endif
+      }
+    }
   };
 
   // ---- prologue: first tile's scores ------------------------------------------------------------
@@ -441,12 +500,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
       const ae_elem8 kf = read_kfrag(f, lds);
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
-        ae_f32x16 c = sacc[f & 1][qb];
-        if (f < 2) {
-#pragma unroll
-          for (int r = 0; r < 16; r++) c[r] = 0.f;
-        }
-        sacc[f & 1][qb] = ae_mfma32(kf, qf[qb][f >> 1], c);
+        sacc[f & 1][qb] = ae_mfma32(kf, qf[qb][f >> 1], f < 2 ? negc[qb] : sacc[f & 1][qb]);
       }
     }
     mx[0] = mx[1] = AE_NEG_INF;
@@ -461,6 +515,21 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // iteration n: loads K(n+2) -> K stage n%2, V(n+1) -> V stage (n+1)%2;
   //              phase 1 multiplies K(n+1) (K stage (n+1)%2), phase 2 multiplies V(n) (V stage n%2).
   int n = 0;
+  // first AE_AHEAD fragments of iteration n's stream: K(j1) if it has a next tile, else V(j0)
+  auto prefetch_ring = [&]() {
+    if (j1 < j_end) {
+      const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
+#pragma unroll
+      for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f, kt);
+    } else {
+      const ae_lds_byte* vt = lds + 2 * AE_K_BYTES + (n & 1) * AE_V_BYTES;
+#pragma unroll
+      for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_vfrag(f, vt);
+    }
+  };
+#if AE_TOP_PREFETCH
+  if (any_tile) prefetch_ring();
+#endif
   auto iteration = [&](auto has_next_tag) {
     constexpr bool HN = decltype(has_next_tag)::value;
     const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
@@ -480,24 +549,23 @@ void ae_prefill_kernel(const ae_attn_params p) {
     auto read_frag = [&](int f) -> ae_elem8 {
       return f < NF1 ? read_kfrag(f, kt) : read_vfrag(f - NF1, vt);
     };
+#if !AE_TOP_PREFETCH
 #pragma unroll
     for (int f = 0; f < AE_AHEAD && f < NF; f++) ring[f % AE_RING] = read_frag(f);
+#endif
+    // (with AE_TOP_PREFETCH the first AE_AHEAD fragments are already on their way: prefetch_ring at the
+    // end of the previous iteration, or of the prologue)
     rsum[0] = rsum[1] = 0.f;
     AE_SB();
 
-    // ---- phase 1: S(j1)^T = K Q^T  ||  p(j0) --------------------------------------------------
+    // ---- phase 1: x(j1)^T = K Q^T - m2  ||  p(j0) ------------------------------------------------
     if (HN) {
 #pragma unroll
       for (int f = 0; f < AE_NKF; f++) {
         if (f + AE_AHEAD < NF) ring[(f + AE_AHEAD) % AE_RING] = read_frag(f + AE_AHEAD);
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
-          ae_f32x16 c = sacc[f & 1][qb];
-          if (f < 2) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) c[r] = 0.f;
-          }
-          sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], c);
+          sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], f < 2 ? negc[qb] : sacc[f & 1][qb]);
           exp_slot(2 * f + qb);
           if (2 * f + qb == AE_KLOAD_SLOT) load_k(j2l, n & 1);
           if (2 * f + qb == AE_VLOAD_SLOT) load_v(j1, (n + 1) & 1);
@@ -509,14 +577,15 @@ void ae_prefill_kernel(const ae_attn_params p) {
     }
     if (HN) mx[0] = mx[1] = AE_NEG_INF;
     AE_SB();
-    // ---- phase 2: O^T += V(j0)^T P^T  ||  read S(j1) -----------------------------------------------
+    // ---- phase 2: O^T += V(j0)^T P^T  ||  maxima of x(j1) -------------------------------------------
 #pragma unroll
     for (int f = 0; f < AE_NVF; f++) {
       const int fs = NF1 + f;
       if (fs + AE_AHEAD < NF) ring[(fs + AE_AHEAD) % AE_RING] = read_frag(fs + AE_AHEAD);
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
-        oacc[qb][f % AE_NDB] = ae_mfma32(ring[fs % AE_RING], pf[qb][f / AE_NDB], oacc[qb][f % AE_NDB]);
+        oacc[qb][f % AE_NDB] = ae_mfma32(ring[fs % AE_RING], __builtin_bit_cast(ae_elem8, pf[qb][f / AE_NDB]),
+                                         oacc[qb][f % AE_NDB]);
         if (HN) {
           exp_slot(2 * AE_NKF + 2 * f + qb);
           read_scores(qb, f * AE_VPS2, AE_VPS2);
@@ -524,21 +593,30 @@ void ae_prefill_kernel(const ae_attn_params p) {
         AE_SB();
       }
     }
-    // running sums (with the factor that belongs to tile j0), then the next tile's maxima and factors
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) r_run[qb] = r_run[qb] * osc[qb] + rsum[qb];
+    for (int qb = 0; qb < 2; qb++) r_run[qb] += rsum[qb];
+#if !AE_TOP_PREFETCH
     if (HN) finish_scores(j1);
+#endif
     // tiles for the next iteration must have landed, and everyone must be done with this one's
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);   // vmcnt(0)
     __syncthreads();
     j0 = j1;
     j1 = j2;
     n++;
+#if AE_TOP_PREFETCH
+    if (HN) {
+      // the next iteration's first fragments go out now, and the new tile's maxima are compared with the
+      // reference while they travel (an iteration that started with the reads would wait for them)
+      prefetch_ring();
+      finish_scores(j0);
+    }
+#endif
   };
 
-  // The rescale of O (rare once the running maximum has settled) stays OUTSIDE the hot loop: inside
-  // it, O would have to be reachable by VALU instructions on every iteration and the register
-  // allocator then shuttles all 128 accumulator registers between the two register files per tile.
+  // The rescale of O (rare once the reference has settled) stays OUTSIDE the hot loop: inside it, O
+  // would have to be reachable by VALU instructions on every iteration and the register allocator
+  // then shuttles all 128 accumulator registers between the two register files per tile.
   auto rescale_o = [&]() {
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
@@ -571,7 +649,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
     frs[0] = 0.f;
     if (any_tile) {
-      st[qb].AE_SM_M = m_run[qb];
+      st[qb].AE_SM_M = m2[qb] * AE_LN2;
       st[qb].AE_SM_R = ae_group_sum(r_run[qb]);
       ae_epilogue<AE_NO>(o, st[qb], frs, ctx[qb], cust[qb]);
       // a row that saw tiles but no visible key: out = 0 (as for a q tile without any tile), not 0/0

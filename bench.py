@@ -24,7 +24,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (ROOT, os.path.join(ROOT, "attentionengine_amd"), os.path.join(ROOT, "tests")):
+for _p in (ROOT, os.path.join(ROOT, "attentionengine_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
@@ -43,20 +43,18 @@ WORKLOADS = {
 }
 
 
-# HBM bytes per launch of each workload's dominant kernel, measured once with the hardware counters
-# FETCH_SIZE and WRITE_SIZE (rocprofv3 --pmc, one counter per run, `--copy-probe` in the same run so
-# that a 256 MiB copy kernel calibrates the counter: FETCH_SIZE reads half the bytes moved, factor
-# 2.0; WRITE_SIZE factor 1.0).  Fetched + written.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    "c2_causal": 422.8e6 + 68.2e6,       # algorithmic Q+K+V+O+lse: 269.5e6 (K/V are fetched twice: the
-                                         # heaviest-first causal order spreads a head's q tiles in time)
-    "c2_full": 201.7e6 + 84.7e6,         # Q+K+V read once: 201.3e6; O + lse written
-    "c3_sigmoid": 201.4e6 + 68.9e6,      # Q+K+V read once; O written (no row scales)
-    "c4_gqa_decode": 2147.9e6 + 4.2e6,   # algorithmic K+V: 2147.5e6 (fp32 partials written: 4.2e6)
-    "c5_mla_decode": 623.1e6 + 16.8e6,   # algorithmic KV: 604.0e6 (+ q 18.9e6 read, out 16.8e6 written)
-    "c2_causal_bwd": 748.0e6 + 134.9e6,      # the dk/dv launch (the longest of the three): q, k, v, dout read
-                                         # about three times over (algorithmic 268e6), dk + dv written once
-}
+# HBM bytes per launch of each workload's dominant kernel, from the hardware counters FETCH_SIZE and
+# WRITE_SIZE (rocprofv3 --pmc, one counter per run, `--copy-probe` in the same run so that a 256 MiB copy
+# kernel calibrates the counter).  The figures live next to the profile summaries they were computed from,
+# in profiles/traffic.json: {workload: {"kernel": ..., "fetch_bytes": ..., "write_bytes": ...}}; a workload
+# without an entry reports null.
+def measured_traffic(name):
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            e = json.load(f)[name]
+        return float(e["fetch_bytes"]) + float(e["write_bytes"])
+    except (OSError, KeyError, ValueError, TypeError):
+        return None
 
 
 def _inputs(name, device):
@@ -118,40 +116,112 @@ def measure(name, steps, warmup):
     # The shader clock of an idle MI355X takes some tens of milliseconds of load to reach its working
     # point (measured: 0.335 ms per step after 10 warm-up steps, 0.29 ms after 50 or more), and the
     # reference's own harness warms up for 25 ms before it times anything (bench_utils.py:14-99).
+    checked = verify(name, kind, mod, args)       # untimed: one slice against eager fp32 torch
+    # MLA decode streams 0.6 GB, about twice the 256 MB of last-level cache: two copies of the KV cache
+    # alternate between steps so that no step finds a part of its input cached by the previous one
+    rotation = [args]
+    if kind == "mla_decode":
+        rotation.append([args[0], args[1], args[2].clone(), args[3].clone()])
     n_warm = 0
     t_w = time.perf_counter()
     while n_warm < max(1, warmup) or (time.perf_counter() - t_w) * 1e3 < CLOCK_RAMP_MS:
-        for _ in range(8):
-            mod(*args)
+        for i in range(8):
+            mod(*rotation[i % len(rotation)])
         n_warm += 8
         torch.cuda.synchronize()
     stream = torch.cuda.current_stream(dev).cuda_stream
     e0, e1 = rt.Event(), rt.Event()
     t0 = time.perf_counter()
     e0.record(stream)
-    for _ in range(steps):
-        mod(*args)
+    for i in range(steps):
+        mod(*rotation[i % len(rotation)])
     e1.record(stream)
     ev_ms = e0.elapsed_ms(e1) / steps          # synchronises on e1
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     res = {"workload": name, "kind": kind, "ms_per_step": wall_ms, "kernel_ms": ev_ms, "warmup_launches": n_warm,
-           **info}
+           "checked": checked, **info}
     res["tflops"] = info["flops"] / (wall_ms * 1e-3) / 1e12
     res["gbs"] = info["bytes"] / (wall_ms * 1e-3) / 1e9
     if kind in ("prefill", "prefill_bwd"):
         ach = info["flops"] / (ev_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                           "frac": ach / PEAK_MFMA_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+                           "frac": ach / PEAK_MFMA_TFLOPS, "traffic": measured_traffic(name)}
     else:
         ach = info["bytes"] / (ev_ms * 1e-3) / 1e9
         res["roofline"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                           "frac": ach / PEAK_HBM_GBS, "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+                           "frac": ach / PEAK_HBM_GBS, "traffic": measured_traffic(name)}
         if kind == "mla_decode":
             res["mfma_frac"] = info["flops"] / (ev_ms * 1e-3) / 1e12 / PEAK_MFMA_TFLOPS
-    del args, mod
+    del args, mod, rotation
     torch.cuda.empty_cache()
     return res
+
+
+def verify(name, kind, mod, args):
+    """One untimed call of the workload, compared on a slice with eager fp32 torch evaluated on the GPU
+    (closed forms of bench_utils.py:1250-1275 and mla_decode_tl.py:266-306 of the reference).  Bars as in
+    the tests: out 2e-2 max-abs, lse 1e-3; gradients 2e-2 + 1 % of their largest magnitude."""
+    import torch
+    rep = {"against": "eager fp32 torch, one slice", "ok": False}
+    with torch.no_grad():
+        if kind == "prefill":
+            q, k, v = args[:3]
+            b, h = q.shape[0] - 1, q.shape[2] - 1
+            out = mod(*args)
+            D = q.shape[3]
+            s = (q[b, :, h].float() @ k[b, :, h].float().T) / math.sqrt(D)
+            if name == "c3_sigmoid":
+                ref = torch.sigmoid(s + args[3].float()) @ v[b, :, h].float()
+                rep["slice"] = f"b{b} h{h}"
+                rep["max_abs_out"] = (out[b, :, h].float() - ref).abs().max().item()
+                rep["ok"] = rep["max_abs_out"] <= 2e-2
+                return rep
+            if name == "c2_causal":
+                s = s.masked_fill(~torch.ones_like(s, dtype=torch.bool).tril(), float("-inf"))
+            ref = torch.softmax(s, -1) @ v[b, :, h].float()
+            lse = mod.final_rowscales["lse"][b, h]
+            rep["slice"] = f"b{b} h{h}"
+            rep["max_abs_out"] = (out[b, :, h].float() - ref).abs().max().item()
+            rep["max_abs_lse"] = (lse - torch.logsumexp(s, -1)).abs().max().item()
+        elif kind == "gqa_decode":
+            q, k, v = args
+            b = q.shape[0] - 1
+            out = mod(*args)
+            g = q.shape[2] // k.shape[2]
+            kk, vv = k[b].float().repeat_interleave(g, 1), v[b].float().repeat_interleave(g, 1)   # [Skv, Hq, D]
+            s = torch.einsum("hd,khd->hk", q[b, 0].float(), kk) / math.sqrt(q.shape[3])
+            ref = torch.einsum("hk,khd->hd", torch.softmax(s, -1), vv)
+            rep["slice"] = f"batch entry {b}"
+            rep["max_abs_out"] = (out[b, 0].float() - ref).abs().max().item()
+            rep["max_abs_lse"] = (mod.final_rowscales["lse"][b, :, 0] - torch.logsumexp(s, -1)).abs().max().item()
+        elif kind == "mla_decode":
+            q, q_pe, kv, k_pe = args
+            b = q.shape[0] - 1
+            out = mod(*args)
+            s = (q[b, 0].float() @ kv[b, :, 0].float().T + q_pe[b, 0].float() @ k_pe[b, :, 0].float().T) / math.sqrt(192)
+            ref = torch.softmax(s, -1) @ kv[b, :, 0].float()
+            rep["slice"] = f"batch entry {b}"
+            rep["max_abs_out"] = (out[b, 0].float() - ref).abs().max().item()
+            rep["max_abs_lse"] = (mod.final_rowscales["lse"][b, :, 0] - torch.logsumexp(s, -1)).abs().max().item()
+        if kind != "prefill_bwd":
+            rep["ok"] = rep["max_abs_out"] <= 2e-2 and rep["max_abs_lse"] <= 1e-3
+            return rep
+    # backward: (q, k, v, out, lse, dout) -> dq, dk, dv; autograd through the eager closed form on one slice
+    q, k, v, out, lse, dout = args
+    b, h = q.shape[0] - 1, q.shape[2] - 1
+    dq, dk, dv = mod(*args)
+    qs, ks, vs = (t[b, :, h].float().detach().requires_grad_(True) for t in (q, k, v))
+    s = (qs @ ks.T) / math.sqrt(q.shape[3])
+    s = s.masked_fill(~torch.ones_like(s, dtype=torch.bool).tril(), float("-inf"))
+    (torch.softmax(s, -1) @ vs).backward(dout[b, :, h].float())
+    rep["slice"] = f"b{b} h{h}"
+    rep["ok"] = True
+    for nm, got, want in (("dq", dq, qs.grad), ("dk", dk, ks.grad), ("dv", dv, vs.grad)):
+        err = (got[b, :, h].float() - want).abs().max().item()
+        rep[f"max_abs_{nm}"] = err
+        rep["ok"] = rep["ok"] and err <= 2e-2 + 1e-2 * want.abs().max().item()
+    return rep
 
 
 COPY_PROBE_BYTES = 256 << 20
@@ -281,6 +351,7 @@ def main():
         "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
         "config": {"workload": a.workload, **head["shape"]},
         "roofline": head["roofline"],
+        "checked": head["checked"],
         "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
                    "clock_khz": info["clock_khz"]},
     }
@@ -296,6 +367,7 @@ def main():
             r = measure(name, max(5, a.steps // 2), max(2, a.warmup // 2))
             others[name] = {"ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
                             "tflops": r["tflops"], "gbs": r["gbs"], "roofline": r["roofline"],
+                            "checked": r["checked"],
                             **({"mfma_frac": r["mfma_frac"]} if "mfma_frac" in r else {})}
         line["other_configs"] = others
     print(json.dumps(line), flush=True)

@@ -55,3 +55,79 @@ def test_do_bench_attention_runs_a_mha_script(capsys):
     out = capsys.readouterr().out
     assert "Max diff" in out and "hip:" in out
     assert lat > 0 and lat_ref > 0 and tf > 0
+
+
+def _meta3(B, H, S, D, DV, dtype):
+    from core import meta_tensor
+    return (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, H, S, D, dtype=dtype),
+            meta_tensor(B, H, S, DV, dtype=dtype))
+
+
+def _diff_lines(out):
+    """(not-close counts, max diffs) of every print_debug block in the captured text."""
+    import re
+    bad = [int(m) for m in re.findall(r"Total elements: \d+, Not close elements: (\d+)", out)]
+    mx = [float(m) for m in re.findall(r"Max diff: ([0-9.eE+-]+) at index", out)]
+    return bad, mx
+
+
+@pytest.mark.gpu
+def test_do_bench_sigmoidattn_runs_the_script_form(capsys):
+    """attn_script/sigmoidattn.py through its harness (bench_utils.py:701-788 of the reference): causal
+    sigmoid attention with the bias as 4th argument, forward and backward compared with eager torch."""
+    import attn_cases as C
+    from attn_engine import AttentionEngine
+    from core import CustomIO
+    B, H, S, D = 1, 4, 256, 64
+    mod = AttentionEngine(_meta3(B, H, S, D, D, torch.float16), CustomIO({"softmax_bias": (1,)}),
+                          score_mod=C.make_sigmoid_score_mod(), mask_mod=C.causal_mask,
+                          online_func=C.OnlineIdentity())
+    lat, tf, lat_ref, tf_ref = bench_utils.do_bench_sigmoidattn(mod, B, H, S, D, D, dtype=torch.float16,
+                                                                requires_grad=True)
+    out = capsys.readouterr().out
+    bad, mx = _diff_lines(out)
+    assert len(bad) == 4 and len(mx) == 4            # dq, dk, dv, then the forward output
+    assert max(bad) == 0, out                       # every element within 1e-2 + 1 % (outputs reach ~50 here)
+    assert "hip:" in out and "hip bwd:" in out and "eager torch:" in out
+    assert lat > 0 and lat_ref > 0 and tf > 0 and tf_ref > 0
+
+
+@pytest.mark.gpu
+def test_do_bench_reluattn_runs_the_script_form(capsys):
+    """attn_script/reluattn.py through its harness (bench_utils.py:949-1022 of the reference), with
+    requires_grad=True as the script passes it."""
+    import attn_cases as C
+    from attn_engine import AttentionEngine
+    from core import CustomIO
+    B, H, S, D = 2, 3, 256, 64
+    mod = AttentionEngine(_meta3(B, H, S, D, D, torch.float16), CustomIO({}),
+                          score_mod=C.make_relu_score_mod(1 / D ** 0.5), mask_mod=None,
+                          online_func=C.OnlineIdentity())
+    lat, tf, lat_ref, tf_ref = bench_utils.do_bench_reluattn(mod, B, H, S, D, D, dtype=torch.float16,
+                                                             requires_grad=True)
+    out = capsys.readouterr().out
+    bad, mx = _diff_lines(out)
+    assert len(bad) == 4 and len(mx) == 4
+    # relu attention sums ~S/2 positive terms of size ~0.4: fp16 results of size ~10, compared at 1e-2 + 1%
+    assert max(bad) <= 4, out
+    assert "hip:" in out and "hip bwd:" in out and "eager torch:" in out
+    assert lat > 0 and lat_ref > 0 and tf > 0 and tf_ref > 0
+
+
+@pytest.mark.gpu
+def test_do_bench_retention_runs_the_script_form(capsys):
+    """attn_script/retention.py through its harness (bench_utils.py:1025-1100 of the reference): the decay
+    mask as 4th argument, value head dim twice the key head dim."""
+    import attn_cases as C
+    from attn_engine import AttentionEngine
+    B, H, S, D, DV = 1, 2, 256, 64, 128
+    dtype = torch.bfloat16
+    mod = AttentionEngine(_meta3(B, H, S, D, DV, dtype), C.retention_custom_inputs(),
+                          score_mod=C.retention_score_mod, mask_mod=C.causal_mask,
+                          online_func=C.OnlineAbsNorm(), mask_value="0")
+    lat, tf, lat_ref, tf_ref = bench_utils.do_bench_retention(mod, B, H, S, D, DV, dtype=dtype)
+    out = capsys.readouterr().out
+    bad, mx = _diff_lines(out)
+    assert len(bad) == 1 and bad[0] == 0, out
+    assert "hip:" in out and "eager torch:" in out
+    assert lat > 0 and lat_ref > 0 and tf > 0 and tf_ref > 0

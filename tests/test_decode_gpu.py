@@ -117,6 +117,68 @@ def test_mla_decode_tl_convention(cuda_device, monkeypatch, B, H, G, S, dtype, k
     assert (mod.final_rowscales["lse"][:, :, 0].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
+@pytest.mark.parametrize("kernel,template", [("", "ae_mla_decode_ws.hip"), ("generic", "ae_mla_decode.hip")])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("S,late_keys", [(1024, False), (1000, False), (1531, True)])
+def test_mla_decode_long_single_split_loop(cuda_device, monkeypatch, kernel, template, dtype, S, late_keys):
+    """The plan the benchmark runs at B128 H128 S4096 is ONE split per workgroup and a loop over many kv
+    tiles that writes out / lse directly, without the merge pass.  Forced here on a small shape
+    (target_workgroups = 1): 32 to 48 tiles per workgroup with a ragged last tile, so the LDS stage ring
+    wraps many times, the hand-off between score and value waves runs a long loop, and -- with keys that
+    score far above everything before them late in the sequence -- the lazy reference moves and O is
+    rescaled in the middle of it."""
+    D, DV, B, H, G = 576, 512, 2, 128, 1
+    scale = 1 / math.sqrt(192)
+    print(f"case mla long loop S{S} {dtype} kernel={kernel or 'default'} late_keys={late_keys}", flush=True)
+    monkeypatch.setenv("AE_MLA_KERNEL", kernel)
+    q, q_pe, kv, k_pe = _mla_inputs(B, H, G, S, DV, D - DV, dtype, seed=17)
+    if late_keys:
+        # (only the rope part of the keys is scaled: the latent part is also V, and outputs beyond ~4 do
+        # not fit bf16's 8 bits inside the 2e-2 bar)
+        k_pe = k_pe.float()
+        k_pe[:, 700:703] *= 12.0          # a jump for every head ...
+        k_pe[:, 1200:] *= 4.0             # ... and a second level that stays
+        k_pe = k_pe.to(dtype)
+    mod = _mla_engine(B, H, G, S, D, DV, dtype, scale)
+    mod.attention.target_workgroups = 1       # read by plan_splits at call time
+    n_split, per = mod.attention.plan_splits(B, H, G, S)
+    assert n_split == 1 and per >= S and per // mod.attention.BLOCK_N >= 2 * mod.attention.WS_STAGES
+    out = mod(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda())
+    assert mod.attention.template == template
+    ref, lse = R.mla_decode(q[:, 0], q_pe[:, 0], kv, k_pe, scale=scale)
+    assert torch.isfinite(out).all()
+    assert (out[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL
+    got = mod.final_rowscales["lse"][:, :, 0].cpu()
+    assert ((got - lse).abs() <= LSE_TOL + 2e-6 * lse.abs()).all()
+
+
+def test_mla_decode_full_size(cuda_device):
+    """BASELINE config 5 at full size (B128 H128 one latent head, D576 DV512, Skv4096, bf16, scale
+    1/sqrt(192)) with the plan the benchmark times: one split, 128 tiles per workgroup.  Oracle on batch
+    entries 0, 127 and two seeded others; everything finite; lse independent of which batch slot a
+    sequence sits in (entry 5 is a copy of entry 77)."""
+    D, DV, B, H, G, S = 576, 512, 128, 128, 1, 4096
+    dtype = torch.bfloat16
+    scale = 1 / math.sqrt(192)
+    q, q_pe, kv, k_pe = _mla_inputs(B, H, G, S, DV, D - DV, dtype, seed=5)
+    for t in (q, q_pe, kv, k_pe):
+        t[5] = t[77]
+    mod = _mla_engine(B, H, G, S, D, DV, dtype, scale)
+    n_split, per = mod.attention.plan_splits(B, H, G, S)
+    assert (n_split, per) == (1, S)                 # what bench.py's c5_mla_decode launches
+    out = mod(q.cuda(), q_pe.cuda(), kv.cuda(), k_pe.cuda())
+    lse = mod.final_rowscales["lse"][:, :, 0]
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert torch.equal(out[5], out[77]) and torch.equal(lse[5], lse[77])
+    import random
+    picks = [0, 127] + random.Random(8).sample(range(1, 127), 2)
+    for b in picks:
+        print(f"case mla full size: oracle on batch entry {b}", flush=True)
+        ref, lref = R.mla_decode(q[b:b + 1, 0], q_pe[b:b + 1, 0], kv[b:b + 1], k_pe[b:b + 1], scale=scale)
+        assert (out[b:b + 1, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL, b
+        assert (lse[b:b + 1].cpu() - lref).abs().max().item() <= LSE_TOL, b
+
+
 def test_mla_decode_cute_convention(cuda_device):
     """mod(q [B,1,H,576], paged kv cache [B*S/64, 64, 1, 576]) -> (out, lse), as in
     attn_script/mla_decode_cute.py:286-303; lse checked with the script's cos-diff bound (107-113)."""

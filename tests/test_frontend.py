@@ -276,6 +276,55 @@ def test_lazy_maximum_only_for_the_online_softmax():
     assert "5.545" not in lf.online_fwd_body
 
 
+def test_softmax_specialisation_needs_the_exact_graph():
+    """Kernels that hard-code exp(c*S - m) (pipelined prefill, wave-specialised MLA decode, the softmax
+    backward) may only be chosen for the online softmax OF the modified scores.  Near misses -- another
+    function of the scores inside exp, another quantity inside the running maximum, other initial
+    values -- stay reference-point invariant (lazy maximum allowed) but must run the generated functor."""
+    from attn_engine import OnlineFunc
+    sm = C.make_scale_score_mod(0.125)
+    assert L.trace_functors(sm, None, C.OnlineSoftmax(), CustomIO({}), torch.float16).softmax == (0.125, "m", "r")
+
+    class TwiceInsideExp(C.OnlineSoftmax):
+        @staticmethod
+        def online_fwd(scores, online_rowscales, b, h, q_idx):
+            m, r = online_rowscales["m"], online_rowscales["r"]
+            m_new = m.max(scores.get_reduce("max"))
+            scale_tmp = (m - m_new).exp()
+            p = (scores * 2.0 - m_new).exp()
+            return p, {"m": m_new, "r": r * scale_tmp + p.get_reduce("sum")}, scale_tmp
+
+    class AbsInsideMax(C.OnlineSoftmax):
+        @staticmethod
+        def online_fwd(scores, online_rowscales, b, h, q_idx):
+            m, r = online_rowscales["m"], online_rowscales["r"]
+            m_new = m.max(scores.abs().get_reduce("max"))
+            scale_tmp = (m - m_new).exp()
+            p = (scores - m_new).exp()
+            return p, {"m": m_new, "r": r * scale_tmp + p.get_reduce("sum")}, scale_tmp
+
+    class StartsAtZero(C.OnlineSoftmax):
+        def __init__(self):
+            OnlineFunc.__init__(self, {"m": SymbolScalar("m", Var("0.0")), "r": SymbolScalar("r", Var("0.0"))},
+                                {"lse": SymbolScalar("lse", Var("0.0"))}, CustomIO())
+
+    for near_miss in (TwiceInsideExp(), AbsInsideMax(), StartsAtZero()):
+        lf = L.trace_functors(sm, None, near_miss, CustomIO({}), torch.float16)
+        assert lf.softmax is None, type(near_miss).__name__
+        # ... and the generic kernel is what the engine then compiles, even on chip-filling shapes
+        tiles = L.choose_prefill_tiles(128, 128, seqlen_q=4096, softmax=lf.softmax, batch_heads=64)
+        assert tiles.template == "ae_prefill.hip"
+    src = L.render_functors(L.trace_functors(sm, None, TwiceInsideExp(), CustomIO({}), torch.float16))
+    assert "0.3606737" in src                    # the functor carries the user's factor: 0.125 * 2 * log2(e)
+    # no backward is derived for them either: the softmax gradient is only valid for the exact graph
+    from core.lower.prefill_bwd_op import PrefillBwdOp
+    from core.lower.prefill_op import PrefillOp
+    for near_miss in (TwiceInsideExp(), AbsInsideMax()):
+        op = PrefillOp(_meta(1, 2, 2, 256, 256, 64, 64, torch.float16), CustomIO({}), sm, None, near_miss, "-inf")
+        with pytest.raises(NotImplementedError):
+            PrefillBwdOp(op, sm, near_miss, CustomIO({}))
+
+
 def test_shapes_broadcast_by_name():
     q = SymbolScalar("q_idx", Var("q_idx"), shape_idx=["block_M"])
     kv = SymbolScalar("kv_idx", Var("kv_idx"), shape_idx=["block_N"])

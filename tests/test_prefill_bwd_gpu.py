@@ -66,6 +66,29 @@ def test_softmax_backward(cuda_device, B, H, Hkv, S, D, dtype, causal):
     _run(B, H, Hkv, S, S, D, D, dtype, C.causal_mask if causal else None, causal)
 
 
+def test_softmax_backward_headline_shape(cuda_device):
+    """The shape bench.py times the backward on (B2 H32 S4096 D128 fp16, causal): every gradient finite,
+    and dq, dk, dv of two (batch, head) slices -- which depend on that slice's tensors only -- against the
+    oracle's closed-form gradients."""
+    B, H, S, D = 2, 32, 4096, 128
+    dtype = torch.float16
+    scale = 1 / math.sqrt(D)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=9)
+    do = torch.randn(B, S, H, D, generator=torch.Generator().manual_seed(109)).to(dtype)
+    mod = _engine(B, H, H, S, D, D, dtype, C.causal_mask, scale)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    mod(qd, kd, vd).backward(do.cuda())
+    for g in (qd.grad, kd.grad, vd.grad):
+        assert torch.isfinite(g).all()
+    for b, h in ((0, 0), (1, 31)):
+        print(f"case backward at the headline shape: oracle on slice b{b} h{h}", flush=True)
+        sl = (slice(b, b + 1), slice(None), slice(h, h + 1))
+        dq, dk, dv = R.softmax_attention_grads(q[sl], k[sl], v[sl], do[sl], scale=scale, causal=True)
+        _check(qd.grad[sl], dq, "dq", (b, h))
+        _check(kd.grad[sl], dk, "dk", (b, h))
+        _check(vd.grad[sl], dv, "dv", (b, h))
+
+
 def test_softmax_backward_elementwise_mask_and_dv(cuda_device):
     """A mask that is not causal is applied per element (sliding window: rows see 37 keys), and the
     value head dim may differ from the key head dim."""
