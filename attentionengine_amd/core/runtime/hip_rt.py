@@ -119,6 +119,8 @@ _SIGNATURES = {
     "ae_prefill_fwd": (C.c_int, [_VP, C.POINTER(AttnParams), C.POINTER(TileCfg), _VP]),
     "ae_decode_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
                                 C.POINTER(TileCfg), _VP]),
+    "ae_decode_fwd_noalloc": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
+                                        C.POINTER(TileCfg), _VP]),
     "ae_mla_decode_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
                                     C.POINTER(TileCfg), _VP]),
     "ae_prefill_split_fwd": (C.c_int, [_VP, _VP, C.POINTER(AttnParams), C.POINTER(TileCfg),
@@ -328,6 +330,17 @@ def decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
     _check(lib().ae_decode_fwd(split.handle, combine.handle if combine else None, C.byref(params),
                                C.byref(cfg), C.byref(combine_cfg) if combine_cfg else None,
                                _VP(stream)))
+
+
+def decode_fwd_noalloc(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,
+                       combine_cfg: TileCfg, stream: int = 0):
+    """ae_decode_fwd on the library's built-in split-KV work buffer (params.partial_* are ignored)."""
+    _check(lib().ae_decode_fwd_noalloc(split.handle, combine.handle if combine else None, C.byref(params),
+                                       C.byref(cfg), C.byref(combine_cfg) if combine_cfg else None,
+                                       _VP(stream)))
+
+
+NOALLOC_SCRATCH_BYTES = 16 << 20      # AE_NOALLOC_SCRATCH_BYTES of include/ae_hip.h
 
 
 def prefill_split_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: TileCfg,

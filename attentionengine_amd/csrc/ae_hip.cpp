@@ -1,7 +1,8 @@
 // libae_hip.so: hipRTC compile + code-object cache + checked launches behind a C ABI.
 // Declarations and the reference interfaces they stand in for: include/ae_hip.h.
 //
-// Host-only translation unit (built with g++ or hipcc); links libamdhip64 + libhiprtc.
+// Host-only translation unit (built with g++ or hipcc); links libamdhip64 + libhiprtc.  The library's
+// second translation unit, ae_noalloc.hip, carries its one piece of device data.
 
 #include "ae_hip.h"
 
@@ -45,6 +46,17 @@ int fail_str(int code, const std::string& s) {
   } while (0)
 
 }  // namespace
+
+// the same for the library's other translation unit (ae_noalloc.hip); not part of the ABI
+extern "C" __attribute__((visibility("hidden"))) int ae_internal_fail(int code, const char* fmt, ...) {
+  char buf[4096];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
 
 struct ae_kernel {
   hipFunction_t fn = nullptr;

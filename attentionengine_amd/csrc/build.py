@@ -1,6 +1,6 @@
 """Build steps for the native side of the package.
 
-  build_library()       g++ -> csrc/libae_hip.so (the C ABI of include/ae_hip.h)
+  build_library()       g++ + hipcc -> csrc/libae_hip.so (the C ABI of include/ae_hip.h)
   check_templates()     hipcc --offload-arch=gfx950 -c of every kernel template, with headers
                         generated for a representative configuration (offline "does it build")
 
@@ -35,11 +35,19 @@ def _run(cmd):
 
 
 def build_library(verbose=False):
-    """Compile csrc/ae_hip.cpp into csrc/libae_hip.so (host code only)."""
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-D__HIP_PLATFORM_AMD__",
-           f"-I{INCLUDE}", f"-I{ROCM}/include", osp.join(CSRC, "ae_hip.cpp"),
-           f"-L{ROCM}/lib", "-lamdhip64", "-lhiprtc", f"-Wl,-rpath,{ROCM}/lib", "-o", LIB + ".tmp"]
-    out = _run(cmd)
+    """csrc/ae_hip.cpp (host code, g++) + csrc/ae_noalloc.hip (the one unit with device data, hipcc for
+    gfx950) -> csrc/libae_hip.so, linked by hipcc so that the device image is registered at load time."""
+    hipcc = osp.join(ROCM, "bin", "hipcc")
+    out = ""
+    with tempfile.TemporaryDirectory() as d:
+        host_o, dev_o = osp.join(d, "ae_hip.o"), osp.join(d, "ae_noalloc.o")
+        out += _run(["g++", "-O2", "-std=c++17", "-fPIC", "-c", "-Wall", "-D__HIP_PLATFORM_AMD__",
+                     f"-I{INCLUDE}", f"-I{ROCM}/include", osp.join(CSRC, "ae_hip.cpp"), "-o", host_o])
+        out += _run([hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-c",
+                     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                     f"-I{INCLUDE}", osp.join(CSRC, "ae_noalloc.hip"), "-o", dev_o])
+        out += _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", host_o, dev_o,
+                     f"-L{ROCM}/lib", "-lamdhip64", "-lhiprtc", f"-Wl,-rpath,{ROCM}/lib", "-o", LIB + ".tmp"])
     os.replace(LIB + ".tmp", LIB)
     if verbose and out.strip():
         print(out)

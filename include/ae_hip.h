@@ -49,7 +49,7 @@ using __hip_internal::uint64_t;
 extern "C" {
 #endif
 
-#define AE_ABI_VERSION 2
+#define AE_ABI_VERSION 3
 
 typedef enum ae_status {
   AE_OK = 0,
@@ -258,6 +258,25 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
  */
 int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
                    const ae_tile_cfg* cfg, void* stream);
+
+/*
+ * ae_decode_fwd_noalloc: ae_decode_fwd for callers that cannot allocate.  It has no counterpart in the
+ *   reference (whose generated _attention.forward allocates its split-KV buffers with torch.empty on every
+ *   call, attn_gqa_decode_tl.py:345-348); it is for code under HIP graph capture, tight serving loops and
+ *   harnesses that forbid hipMalloc.  Same arguments and checks as ae_decode_fwd, but p->partial_o and
+ *   p->partial_rs are ignored: the split-KV partials go to a work buffer of AE_NOALLOC_SCRATCH_BYTES that
+ *   is part of the library's device image (one copy per GPU, held until the process ends).  The entry
+ *   point calls no hipMalloc / hipFree or any allocating routine; its first call on a device looks up the
+ *   buffer's address once (make that call outside a graph capture).  A launch whose partials
+ *   (B*Hq*num_splits*(DV + max(1,n_rowscales)) fp32 values, the first part rounded up to 256 bytes) do not
+ *   fit returns AE_ERR_INVALID_ARG and launches nothing.  All calls on one GPU share that GPU's buffer:
+ *   calls that may overlap in time on one GPU (different streams, different threads) race -- serialise
+ *   them, or use ae_decode_fwd with separate buffers.  Nothing in the buffer has to be cleared between
+ *   calls (every partial that is read has been written by the same call).
+ */
+#define AE_NOALLOC_SCRATCH_BYTES (16u << 20)
+int ae_decode_fwd_noalloc(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                          const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
 
 /* ---- timing on the launch stream ------------------------------------------------- */
 int ae_event_create(ae_event** out);

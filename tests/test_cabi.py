@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in ae_hip.h but not exported"
     assert sorted(rt.EXPORTED_SYMBOLS) == names
-    assert rt.lib().ae_abi_version() == 2
+    assert rt.lib().ae_abi_version() == 3
 
 
 def test_struct_layout_matches_the_header():
