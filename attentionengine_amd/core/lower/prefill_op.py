@@ -208,8 +208,17 @@ class PrefillOp:
         q, k, v = (t if t.stride(3) == 1 else t.contiguous() for t in (q, k, v))
         dev = q.device
 
+        if extern_mask is not None and extern_mask is self.block_mask and not self.extern_block_mask:
+            # the block mask this engine inferred from mask_mod itself (AttentionEngine appends it to every
+            # call, attn_engine.py:391-392 of the reference): the tile-class table planned from the same
+            # mask_mod says the same at the kernel's own tile granularity, whatever infer_mask_block_M/N are
+            extern_mask = None
         if extern_mask is not None:
             bm, bn = self.mask_block
+            if bn % self.tiles.block_n or (self.tiles.block_m % bm and bm % self.tiles.block_m):
+                raise NotImplementedError(
+                    f"a block mask of {bm}x{bn} blocks does not fit the kernel's {self.tiles.block_m}x"
+                    f"{self.tiles.block_n} tiles (construct the engine with extern_block_mask=True)")
             table = extern_mask
             if table.dim() != 4:
                 raise ValueError("block_mask must be [B|1, H|1, Sq/bm, Skv/bn]")

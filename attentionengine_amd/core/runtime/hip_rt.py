@@ -108,6 +108,7 @@ _SIGNATURES = {
     "ae_device_info": (C.c_int, [C.c_int, C.POINTER(DevInfo)]),
     "ae_compile": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int,
                              C.POINTER(C.c_char_p), C.POINTER(C.c_char_p), C.c_int, C.POINTER(_VP)]),
+    "ae_compiler_version": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "ae_module_log": (C.c_char_p, [_VP]),
     "ae_module_code": (C.c_int, [_VP, C.POINTER(_VP), C.POINTER(C.c_size_t)]),
     "ae_module_save": (C.c_int, [_VP, C.c_char_p]),
@@ -172,6 +173,20 @@ def device_info(device: int = 0) -> dict:
     out["name"] = info.name.decode()
     out["arch"] = info.arch.decode()
     return out
+
+
+_compiler_version = None
+
+
+def compiler_version() -> str:
+    """"major.minor" of the hipRTC that ae_compile uses (part of the code-object cache key: objects
+    cached by one toolchain are not reused by another)."""
+    global _compiler_version
+    if _compiler_version is None:
+        major, minor = C.c_int(), C.c_int()
+        _check(lib().ae_compiler_version(C.byref(major), C.byref(minor)))
+        _compiler_version = f"hiprtc {major.value}.{minor.value}"
+    return _compiler_version
 
 
 def cache_dir() -> str:
@@ -263,7 +278,7 @@ def compile_module(template: str, headers: dict, arch: str = None, use_cache: bo
     }
     all_headers.update(headers)
     hsh = hashlib.sha256()
-    for part in [template, src, arch, " ".join(COMPILE_OPTS)]:
+    for part in [template, src, arch, " ".join(COMPILE_OPTS), compiler_version()]:
         hsh.update(part.encode())
         hsh.update(b"\0")
     for name in sorted(all_headers):

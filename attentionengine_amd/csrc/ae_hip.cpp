@@ -9,6 +9,9 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
+#include <unistd.h>
+
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -168,6 +171,14 @@ int ae_compile(const char* src, const char* name, const char* arch,
   return AE_OK;
 }
 
+int ae_compiler_version(int* major, int* minor) {
+  if (!major || !minor) return fail(AE_ERR_INVALID_ARG, "ae_compiler_version: NULL argument");
+  hiprtcResult r = hiprtcVersion(major, minor);
+  if (r != HIPRTC_SUCCESS)
+    return fail(AE_ERR_COMPILE, "hiprtcVersion failed: %s", hiprtcGetErrorString(r));
+  return AE_OK;
+}
+
 const char* ae_module_log(const ae_module* m) { return m ? m->log.c_str() : ""; }
 
 int ae_module_code(const ae_module* m, const void** data, size_t* size) {
@@ -179,8 +190,11 @@ int ae_module_code(const ae_module* m, const void** data, size_t* size) {
 
 int ae_module_save(const ae_module* m, const char* path) {
   if (!m || !path) return fail(AE_ERR_INVALID_ARG, "ae_module_save: NULL argument");
-  // write to a temporary name first so a concurrent reader never sees a torn file
-  std::string tmp = std::string(path) + ".tmp";
+  // write to a temporary name first so a concurrent reader never sees a torn file; the name is unique
+  // per process and call, so two processes compiling the same key never write one temporary file
+  static std::atomic<unsigned> counter{0};
+  std::string tmp = std::string(path) + ".tmp." + std::to_string((long)getpid()) + "." +
+                    std::to_string(counter.fetch_add(1));
   FILE* f = fopen(tmp.c_str(), "wb");
   if (!f) return fail(AE_ERR_IO, "ae_module_save: cannot open %s", tmp.c_str());
   size_t n = fwrite(m->code.data(), 1, m->code.size(), f);
@@ -331,6 +345,11 @@ int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg
   if (cfg->mask_mode == 2 && (cfg->block_m % p->mask_block_m != 0 && p->mask_block_m % cfg->block_m != 0))
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: mask block rows %d incompatible with tile %d",
                 p->mask_block_m, cfg->block_m);
+  // a kv tile must lie inside ONE column of the table: the kernels classify a tile by the column of its
+  // first key
+  if (cfg->mask_mode == 2 && p->mask_block_n % cfg->block_n != 0)
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: block-mask columns of %d keys are not a multiple of the %d-key kv tile",
+                p->mask_block_n, cfg->block_n);
   // ids are 8*slot + xcd with slot = (batch*head / 8)*q_tiles + q_tile, see ae_prefill.hip
   uint64_t q_tiles = ((uint64_t)p->seqlen_q + cfg->block_m - 1) / cfg->block_m;
   uint64_t bh = (uint64_t)p->heads_q * (uint64_t)p->batch;

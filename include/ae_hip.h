@@ -182,6 +182,9 @@ int ae_compile(const char* src, const char* name, const char* arch,
                const char* const* opts, int nopts,
                const char* const* header_names, const char* const* headers, int nheaders,
                ae_module** out);
+/* Version of the hipRTC that ae_compile drives (callers fold it into their code-object cache keys; the
+ * reference's cache key is an md5 of the rendered source only, attn_engine.py:369-375). */
+int ae_compiler_version(int* major, int* minor);
 /* hipRTC log of the compilation that produced the module (warnings; "" if none). */
 const char* ae_module_log(const ae_module* m);
 /* Borrowed view of the code object bytes. */

@@ -37,12 +37,34 @@ def test_every_declared_symbol_is_exported_and_bound():
 
 
 def test_struct_layout_matches_the_header():
-    """sizeof(ae_attn_params) as the device compiler sees it == the ctypes mirror."""
+    """Size and every field offset of the three parameter structs, as the DEVICE compiler lays them out
+    from include/ae_hip.h, equal the ctypes mirrors: a probe whose static_asserts carry the ctypes figures
+    is compiled for gfx950 through ae_compile (needs no GPU).  A reordered or retyped field of equal size
+    in either place fails the compilation."""
     # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints
     assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16
     assert ctypes.sizeof(rt.TileCfg) == 4 * 12
     # backward: 12 + 4 pointers, 8 tensors x 3 strides, 7 + 1 ints
     assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 16 + 8 * 24 + 4 * 8
+    lines = ['#include "ae_hip.h"']
+    n_fields = 0
+    for cname, mirror in (("ae_attn_params", rt.AttnParams), ("ae_tile_cfg", rt.TileCfg),
+                          ("ae_attn_bwd_params", rt.AttnBwdParams), ("ae_devinfo", rt.DevInfo)):
+        lines.append(f'static_assert(sizeof({cname}) == {ctypes.sizeof(mirror)}, "sizeof {cname}");')
+        for fname, ftype in mirror._fields_:
+            off, size = getattr(mirror, fname).offset, ctypes.sizeof(ftype)
+            lines.append(f'static_assert(__builtin_offsetof({cname}, {fname}) == {off}, "{cname}.{fname} offset");')
+            lines.append(f'static_assert(sizeof((({cname}*)0)->{fname}) == {size}, "{cname}.{fname} size");')
+            n_fields += 1
+    lines.append('extern "C" __global__ void probe(int* p) { p[0] = 0; }')
+    assert n_fields > 80
+    rc, handle = _compile("\n".join(lines))
+    assert rc == 0, rt.lib().ae_last_error().decode()
+    rt.lib().ae_module_free(handle)
+    # ... and the probe does notice a wrong figure
+    bad = "\n".join(lines).replace("__builtin_offsetof(ae_attn_params, k2) == ", "__builtin_offsetof(ae_attn_params, k2) == 1 + ")
+    rc, _ = _compile(bad)
+    assert rc != 0 and "ae_attn_params.k2 offset" in rt.lib().ae_last_error().decode()
 
 
 def _compile(src, opts=()):

@@ -377,3 +377,17 @@ def test_elementwise_backward_lowering():
     with pytest.raises(NotImplementedError):
         lower_elementwise_backward(C.retention_score_mod, C.OnlineIdentity(), C.retention_custom_inputs(),
                                    torch.float16)
+
+
+def test_inferred_block_mask_granularity_does_not_reach_the_kernel():
+    """infer_mask_block_M/N only shape the block mask kept on mod.block_mask (lower.py:721-738 of the
+    reference); the kernel classifies its own tiles from mask_mod, so a granularity that no kv tile fits
+    (96 keys against 64-key tiles) is harmless, and handing the engine such a mask from outside is refused
+    instead of skipping visible keys."""
+    from core.lower.prefill_op import PrefillOp
+    op = PrefillOp(_meta(1, 2, 2, 384, 384, 64, 64, torch.float16), CustomIO({}), C.make_scale_score_mod(0.125),
+                   C.make_sliding_window_mask(100), C.OnlineSoftmax(), "-inf", infer_mask=True,
+                   infer_mask_block_M=128, infer_mask_block_N=96)
+    assert op.block_mask is not None and op.block_mask.shape == (1, 2, 3, 4)
+    plan = op._plan(1, 2, 384, 384, device=None)
+    assert (plan.block_m, plan.block_n) == (op.tiles.block_m, op.tiles.block_n)

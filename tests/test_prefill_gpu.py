@@ -178,6 +178,26 @@ def test_masked_softmax_prefill(cuda_device, name, mask_mod):
         assert torch.isneginf(lse[~visible]).all()
 
 
+def test_inferred_block_mask_of_odd_granularity(cuda_device):
+    """infer_mask_block_N = 96 keys against 64-key kv tiles: the inferred block mask is appended to every
+    call (as in the reference) but the kernel classifies its tiles from mask_mod itself, so no visible
+    key is lost at a tile that straddles two mask columns."""
+    B, H, S, D = 1, 2, 384, 64
+    dtype = torch.float16
+    mask_mod = C.make_sliding_window_mask(100)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=12)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod, C.OnlineSoftmax(),
+                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=96)
+    assert mod.block_mask is not None
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    ref, lse = R.softmax_attention(q, k, v, mask=_dense(mask_mod, B, H, S, S))
+    assert (out - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+    # a mask of that granularity handed in from outside cannot be honoured tile by tile: refused
+    with pytest.raises(NotImplementedError, match="does not fit"):
+        mod(q.cuda(), k.cuda(), v.cuda(), block_mask=mod.block_mask.clone().cuda())
+
+
 def test_mask_is_bit_exact(cuda_device):
     """Probe the effective device mask.  The score_mod maps every finite score to exactly 1 and a
     masked (-inf) score to exactly 0 (tanh saturates), rowscales are the identity and V holds
