@@ -47,14 +47,17 @@ class OnlineFunc:
 
     @staticmethod
     def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
-        """Recompute rule of the backward pass, p from the modified scores and the final row scales.  The
-        backward checks that it is the identity for online functions without row scales; for softmax
-        attention the gradient is fixed by the proven forward and the rule is not traced."""
+        """Recompute rule of the backward pass, p from the modified scores and the final row scales.  Traced
+        for online functions that keep a final row scale of their own and override it (retention); checked
+        to be the identity for online functions without row scales; for softmax attention the gradient is
+        fixed by the proven forward and the rule is not traced."""
         return scores
 
     @staticmethod
     def backward(dp, scores, final_rowscales, b, h, q_idx, kv_idx):
-        """Backward rule, dscores from dp (see ``forward``)."""
+        """Backward rule, dscores from dp, the recomputed p (``scores``) and the final row scales; overrides
+        may take the rowsum(do * o) row scale as a fourth argument, as attn_script/retention.py:65 does
+        (see ``forward``)."""
         return dp
 
     @staticmethod

@@ -134,6 +134,19 @@ class OnlineAbsNorm(OnlineFunc):
         return o, {"r": online_rowscales["r"]}
 
 
+class OnlineRetention(OnlineAbsNorm):
+    """attn_script/retention.py:19-70 in full: the abs-sum normalisation above plus the recompute and
+    backward rules of its backward pass (the row scale is treated as a constant there, as in the script)."""
+
+    @staticmethod
+    def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+        return scores / final_rowscales["r"]
+
+    @staticmethod
+    def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+        return dp / final_rowscales["r"]
+
+
 def retention_score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
     """attn_script/retention.py:14-16: the scores times a decay mask given as a [1,H,S,S] input."""
     return score * custom_fwd_inputs.input_tensors["mask"]

@@ -25,16 +25,20 @@ def _topo(root):
     return order
 
 
-def derivative(out: SymbolScalar, wrt: SymbolScalar) -> SymbolScalar:
-    """d out / d wrt as a traced expression (a constant 0 if ``out`` does not depend on ``wrt``)."""
+def _reverse(out: SymbolScalar, seed: SymbolScalar, wrt):
+    """Reverse sweep from ``out`` seeded with ``seed``: {id(symbol): gradient expression} for the symbols on
+    a path from ``out`` to one of ``wrt`` (to any leaf when ``wrt`` is None)."""
     order = _topo(out)
-    depends = {id(wrt)}
-    for s in order:
-        if any(id(x) in depends for x in s.prev):
-            depends.add(id(s))
+    if wrt is None:
+        depends = {id(s) for s in order}
+    else:
+        depends = {id(w) for w in wrt}
+        for s in order:
+            if any(id(x) in depends for x in s.prev):
+                depends.add(id(s))
     if id(out) not in depends:
-        return SymbolicConst(0.0)
-    grads = {id(out): SymbolicConst(1.0)}
+        return {}, order
+    grads = {id(out): seed}
 
     def add(sym, g):
         if id(sym) not in depends:
@@ -79,4 +83,21 @@ def derivative(out: SymbolScalar, wrt: SymbolScalar) -> SymbolScalar:
             add(b, g.maxbwd(b, a))
         else:
             raise NotImplementedError(f"derivative of {t}")
+    return grads, order
+
+
+def derivative(out: SymbolScalar, wrt: SymbolScalar) -> SymbolScalar:
+    """d out / d wrt as a traced expression (a constant 0 if ``out`` does not depend on ``wrt``)."""
+    grads, _ = _reverse(out, SymbolicConst(1.0), [wrt])
     return grads.get(id(wrt), SymbolicConst(0.0))
+
+
+def backward(out: SymbolScalar, grad=None) -> None:
+    """``out.backward(grad)`` of the reference (core/transform/core.py:119-199): leave on every symbol the
+    output was computed from its gradient expression in ``.grad`` (``grad`` times d out / d symbol; ``grad``
+    defaults to 1).  Symbols that ``out`` reaches on several paths get the sum."""
+    seed = SymbolicConst(1.0) if grad is None else grad
+    grads, order = _reverse(out, seed, None)
+    for sym in order:
+        if id(sym) in grads:
+            sym.grad = grads[id(sym)]

@@ -114,7 +114,10 @@ class SymbolScalar:
         return out
 
     def backward(self, grad=None):
-        raise NotImplementedError("use core.transform.autodiff.derivative(out, wrt): the derivative as a traced expression")
+        """Symbolic reverse-mode differentiation (core/transform/core.py:119-199 of the reference): after the
+        call every symbol this one was computed from carries its gradient expression in ``.grad``."""
+        from .autodiff import backward as _backward
+        _backward(self, grad)
 
     def __add__(self, other):
         return self.op(Add, [other])

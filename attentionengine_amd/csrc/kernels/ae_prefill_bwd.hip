@@ -35,13 +35,18 @@
 // (LDS fragments, MFMA results, the p/ds arithmetic between two sets of MFMAs) and the second wave
 // fills it - 0.59 -> 0.44 ms for B2 H32 S4096 D128 causal.
 //
+// AE_BWD_KIND 2: online functions with one final row scale of their own (retention): p and ds come from the
+// generated ae_bwd_pd2, which holds the traced OnlineFunc.forward / OnlineFunc.backward
+// (attention_engine/core/lower/lower.py:413-453 of the reference), the symbolic derivative of score_mod and
+// the reads of its custom inputs (per score where they have a kv dimension); the `lse` argument carries
+// that row scale.
 // AE_BWD_KIND 1: graphs whose online function does nothing, out = sum_kv f(s) v with f = score_mod (sigmoid
 // and relu attention, attn_script/sigmoidattn.py, reluattn.py): p = f(s), ds = dp * f'(s), both from the
 // generated ae_bwd_pd (f' by symbolic differentiation of the traced score_mod); no row scales, scale 1.
 //
 // Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0, 1, 2) AE_HAS_MASK_MOD
 // AE_SM_SCALE AE_BWD_ROLE AE_BWD_KIND, optional AE_BWD_NWAVES (4 or 8) AE_BWD_WAVES_PER_EU AE_AHEAD.  Functors used ("ae_functors.h"): ae_mask_mod; kind 1: ae_bwd_pd,
-// ae_bwd_load_custom.
+// ae_bwd_load_custom; kind 2: ae_bwd_pd2.
 
 #include "ae_hip.h"
 #include "ae_config.h"
@@ -419,11 +424,15 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #if AE_BWD_KIND == 0
         float pv = ae_exp2(__builtin_fmaf(sacc[r], AE_SM_SCALE * AE_LOG2E, -l2));
         const float dfac = pacc[r] - dl;
-#else
+#elif AE_BWD_KIND == 1
         float pv, dfac;
         ae_bwd_pd(sacc[r], (float)b, (float)hq, (float)qi, (float)ki, cust, pv, dfac);
         dfac *= pacc[r];
         (void)l2; (void)dl;
+#else
+        // traced OnlineFunc.forward / backward: l2 is the row's final row scale as the forward wrote it
+        float pv, dfac;
+        ae_bwd_pd2(sacc[r], pacc[r], l2, dl, b, hq, qi, ki, p, pv, dfac);
 #endif
         bool vis = true;
         if (decltype(masked)::value) {
@@ -557,8 +566,13 @@ void ae_bwd_delta_kernel(const ae_attn_bwd_params p) {
     const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + s;
     const float l = p.lse ? p.lse[ri] : 0.f;
     p.delta[ri] = acc;
+#if AE_BWD_KIND == 2
+    // second plane: the online function's final row scale, as the forward wrote it
+    p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = l;
+#else
     // second plane: lse in log2 units, +inf for a row without a visible key (its p is 0 everywhere)
     p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;
+#endif
   }
 }
 #endif

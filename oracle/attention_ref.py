@@ -175,6 +175,29 @@ def retention_attention(q, k, v, mask, compute_dtype=torch.float32):
     return _apply_p(s / r, v, compute_dtype), r.reshape(B, Hq, Sq)
 
 
+def retention_attention_grads(q, k, v, mask, do, compute_dtype=torch.float32):
+    """Gradients (dq, dk, dv) the reference's backward produces for attn_script/retention.py: recompute
+    p = (s * mask) / r with the SAVED row scale r (OnlineRetention.forward, retention.py:60-63),
+    dv = p^T do, dp = do v^T, dscores = dp / r (OnlineRetention.backward, retention.py:65-70: r is a
+    constant there, its dependence on the scores is not differentiated), score_mod's derivative (the mask,
+    retention.py:14-16), dq = ds k, dk = ds^T q.  Pinned in tests/test_oracle.py against torch.autograd
+    through ``retention_attention``'s formula with r detached."""
+    B, Sq, Hq, D = q.shape
+    Skv, Hkv = k.shape[1], k.shape[2]
+    G = Hq // Hkv
+    m = mask.to(compute_dtype).expand(B, Hq, Sq, Skv).reshape(B, Hkv, G, Sq, Skv)
+    s = _grouped_scores(q, k, compute_dtype) * m
+    r = s.abs().sum(dim=-1, keepdim=True).clamp(min=1.0)
+    p = s / r
+    dog = do.to(compute_dtype).reshape(B, Sq, Hkv, G, -1)
+    dv = torch.einsum("bhgst,bshgd->bthd", p, dog)
+    dp = torch.einsum("bshgd,bthd->bhgst", dog, v.to(compute_dtype))
+    ds = dp / r * m
+    dq = torch.einsum("bhgst,bthd->bshgd", ds, k.to(compute_dtype)).reshape(B, Sq, Hq, D)
+    dk = torch.einsum("bhgst,bshgd->bthd", ds, q.to(compute_dtype).reshape(B, Sq, Hkv, G, D))
+    return dq, dk, dv
+
+
 def mla_decode(q, q_pe, kv, k_pe, scale=None, compute_dtype=torch.float32):
     """MLA decode: K = [kv | k_pe], V = kv, one latent kv head shared by all q heads.
 

@@ -391,3 +391,39 @@ def test_inferred_block_mask_granularity_does_not_reach_the_kernel():
     assert op.block_mask is not None and op.block_mask.shape == (1, 2, 3, 4)
     plan = op._plan(1, 2, 384, 384, device=None)
     assert (plan.block_m, plan.block_n) == (op.tiles.block_m, op.tiles.block_n)
+
+
+def test_traced_backward_of_an_online_function_with_its_own_row_scale():
+    """attn_script/retention.py: OnlineFunc.forward / backward are traced into ae_bwd_pd2 together with the
+    derivative of score_mod (the decay mask, read per score); an online function that keeps row scales
+    without defining them gets no backward."""
+    from core.lower.prefill_bwd_op import lower_traced_backward
+    src, name = lower_traced_backward(C.retention_score_mod, C.OnlineRetention(), C.retention_custom_inputs(),
+                                      torch.float16)
+    assert name == "r" and "ae_bwd_pd2" in src
+    assert "p.custom[0]" in src and "p.seqlen_kv" in src          # the mask element of (head, q, kv)
+    body = src.split("ae_bwd_pd2", 2)[-1]
+    assert "rs0" in body and "cv_mask" in body and "dp" in body
+    with pytest.raises(NotImplementedError, match="forward"):
+        lower_traced_backward(C.retention_score_mod, C.OnlineAbsNorm(), C.retention_custom_inputs(), torch.float16)
+
+
+def test_symbol_backward_leaves_gradient_expressions_on_the_leaves():
+    """SymbolScalar.backward (core/transform/core.py:119-199 of the reference): after
+    ``f(x, y).backward(g)`` the leaves carry g * df/dx and g * df/dy as traced expressions; evaluated by the
+    oracle's graph interpreter against torch.autograd."""
+    from oracle.online_interp import evaluate
+    x = SymbolScalar("x", Var("x"), shape_idx=[])
+    y = SymbolScalar("y", Var("y"), shape_idx=[])
+    g = SymbolScalar("g", Var("g"), shape_idx=[])
+    f = (x * y + x.exp()) / (y * y + 2.0) - (x * 0.5).tanh()
+    f.backward(g)
+    assert x.grad is not None and y.grad is not None
+    xv = torch.linspace(-1.5, 1.2, 17, dtype=torch.float64).requires_grad_(True)
+    yv = torch.linspace(0.3, 2.1, 17, dtype=torch.float64).requires_grad_(True)
+    gv = torch.linspace(-0.7, 0.9, 17, dtype=torch.float64)
+    ref = (xv * yv + xv.exp()) / (yv * yv + 2.0) - (xv * 0.5).tanh()
+    gx, gy = torch.autograd.grad(ref, (xv, yv), gv)
+    env = {id(x): xv.detach(), id(y): yv.detach(), id(g): gv}
+    assert torch.allclose(evaluate(x.grad, env), gx, atol=1e-12)
+    assert torch.allclose(evaluate(y.grad, env), gy, atol=1e-12)

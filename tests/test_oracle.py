@@ -264,3 +264,36 @@ def test_elementwise_gradients_match_autograd():
                                                    compute_dtype=torch.float64, **kw)
         for a, b in ((dq, gq), (dk, gk), (dv, gv)):
             assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)
+
+
+def test_retention_gradients_match_autograd_with_a_constant_row_scale():
+    """The backward rule of attn_script/retention.py:60-70 treats the saved row scale r as a constant: the
+    oracle's closed-form gradients against torch.autograd through out = ((q k^T) * mask / r.detach()) v in
+    fp64, with grouped heads and rows on both sides of the clamp (some r = 1, some r > 1).  With r
+    differentiated as well, autograd gives something else -- checked, so the test cannot pass vacuously."""
+    g = torch.Generator().manual_seed(8)
+    B, Sq, Skv, Hq, Hkv, D, DV = 2, 9, 9, 4, 2, 8, 6
+    q = torch.randn(B, Sq, Hq, D, generator=g, dtype=torch.float64, requires_grad=True)
+    k = torch.randn(B, Skv, Hkv, D, generator=g, dtype=torch.float64, requires_grad=True)
+    v = torch.randn(B, Skv, Hkv, DV, generator=g, dtype=torch.float64, requires_grad=True)
+    do = torch.randn(B, Sq, Hq, DV, generator=g, dtype=torch.float64)
+    mask = (torch.rand(1, Hq, Sq, Skv, generator=g, dtype=torch.float64) * 0.6).tril()
+    G = Hq // Hkv
+
+    def forward(detach_r):
+        kk = k.repeat_interleave(G, dim=2)
+        s = torch.einsum("bshd,bthd->bhst", q, kk) * mask
+        r = s.abs().sum(-1, keepdim=True).clamp(min=1.0)
+        assert (r == 1.0).any() and (r > 1.0).any()
+        p = s / (r.detach() if detach_r else r)
+        return torch.einsum("bhst,bthd->bshd", p, v.repeat_interleave(G, dim=2))
+    out = forward(True)
+    ref_out, _ = R.retention_attention(q.detach(), k.detach(), v.detach(), mask, compute_dtype=torch.float64)
+    assert torch.allclose(out, ref_out, atol=1e-12)
+    gq, gk, gv = torch.autograd.grad(out, (q, k, v), do)
+    dq, dk, dv = R.retention_attention_grads(q.detach(), k.detach(), v.detach(), mask, do,
+                                             compute_dtype=torch.float64)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)
+    fq, _, _ = torch.autograd.grad(forward(False), (q, k, v), do)
+    assert not torch.allclose(fq, gq, atol=1e-6)

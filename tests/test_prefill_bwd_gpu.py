@@ -166,9 +166,41 @@ def test_sigmoid_and_relu_backward(cuda_device):
         _check(vd.grad, dv, "dv", case)
 
 
+@pytest.mark.parametrize("B,H,Hkv,S,D,DV,dtype", [
+    (1, 2, 2, 256, 64, 128, torch.float16),       # value head dim twice the key head dim, as in the script
+    (2, 4, 2, 200, 128, 128, torch.bfloat16),     # ragged tiles, grouped heads, batch > 1 against a [1,H,S,S] mask
+    (1, 3, 3, 448, 128, 64, torch.float16),
+])
+def test_retention_backward(cuda_device, B, H, Hkv, S, D, DV, dtype):
+    """attn_script/retention.py with its forward() / backward() rules: the traced backward (the saved row
+    scale r as a constant, the decay mask read per score and as the derivative of score_mod) against the
+    oracle's closed form."""
+    print(f"case retention backward B{B} H{H} Hkv{Hkv} S{S} D{D} DV{DV} {dtype}", flush=True)
+    q, k, v = C.make_inputs(B, S, S, H, Hkv, D, DV, dtype, seed=21)
+    q = (q.float() * (1 / D) ** 0.5).to(dtype)                       # bench_utils.py:1034-1036 of the reference
+    g = torch.Generator().manual_seed(22)
+    mask = (torch.rand(1, H, S, S, generator=g) * 1.5).tril().to(dtype).contiguous()
+    do = torch.randn(B, S, H, DV, generator=g).to(dtype)
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+            meta_tensor(B, Hkv, S, DV, dtype=dtype))
+    mod = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
+                          mask_mod=C.causal_mask, online_func=C.OnlineRetention(), mask_value="0")
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = mod(qd, kd, vd, mask.cuda())
+    ref, r = R.retention_attention(q, k, v, mask)
+    assert (r > 1.0).any() and (r == 1.0).any()
+    assert (out.detach().float().cpu() - ref).abs().max().item() <= 2e-2
+    out.backward(do.cuda())
+    dq, dk, dv = R.retention_attention_grads(q, k, v, mask, do)
+    case = (B, H, Hkv, S, D, DV, dtype)
+    _check(qd.grad, dq, "dq", case)
+    _check(kd.grad, dk, "dk", case)
+    _check(vd.grad, dv, "dv", case)
+
+
 def test_backward_of_other_graphs_is_refused(cuda_device):
-    """Softmax attention and graphs whose online function does nothing have a backward; an online function
-    that keeps other row scales (here: the running sum of |s|) says it has none."""
+    """An online function that keeps row scales of its own but defines no forward() / backward() rules
+    (here: the running sum of |s| without them) says it has no backward."""
     B, H, S, D = 1, 2, 128, 64
     meta = (meta_tensor(B, H, S, D, dtype=torch.float16),) * 3
     mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(0.125), mask_mod=None,
