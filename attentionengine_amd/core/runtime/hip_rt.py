@@ -62,6 +62,9 @@ class AttnParams(C.Structure):
         ("mask_block_m", C.c_int32), ("mask_block_n", C.c_int32),
         ("num_splits", C.c_int32), ("kv_per_split", C.c_int32),
         ("reserved", C.c_int32 * 3),
+        ("block_table", C.c_void_p), ("seqlens_k", C.c_void_p),
+        ("block_table_stride", C.c_int32), ("page_block_size", C.c_int32), ("num_pages", C.c_int32),
+        ("reserved2", C.c_int32),
     ]
 
 
@@ -84,7 +87,7 @@ class TileCfg(C.Structure):
         ("block_m", C.c_int32), ("block_n", C.c_int32), ("threads", C.c_int32),
         ("lds_bytes", C.c_int32), ("head_dim", C.c_int32), ("head_dim_v", C.c_int32),
         ("elem_bytes", C.c_int32), ("n_rowscales", C.c_int32), ("mask_mode", C.c_int32),
-        ("reserved", C.c_int32 * 3),
+        ("paged", C.c_int32), ("reserved", C.c_int32 * 2),
     ]
 
 
@@ -275,6 +278,7 @@ def compile_module(template: str, headers: dict, arch: str = None, use_cache: bo
         "ae_hip.h": _read(osp.join(INCLUDE_DIR, "ae_hip.h")),
         "ae_device.h": _read(osp.join(KERNEL_DIR, "ae_device.h")),
         "ae_combine.h": _read(osp.join(KERNEL_DIR, "ae_combine.h")),
+        "ae_mla_paged.h": _read(osp.join(KERNEL_DIR, "ae_mla_paged.h")),
     }
     all_headers.update(headers)
     hsh = hashlib.sha256()

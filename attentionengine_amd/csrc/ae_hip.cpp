@@ -302,7 +302,7 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes, const uint3
   return AE_OK;
 }
 
-static int check_common(const char* who, const ae_attn_params* p, const ae_tile_cfg* cfg) {
+static int check_common(const char* who, const ae_attn_params* p, const ae_tile_cfg* cfg, bool paged_ok = false) {
   if (!p || !cfg) return fail(AE_ERR_INVALID_ARG, "%s: params/cfg is NULL", who);
   if (!p->q || !p->k || !p->v || !p->out)
     return fail(AE_ERR_INVALID_ARG, "%s: q/k/v/out pointer is NULL", who);
@@ -319,6 +319,9 @@ static int check_common(const char* who, const ae_attn_params* p, const ae_tile_
                 who, cfg->block_m, cfg->block_n, cfg->threads, cfg->lds_bytes);
   if (cfg->n_rowscales < 0 || cfg->n_rowscales > AE_MAX_ROWSCALES)
     return fail(AE_ERR_INVALID_ARG, "%s: n_rowscales=%d out of range", who, cfg->n_rowscales);
+  // only ae_mla_decode_fwd knows the paged cache (and checks the table's geometry itself)
+  if (!paged_ok && (cfg->paged || p->block_table || p->seqlens_k))
+    return fail(AE_ERR_INVALID_ARG, "%s: a block table / per-entry lengths were passed to a launch that reads a dense cache", who);
   if (cfg->mask_mode == 2) {
     if (!p->block_mask) return fail(AE_ERR_INVALID_ARG, "%s: block-mask kernel without a mask", who);
     if (p->mask_block_m <= 0 || p->mask_block_n <= 0 || p->mask_nq <= 0 || p->mask_nkv <= 0)
@@ -458,8 +461,25 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
                       const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
   if (!split || !combine_cfg)
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: kernel/cfg is NULL");
-  int rc = check_common("ae_mla_decode_fwd", p, cfg);
+  int rc = check_common("ae_mla_decode_fwd", p, cfg, true);
   if (rc) return rc;
+  if (cfg->paged) {
+    if (!p->block_table || !p->seqlens_k)
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: paged kernel without block_table / seqlens_k");
+    if (p->page_block_size <= 0 || p->page_block_size % cfg->block_n != 0)
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: pages of %d tokens are not a multiple of the %d-token kv tile",
+                  p->page_block_size, cfg->block_n);
+    if (p->num_pages <= 0)
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: num_pages=%d", p->num_pages);
+    if ((int64_t)p->block_table_stride * p->page_block_size < p->seqlen_kv)
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: %d table entries of %d tokens do not cover Skv=%d",
+                  p->block_table_stride, p->page_block_size, p->seqlen_kv);
+    if (p->kv_per_split % cfg->block_n != 0)
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: kv_per_split=%d is not a multiple of the %d-token kv tile",
+                  p->kv_per_split, cfg->block_n);
+  } else if (p->block_table || p->seqlens_k) {
+    return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: block_table / seqlens_k passed to a kernel built for a dense cache");
+  }
   // with one split the kernel writes `out` itself and no merge pass runs
   const bool direct = p->num_splits == 1;
   if (!direct && !combine)

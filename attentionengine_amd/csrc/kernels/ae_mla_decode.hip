@@ -59,6 +59,13 @@ static_assert(AE_CPR % 8 == 0 && AE_CPR1 % 8 == 0, "chunk groups of eight must n
 static_assert((AE_BN * AE_CPR) % 64 == 0, "tile must be a whole number of 1 KiB blocks");
 static_assert(2 * AE_LOADS <= 63, "vmcnt bookkeeping");
 
+#ifndef AE_PAGED
+#define AE_PAGED 0
+#endif
+#if AE_PAGED
+#include "ae_mla_paged.h"
+#endif
+
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 
 extern "C" __global__ __launch_bounds__(AE_NT)
@@ -98,13 +105,31 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
 #pragma unroll
   for (int ks = 0; ks < AE_D2 / 32; ks++) qf[AE_D1 / 32 + ks] = *(const ae_elem8*)(q2 + ks * 32 + g4 * 8);
 
+#if AE_PAGED
+  // paged cache (cute_template_kvshared/kernels/params.h:33-36): rows are found through the block table,
+  // every batch entry has its own length; a kv tile never straddles two pages
+  const ae_elem* k1 = (const ae_elem*)p.k + (int64_t)hk * p.k_stride_h;
+  const ae_elem* k2 = (const ae_elem*)p.k2 + (int64_t)hk * p.k2_stride_h;
+  const int32_t* pages = p.block_table + (int64_t)b * p.block_table_stride;
+  int seqlen_b = p.seqlens_k[b];
+  seqlen_b = seqlen_b < p.seqlen_kv ? seqlen_b : p.seqlen_kv;
+  seqlen_b = __builtin_amdgcn_readfirstlane(seqlen_b > 0 ? seqlen_b : 0);
+#else
   const ae_elem* k1 = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
   const ae_elem* k2 = (const ae_elem*)p.k2 + (int64_t)b * p.k2_stride_b + (int64_t)hk * p.k2_stride_h;
+  const int seqlen_b = p.seqlen_kv;
+#endif
 
   const int kv_begin = split * p.kv_per_split;
   int kv_end = kv_begin + p.kv_per_split;
-  kv_end = kv_end < p.seqlen_kv ? kv_end : p.seqlen_kv;
+  kv_end = kv_end < seqlen_b ? kv_end : seqlen_b;
   const int n_tiles = kv_end > kv_begin ? (kv_end - kv_begin + AE_BN - 1) / AE_BN : 0;
+#if AE_PAGED
+  if (n_tiles == 0) {       // a split beyond this entry's length
+    ae_mla_write_no_keys(p, b, hk, ht, split, group, tid);
+    return;
+  }
+#endif
 
   // Direct HBM -> LDS tile load.  Instruction i of wave w fills the 1 KiB block
   // (w*AE_LOADS + i) mod AE_BLOCKS (a few blocks are fetched twice so every wave issues the same
@@ -113,6 +138,19 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   auto load_tile = [&](int t, int stage) {
     const int kv0 = kv_begin + t * AE_BN;
     ae_lds_byte* dst = lds + stage * AE_STAGE_BYTES;
+#if AE_PAGED
+    // t < n_tiles, so kv0 < seqlen_b and its table entry is set; an entry outside the cache is clamped
+    const int slot = kv0 / p.page_block_size;
+    int page = pages[slot];
+    page = page < 0 ? 0 : (page < p.num_pages ? page : p.num_pages - 1);
+    page = __builtin_amdgcn_readfirstlane(page);
+    const int page_row0 = slot * p.page_block_size;
+    const ae_elem* k1t = k1 + (int64_t)page * p.k_stride_b - (int64_t)page_row0 * p.k_stride_s;
+    const ae_elem* k2t = k2 + (int64_t)page * p.k2_stride_b - (int64_t)page_row0 * p.k2_stride_s;
+#else
+    const ae_elem* k1t = k1;
+    const ae_elem* k2t = k2;
+#endif
 #pragma unroll
     for (int i = 0; i < AE_LOADS; i++) {
       const int blk = (wave * AE_LOADS + i) % AE_BLOCKS;
@@ -120,9 +158,9 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
       const int row = sidx / AE_CPR, cp = sidx % AE_CPR;
       const int c = cp ^ AE_SWZ(row);
       int kv = kv0 + row;
-      kv = kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
-      const ae_elem* src = c < AE_CPR1 ? k1 + (int64_t)kv * p.k_stride_s + c * 8
-                                       : k2 + (int64_t)kv * p.k2_stride_s + (c - AE_CPR1) * 8;
+      kv = kv < seqlen_b ? kv : seqlen_b - 1;
+      const ae_elem* src = c < AE_CPR1 ? k1t + (int64_t)kv * p.k_stride_s + c * 8
+                                       : k2t + (int64_t)kv * p.k2_stride_s + (c - AE_CPR1) * 8;
       ae_load_lds16(src, dst + blk * 1024);
     }
   };

@@ -26,7 +26,9 @@
 // waiting until only the newest tile request is outstanding.
 //
 // Configuration ("ae_config.h"): AE_D1 AE_D2 AE_DV AE_DTYPE_BF16 AE_N_ROWSCALES AE_NSPLIT
-// AE_COMBINE_THREADS, plus AE_SM_SCALE (the constant c > 0) and AE_SM_M / AE_SM_R (names of the
+// AE_COMBINE_THREADS AE_PAGED (1: the cache is paged, rows are found through ae_attn_params.block_table and
+// every batch entry has its own length seqlens_k[b], as in the reference's
+// cute_template_kvshared/kernels/params.h:33-36; a kv tile never straddles two pages), plus AE_SM_SCALE (the constant c > 0) and AE_SM_M / AE_SM_R (names of the
 // running-max and running-sum fields of ae_rowstate).  Functors used ("ae_functors.h"): ae_rowstate,
 // ae_rowstate_init, ae_epilogue, ae_load_custom, ae_combine.
 
@@ -76,6 +78,13 @@ static_assert((AE_BN * AE_CPR) % 64 == 0, "tile must be a whole number of 1 KiB 
 static_assert(AE_L1 <= 8 && AE_L2 >= 1 && AE_BLOCKS >= AE_LOADS, "two bursts of at most eight loads per wave and tile");
 static_assert(AE_NSTAGE >= 3, "a tile is multiplied by K one trip before it is multiplied as V");
 
+#ifndef AE_PAGED
+#define AE_PAGED 0
+#endif
+#if AE_PAGED
+#include "ae_mla_paged.h"
+#endif
+
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 typedef __attribute__((address_space(3))) float ae_lds_f32;
 typedef __attribute__((address_space(3))) int ae_lds_i32;
@@ -92,7 +101,6 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool score_wave = wave < 2;
-  if (wave == 4 || wave == 5) return;      // placeholders: they only steer the value waves onto SIMD 2, 3
 
   // ---- which (head tile, split, kv head, batch): 1-D grid, ids 8 apart share their KV range ---------
   const int group = p.heads_q / p.heads_kv;
@@ -105,13 +113,32 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   const int hk = (u / p.num_splits) % p.heads_kv;
   const int b = u / (p.num_splits * p.heads_kv);
 
+#if AE_PAGED
+  const ae_elem* k1 = (const ae_elem*)p.k + (int64_t)hk * p.k_stride_h;
+  const ae_elem* k2 = (const ae_elem*)p.k2 + (int64_t)hk * p.k2_stride_h;
+  const int32_t* pages = p.block_table + (int64_t)b * p.block_table_stride;
+  int seqlen_b = p.seqlens_k[b];
+  seqlen_b = seqlen_b < p.seqlen_kv ? seqlen_b : p.seqlen_kv;
+  seqlen_b = __builtin_amdgcn_readfirstlane(seqlen_b > 0 ? seqlen_b : 0);
+#else
   const ae_elem* k1 = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
   const ae_elem* k2 = (const ae_elem*)p.k2 + (int64_t)b * p.k2_stride_b + (int64_t)hk * p.k2_stride_h;
+  const int seqlen_b = p.seqlen_kv;
+#endif
 
   const int kv_begin = split * p.kv_per_split;
   int kv_end = kv_begin + p.kv_per_split;
-  kv_end = kv_end < p.seqlen_kv ? kv_end : p.seqlen_kv;
+  kv_end = kv_end < seqlen_b ? kv_end : seqlen_b;
   const int n_tiles = kv_end > kv_begin ? (kv_end - kv_begin + AE_BN - 1) / AE_BN : 0;
+#if AE_PAGED
+  // a split beyond this entry's length: nothing to read (its table entries may be unset), the partial
+  // result is "no keys"
+  if (n_tiles == 0) {
+    ae_mla_write_no_keys(p, b, hk, ht, split, group, tid);
+    return;
+  }
+#endif
+  if (wave == 4 || wave == 5) return;      // placeholders: they only steer the value waves onto SIMD 2, 3
 
   if (score_wave) {
     // =============================== score wave: 32 heads ==============================================
@@ -245,10 +272,15 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     const int sidx = (blk0 + i) * 64 + lane;
     const int row = sidx / AE_CPR, cp = sidx % AE_CPR;
     const int c = cp ^ AE_SWZ(row);
+#if AE_PAGED
+    const int row0 = row;            // the tile's page and first row inside it are added per tile
+#else
+    const int row0 = kv_begin + row;
+#endif
     if (c < AE_CPR1) {
-      ld_ptr[i] = (const char*)(k1 + c * 8) + (int64_t)(kv_begin + row) * stride1;
+      ld_ptr[i] = (const char*)(k1 + c * 8) + (int64_t)row0 * stride1;
     } else {
-      ld_ptr[i] = (const char*)(k2 + (c - AE_CPR1) * 8) + (int64_t)(kv_begin + row) * stride2;
+      ld_ptr[i] = (const char*)(k2 + (c - AE_CPR1) * 8) + (int64_t)row0 * stride2;
       ld_rope |= 1u << i;
     }
     // immediate offset of load i inside its burst
@@ -259,16 +291,30 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     tt = tt < 0 ? 0 : tt;
     const int kv0 = kv_begin + tt * AE_BN;
     ae_lds_byte* dst = lds + (t % AE_NSTAGE) * AE_STAGE_BYTES;
-    const bool ragged = kv0 + AE_BN > p.seqlen_kv;     // wave-uniform
+    const bool ragged = kv0 + AE_BN > seqlen_b;     // wave-uniform
+#if AE_PAGED
+    // tt < n_tiles, so kv0 < seqlen_b and its table entry is set; an entry outside the cache is clamped
+    const int slot = kv0 / p.page_block_size;
+    int page = pages[slot];
+    page = page < 0 ? 0 : (page < p.num_pages ? page : p.num_pages - 1);
+    page = __builtin_amdgcn_readfirstlane(page);
+    const int in_page = kv0 - slot * p.page_block_size;
+    const int64_t tile_off1 = ((int64_t)page * p.k_stride_b + (int64_t)in_page * p.k_stride_s) * 2;
+    const int64_t tile_off2 = ((int64_t)page * p.k2_stride_b + (int64_t)in_page * p.k2_stride_s) * 2;
+#endif
     const void* g[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int j = i < 8 ? (i < AE_L1 ? i : 0) : (i - 8 < AE_L2 ? AE_L1 + i - 8 : AE_L1);
       const unsigned stride = ((ld_rope >> j) & 1u) ? stride2 : stride1;
+#if AE_PAGED
+      g[i] = ld_ptr[j] + (((ld_rope >> j) & 1u) ? tile_off2 : tile_off1);
+#else
       g[i] = ld_ptr[j] + (uint64_t)((unsigned)(tt * AE_BN) * (uint64_t)stride);
+#endif
       if (__builtin_expect(ragged, 0)) {                      // rows past the end re-read the last row
         const int row = ((blk0 + j) * 64 + lane) / AE_CPR;
-        int over = kv0 + row - (p.seqlen_kv - 1);
+        int over = kv0 + row - (seqlen_b - 1);
         over = over > 0 ? over : 0;
         g[i] = (const char*)g[i] - (uint64_t)((unsigned)over * (uint64_t)stride);
       }

@@ -49,7 +49,7 @@ using __hip_internal::uint64_t;
 extern "C" {
 #endif
 
-#define AE_ABI_VERSION 3
+#define AE_ABI_VERSION 4
 
 typedef enum ae_status {
   AE_OK = 0,
@@ -98,6 +98,19 @@ typedef struct ae_attn_params {
   int32_t num_splits;                        /* decode: KV splits per (batch, q-head)     */
   int32_t kv_per_split;                      /* decode: KV positions per split            */
   int32_t reserved[3];
+  /* MLA decode on a paged cache (kernels whose ae_tile_cfg.paged is 1; NULL / 0 otherwise): the cache is
+   * [num_pages, page_block_size, Hkv, D] (k_stride_b = elements between pages, k_stride_s between the
+   * rows of a page), token t of batch entry b is row t % page_block_size of page
+   * block_table[b * block_table_stride + t / page_block_size], and entry b holds
+   * min(seqlens_k[b], seqlen_kv) tokens.  Stands where the reference passes block_table,
+   * block_table_batch_stride, page_block_size and seqlens_k_ptr
+   * (core/template/cute_template_kvshared/kernels/params.h:33-36, flash_api.cpp:61-72). */
+  const int32_t* block_table;                /* int32 [B, block_table_stride]             */
+  const int32_t* seqlens_k;                  /* int32 [B]                                 */
+  int32_t block_table_stride;                /* entries per batch row of block_table      */
+  int32_t page_block_size;                   /* tokens per page, a multiple of block_n    */
+  int32_t num_pages;                         /* pages in the cache: table entries are clamped to it */
+  int32_t reserved2;
 } ae_attn_params;
 
 /* Static facts of one compiled kernel instance, filled by the code generator. */
@@ -111,7 +124,8 @@ typedef struct ae_tile_cfg {
   int32_t elem_bytes;  /* 2 for fp16/bf16                                                 */
   int32_t n_rowscales; /* number of final rowscales the kernel writes                     */
   int32_t mask_mode;   /* 0 none, 1 analytic causal, 2 block table                        */
-  int32_t reserved[3];
+  int32_t paged;       /* MLA decode: 1 when the kernel reads KV through block_table / seqlens_k */
+  int32_t reserved[2];
 } ae_tile_cfg;
 
 /*

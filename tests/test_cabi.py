@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in ae_hip.h but not exported"
     assert sorted(rt.EXPORTED_SYMBOLS) == names
-    assert rt.lib().ae_abi_version() == 3
+    assert rt.lib().ae_abi_version() == 4
 
 
 def test_struct_layout_matches_the_header():
@@ -41,8 +41,8 @@ def test_struct_layout_matches_the_header():
     from include/ae_hip.h, equal the ctypes mirrors: a probe whose static_asserts carry the ctypes figures
     is compiled for gfx950 through ae_compile (needs no GPU).  A reordered or retyped field of equal size
     in either place fails the compilation."""
-    # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints
-    assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16
+    # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints, then the paged-cache part: 2 pointers, 3 + 1 ints
+    assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16 + 8 * 2 + 4 * 4
     assert ctypes.sizeof(rt.TileCfg) == 4 * 12
     # backward: 12 + 4 pointers, 8 tensors x 3 strides, 7 + 1 ints
     assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 16 + 8 * 24 + 4 * 8
@@ -114,6 +114,54 @@ def test_bad_arguments_fail_without_exiting(tmp_path):
     p, cfg = rt.AttnParams(), rt.TileCfg()
     assert lib.ae_prefill_fwd(None, ctypes.byref(p), ctypes.byref(cfg), None) == 1
     assert lib.ae_device_info(0, None) == 1
+
+
+def test_paged_cache_arguments_are_checked_before_any_launch():
+    """ae_mla_decode_fwd refuses an inconsistent block table; the other launches refuse any.  Every case
+    fails in the argument checks, so the kernel handle (never dereferenced before them) is a dummy."""
+    lib = rt.lib()
+    fake = ctypes.c_void_p(8)
+    buf = ctypes.create_string_buffer(64)
+    addr = ctypes.addressof(buf)
+
+    def params(**kw):
+        p = rt.AttnParams()
+        p.q = p.k = p.v = p.out = p.q2 = p.k2 = addr
+        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = 2, 128, 1, 1, 256
+        p.num_splits, p.kv_per_split = 1, 256
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
+
+    def cfg(**kw):
+        c = rt.TileCfg(block_m=64, block_n=32, threads=512, lds_bytes=1024, head_dim=576, head_dim_v=512,
+                       elem_bytes=2, n_rowscales=0, mask_mode=0)
+        for k, v in kw.items():
+            setattr(c, k, v)
+        return c
+
+    def mla(p, c):
+        cc = rt.TileCfg(block_m=1, block_n=p.num_splits, threads=128)
+        rc = lib.ae_mla_decode_fwd(fake, fake, ctypes.byref(p), ctypes.byref(c), ctypes.byref(cc), None)
+        return rc, lib.ae_last_error().decode()
+
+    rc, msg = mla(params(), cfg(paged=1))
+    assert rc == 1 and "without block_table" in msg
+    table = dict(block_table=addr, seqlens_k=addr, block_table_stride=4, page_block_size=64, num_pages=8)
+    rc, msg = mla(params(**table), cfg())
+    assert rc == 1 and "built for a dense cache" in msg
+    rc, msg = mla(params(**{**table, "page_block_size": 48}), cfg(paged=1))
+    assert rc == 1 and "not a multiple of the 32-token kv tile" in msg
+    rc, msg = mla(params(**{**table, "block_table_stride": 3}), cfg(paged=1))
+    assert rc == 1 and "do not cover Skv=256" in msg
+    rc, msg = mla(params(**{**table, "num_pages": 0}), cfg(paged=1))
+    assert rc == 1 and "num_pages" in msg
+    p = params(**table)
+    assert lib.ae_prefill_fwd(fake, ctypes.byref(p), ctypes.byref(cfg()), None) == 1
+    assert "reads a dense cache" in lib.ae_last_error().decode()
+    cc = rt.TileCfg(block_m=1, block_n=1, threads=128)
+    assert lib.ae_decode_fwd(fake, fake, ctypes.byref(p), ctypes.byref(cfg()), ctypes.byref(cc), None) == 1
+    assert "reads a dense cache" in lib.ae_last_error().decode()
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")

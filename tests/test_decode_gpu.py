@@ -198,6 +198,55 @@ def test_mla_decode_cute_convention(cuda_device):
     assert (x - y).abs().max().item() <= LSE_TOL
 
 
+@pytest.mark.parametrize("kernel", ["ws", "generic"])
+@pytest.mark.parametrize("dtype,B,H,page,lens,target", [
+    (torch.bfloat16, 3, 128, 64, [1000, 37, 640], 256),    # split launch; entry 1 leaves most splits without a key
+    (torch.float16, 2, 16, 32, [513, 2048], 1),            # one split, long loop, ragged tails, 16 of 64 head rows
+    (torch.bfloat16, 2, 64, 128, [128, 1], 8),             # pages larger than a tile, a one-token entry
+])
+def test_mla_decode_paged_cache(cuda_device, monkeypatch, kernel, dtype, B, H, page, lens, target):
+    """mod(q, kv_cache, block_table=..., cache_seqlens=...): pages in a shuffled order, every batch entry
+    with its own length (cute_template_kvshared/flash_api.cpp:61-72, kernels/params.h:33-36).  Unused
+    table entries hold an out-of-range page number and unused pages NaN, so a read beyond an entry's
+    length shows."""
+    print(f"case mla paged {kernel} {dtype} B{B} H{H} page{page} lens{lens} target{target}", flush=True)
+    if kernel == "generic":
+        monkeypatch.setenv("AE_MLA_KERNEL", "generic")
+    G, D, DV = 1, 576, 512
+    scale = 1 / math.sqrt(D)
+    max_pages = -(-max(lens) // page) + 1
+    n_pages = B * max_pages + 3
+    g = torch.Generator().manual_seed(11)
+    perm = torch.randperm(n_pages, generator=g)
+    table = torch.full((B, max_pages), n_pages + 7, dtype=torch.int32)
+    cache = torch.full((n_pages, page, G, D), float("nan"), dtype=dtype)
+    q, q_pe, kv, k_pe = _mla_inputs(B, H, G, max_pages * page, DV, D - DV, dtype, seed=5)
+    dense = torch.cat([kv, k_pe], -1)
+    used = 0
+    for b in range(B):
+        for j in range(-(-lens[b] // page)):
+            pg = int(perm[used]); used += 1
+            table[b, j] = pg
+            cache[pg] = dense[b, j * page:(j + 1) * page]
+    # rows of the last used page beyond the entry's length stay finite (any value): the kernels may load
+    # them, they must not let them reach the result
+    mod = _mla_engine(B, H, G, max_pages * page, D, DV, dtype, scale, backend="cute")
+    mod.attention.target_workgroups = target
+    out, lse = mod(torch.cat([q, q_pe], -1).cuda(), cache.cuda(), block_table=table.cuda(),
+                   cache_seqlens=torch.tensor(lens, dtype=torch.int32).cuda())
+    assert out.shape == (B, 1, H, DV) and lse.shape == (B, H, 1)
+    for b in range(B):
+        n = lens[b]
+        ref, lref = R.mla_decode(q[b:b + 1, 0], q_pe[b:b + 1, 0], kv[b:b + 1, :n], k_pe[b:b + 1, :n], scale=scale)
+        assert (out[b:b + 1, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL, b
+        assert (lse[b:b + 1, :, 0].cpu() - lref).abs().max().item() <= LSE_TOL, b
+    # the same engine still reads a dense cache when no table is given
+    n0 = -(-max(lens) // page) * page
+    out2, _ = mod(torch.cat([q, q_pe], -1).cuda(), dense[:, :n0].reshape(-1, page, G, D).contiguous().cuda())
+    ref, _ = R.mla_decode(q[:, 0], q_pe[:, 0], kv[:, :n0], k_pe[:, :n0], scale=scale)
+    assert (out2[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL
+
+
 def _mha_decode_engine(B, H, Sq, Skv, D, dtype, online, mask_mod=None):
     meta = (meta_tensor(B, H, Sq, D, dtype=dtype), meta_tensor(B, H, Skv, D, dtype=dtype),
             meta_tensor(B, H, Skv, D, dtype=dtype))
