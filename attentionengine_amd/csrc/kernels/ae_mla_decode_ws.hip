@@ -65,6 +65,7 @@
 #define AE_TAU2 8.0f                      // the running maximum (log2 units) is refreshed only when it moved by more
 #define AE_SWZ(r) ((((r) >> 1) & 3) * 2 + (((r) >> 3) & 1))
 #define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+#define AE_VMCNT_LGKM0(n) (0x0070 | ((n) & 15) | (((n) >> 4) << 14))
 #ifndef AE_AHEAD
 #define AE_AHEAD 4
 #endif
@@ -88,6 +89,7 @@ static_assert(AE_NSTAGE >= 3, "a tile is multiplied by K one trip before it is m
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 typedef __attribute__((address_space(3))) float ae_lds_f32;
 typedef __attribute__((address_space(3))) int ae_lds_i32;
+template <bool B> struct ae_const_bool { static constexpr bool value = B; };
 
 extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void ae_mla_decode_split_kernel(const ae_attn_params p) {
@@ -126,10 +128,13 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   const int seqlen_b = p.seqlen_kv;
 #endif
 
-  const int kv_begin = split * p.kv_per_split;
-  int kv_end = kv_begin + p.kv_per_split;
-  kv_end = kv_end < seqlen_b ? kv_end : seqlen_b;
-  const int n_tiles = kv_end > kv_begin ? (kv_end - kv_begin + AE_BN - 1) / AE_BN : 0;
+  // (wave-uniform values are pinned to scalar registers: a copy in a vector register that gets spilled is
+  // reloaded with a scratch load, which the tile loads' vmcnt bookkeeping would have to wait for)
+  const int kv_begin = __builtin_amdgcn_readfirstlane(split * p.kv_per_split);
+  int kv_end_ = kv_begin + p.kv_per_split;
+  kv_end_ = kv_end_ < seqlen_b ? kv_end_ : seqlen_b;
+  const int kv_end = __builtin_amdgcn_readfirstlane(kv_end_);
+  const int n_tiles = __builtin_amdgcn_readfirstlane(kv_end > kv_begin ? (kv_end - kv_begin + AE_BN - 1) / AE_BN : 0);
 #if AE_PAGED
   // a split beyond this entry's length: nothing to read (its table entries may be unset), the partial
   // result is "no keys"
@@ -168,75 +173,104 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     // K fragment of k-step ks: row lane%32, global chunk 2*ks + lane/32
     const int k_row_off = l32s * AE_KSTR;
     const int k_sw = AE_SWZ(l32s);
-    for (int t = -1; t < n_tiles; t++) {
-      const int tn = t + 1;                      // the tile this wave multiplies by Q now
-      if (tn < n_tiles) {
-        const ae_lds_byte* kt = lds + (tn % AE_NSTAGE) * AE_STAGE_BYTES + k_row_off;
-        ae_f32x16 sacc[2];   // even / odd k-steps: two independent MFMA chains
+    // A trip multiplies tile n by Q^T and, in the issue slots between those MFMAs, runs the softmax of tile
+    // n - 1 (its raw scores wait in `xs`): the wave's matrix work and its softmax overlap instead of
+    // following each other.  P of tile n - 1 is handed over by the barrier that ends trip n.
+    ae_f32x16 xs;        // raw scores of the tile before the one being multiplied
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+    for (int r = 0; r < 16; r++) xs[r] = 0.f;
+    // lane owns head lane%32 and kv rows 8*(e/4) + 4*(lane/32) + e%4 of a tile
+    float x[16], mx, mn, osc, rs;
+    bool need;
+    ae_lds_byte* prow;
+    ae_lds_byte* xb;
+    // start of the softmax of tile tp: scores beyond the end of the range are taken out (ragged tail only)
+    auto soft_begin = [&](int tp) {
 #pragma unroll
-          for (int r = 0; r < 16; r++) sacc[c][r] = 0.f;
-        // read AE_AHEAD fragments before the MFMA that uses them (the compiler on its own keeps one read
-        // in flight, which leaves the LDS latency exposed)
-        auto read_kfrag = [&](int ks) -> ae_elem8 {
-          return *(const __attribute__((address_space(3))) ae_elem8*)(kt + (((2 * ks + hfs) ^ k_sw) << 4));
-        };
-        ae_elem8 ring[AE_RING];
+      for (int e = 0; e < 16; e++) x[e] = xs[e];   // raw scores: the scale is folded into the exponent
+      const bool tail = kv_begin + tp * AE_BN + AE_BN > kv_end;
+      if (__builtin_expect(tail, 0)) {
+        // the empty asm keeps this a branch: flattened into selects it costs 5 instructions per score
+        // on every tile
+        asm volatile("" ::: "memory");
+        const int kvb = kv_begin + tp * AE_BN + 4 * hfs;
 #pragma unroll
-        for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int f = 0; f < AE_NKS; f++) {
-          if (f + AE_AHEAD < AE_NKS) ring[(f + AE_AHEAD) % AE_RING] = read_kfrag(f + AE_AHEAD);
-          sacc[f & 1] = ae_mfma32(ring[f % AE_RING], qf[f], sacc[f & 1]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        // lane owns head lane%32 and kv rows 8*(e/4) + 4*(lane/32) + e%4 of the tile
-        float x[16];
-        const int kvb = kv_begin + tn * AE_BN + 4 * hfs;
-        const bool tail = kv_begin + tn * AE_BN + AE_BN > kv_end;
-        float mx = AE_NEG_INF;
-#pragma unroll
-        for (int e = 0; e < 16; e++) x[e] = sacc[0][e] + sacc[1][e];   // raw scores: the scale is folded into the exponent
-        if (__builtin_expect(tail, 0)) {
-          // the empty asm keeps this a branch: flattened into selects it costs 5 instructions per score
-          // on every tile
-          asm volatile("" ::: "memory");
-#pragma unroll
-          for (int e = 0; e < 16; e++) x[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
-        }
-#pragma unroll
-        for (int e = 0; e < 16; e++) mx = __builtin_fmaxf(mx, x[e]);
-        {
-          float hi;
-          const float lo = ae_swap32_lo_hi(mx, hi);
-          mx = __builtin_fmaxf(lo, hi) * (AE_SM_SCALE * AE_LOG2E);   // the scale is positive
-        }
-        const bool need = (mx - m2) > AE_TAU2;
-        const float mn = need ? mx : m2;
-        const float osc = need ? ae_exp2(m2 - mn) : 1.0f;
+        for (int e = 0; e < 16; e++) x[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
+      }
+      mx = AE_NEG_INF;
+      rs = 0.f;
+      prow = pbuf + (tp & 1) * AE_P_BYTES + (wave * 32 + l32s) * AE_PSTR + 8 * hfs;
+      xb = xbuf + (tp & 1) * AE_X_BYTES;
+    };
+    // the softmax of one tile in AE_NKS pieces, piece f issued behind the MFMA of k-step f
+    auto soft_slot = [&](int f) {
+      if (f < 4) {
+        mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[4 * f]), x[4 * f + 1]);
+        mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[4 * f + 2]), x[4 * f + 3]);
+      } else if (f == 4) {
+        float hi;
+        const float lo = ae_swap32_lo_hi(mx, hi);
+        mx = __builtin_fmaxf(lo, hi) * (AE_SM_SCALE * AE_LOG2E);   // the scale is positive
+      } else if (f == 5) {
+        need = (mx - m2) > AE_TAU2;
+        mn = need ? mx : m2;
+        osc = need ? ae_exp2(m2 - mn) : 1.0f;
         m2 = mn;
-        float rs = 0.f;
-        ae_lds_byte* prow = pbuf + (tn & 1) * AE_P_BYTES + (wave * 32 + l32s) * AE_PSTR + 8 * hfs;
+      } else if (f < 22) {
+        const int e = f - 6;
+        x[e] = ae_exp2(__builtin_fmaf(x[e], AE_SM_SCALE * AE_LOG2E, -mn));
+        rs += x[e];
+      } else if (f < 26) {
+        const int rb = f - 22;
+        ae_elem4 w;
 #pragma unroll
-        for (int rb = 0; rb < 4; rb++) {
-          ae_elem4 w;
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const float pv = ae_exp2(__builtin_fmaf(x[4 * rb + i], AE_SM_SCALE * AE_LOG2E, -mn));
-            rs += pv;
-            w[i] = (ae_elem)pv;
-          }
-          *(__attribute__((address_space(3))) ae_elem4*)(prow + 16 * rb) = w;
-        }
+        for (int i = 0; i < 4; i++) w[i] = (ae_elem)x[4 * rb + i];
+        *(__attribute__((address_space(3))) ae_elem4*)(prow + 16 * rb) = w;
+      } else if (f == 26) {
         r_run = r_run * osc + rs;
-        ae_lds_byte* xb = xbuf + (tn & 1) * AE_X_BYTES;
         if (hfs == 0) ((ae_lds_f32*)xb)[wave * 32 + l32s] = osc;
         const bool any = __builtin_amdgcn_ballot_w64(need) != 0;
         if (lane == 0) ((ae_lds_i32*)(xb + AE_HEADS_PER_WG * 4))[wave] = any ? 1 : 0;
       }
-      __syncthreads();                           // end of the trip: P is handed over, tile tn + 1 has landed
+    };
+    static_assert(AE_NKS >= 27, "the softmax of a tile is spread over 27 k-steps");
+    // S^T of tile tn into xs; with SOFT the softmax of tile tn - 1 rides along
+    auto score_trip = [&](int tn, auto with_soft) {
+      constexpr bool SOFT = decltype(with_soft)::value;
+      const ae_lds_byte* kt = lds + (tn % AE_NSTAGE) * AE_STAGE_BYTES + k_row_off;
+      // read AE_AHEAD fragments before the MFMA that uses them (the compiler on its own keeps one read
+      // in flight, which leaves the LDS latency exposed)
+      auto read_kfrag = [&](int ks) -> ae_elem8 {
+        return *(const __attribute__((address_space(3))) ae_elem8*)(kt + (((2 * ks + hfs) ^ k_sw) << 4));
+      };
+      ae_elem8 ring[AE_RING];
+#pragma unroll
+      for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f);
+      if (SOFT) soft_begin(tn - 1);
+      ae_f32x16 sacc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int f = 0; f < AE_NKS; f++) {
+        if (f + AE_AHEAD < AE_NKS) ring[(f + AE_AHEAD) % AE_RING] = read_kfrag(f + AE_AHEAD);
+        sacc = ae_mfma32(ring[f % AE_RING], qf[f], sacc);
+        if (SOFT) soft_slot(f);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      xs = sacc;
+    };
+    if (n_tiles > 0) score_trip(0, ae_const_bool<false>());
+    __syncthreads();                             // end of trip 0: tile 1 has landed
+    for (int tn = 1; tn < n_tiles; tn++) {
+      score_trip(tn, ae_const_bool<true>());
+      __syncthreads();                           // end of the trip: P of tile tn - 1 is handed over, tile tn + 1 has landed
+    }
+    if (n_tiles > 0) {                           // the last tile's softmax has no MFMAs to hide behind
+      soft_begin(n_tiles - 1);
+#pragma unroll
+      for (int f = 0; f < 27; f++) soft_slot(f);
+      __syncthreads();
     }
     // final row state for the value waves
     {
@@ -258,13 +292,14 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   // Direct HBM -> LDS tile load, by the four value waves: wave w fills AE_LOADS consecutive 1 KiB blocks of
   // the tile, starting at block min(w*AE_LOADS, AE_BLOCKS-AE_LOADS) (the last wave overlaps its neighbour, so
   // every wave issues the same number of loads); LDS chunk c' of row r receives global chunk c' ^ f(r).
-  // Which row and chunk a lane fetches never changes, so its source pointer inside the split's first tile
-  // is computed once; per tile only tile * 32 rows * stride is added.  The loads of a wave go out as two
-  // bursts, each behind a single write of M0 (see ae_load_lds16_burst; the pointers carry the
-  // compensation for its immediate offsets).  Tiles past the end re-read the last tile, so every trip
-  // issues the same number of loads; rows past seqlen_kv re-read the last row.
+  // Which row and chunk a lane fetches never changes: its byte offset inside a tile is computed once (one
+  // register per load) and added per tile to the tile's wave-uniform address in the latent or in the rope
+  // tensor.  The loads of a wave go out as two bursts, each behind a single write of M0 (see
+  // ae_load_lds16_burst; the offsets carry the compensation for its immediate offsets).  Tiles past the
+  // end re-read the last tile, so every trip issues the same number of loads; rows past the end re-read
+  // the last row.
   const int blk0 = dvw * AE_LOADS < AE_BLOCKS - AE_LOADS ? dvw * AE_LOADS : AE_BLOCKS - AE_LOADS;
-  const char* ld_ptr[AE_LOADS];   // this lane's source of load i in the first tile of the split
+  int ld_off[AE_LOADS];           // this lane's byte offset of load i inside a tile (may be negative)
   unsigned ld_rope = 0;           // bit i: load i reads from the rope tensor (k2), else from the latent (k1)
   const unsigned stride1 = (unsigned)p.k_stride_s * 2, stride2 = (unsigned)p.k2_stride_s * 2;   // bytes per kv row
 #pragma unroll
@@ -272,21 +307,17 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     const int sidx = (blk0 + i) * 64 + lane;
     const int row = sidx / AE_CPR, cp = sidx % AE_CPR;
     const int c = cp ^ AE_SWZ(row);
-#if AE_PAGED
-    const int row0 = row;            // the tile's page and first row inside it are added per tile
-#else
-    const int row0 = kv_begin + row;
-#endif
     if (c < AE_CPR1) {
-      ld_ptr[i] = (const char*)(k1 + c * 8) + (int64_t)row0 * stride1;
+      ld_off[i] = c * 16 + row * (int)stride1;
     } else {
-      ld_ptr[i] = (const char*)(k2 + (c - AE_CPR1) * 8) + (int64_t)row0 * stride2;
+      ld_off[i] = (c - AE_CPR1) * 16 + row * (int)stride2;
       ld_rope |= 1u << i;
     }
     // immediate offset of load i inside its burst
-    ld_ptr[i] -= i < AE_L1 ? (i - AE_L1 / 2) * 1024 : (i - AE_L1 - AE_L2 / 2) * 1024;
+    ld_off[i] -= i < AE_L1 ? (i - AE_L1 / 2) * 1024 : (i - AE_L1 - AE_L2 / 2) * 1024;
   }
-  auto load_tile = [&](int t) {
+  auto load_tile = [&](int t_) {
+    const int t = __builtin_amdgcn_readfirstlane(t_);
     int tt = t < n_tiles ? t : n_tiles - 1;
     tt = tt < 0 ? 0 : tt;
     const int kv0 = kv_begin + tt * AE_BN;
@@ -299,33 +330,40 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     page = page < 0 ? 0 : (page < p.num_pages ? page : p.num_pages - 1);
     page = __builtin_amdgcn_readfirstlane(page);
     const int in_page = kv0 - slot * p.page_block_size;
-    const int64_t tile_off1 = ((int64_t)page * p.k_stride_b + (int64_t)in_page * p.k_stride_s) * 2;
-    const int64_t tile_off2 = ((int64_t)page * p.k2_stride_b + (int64_t)in_page * p.k2_stride_s) * 2;
-#endif
-    const void* g[16];
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int j = i < 8 ? (i < AE_L1 ? i : 0) : (i - 8 < AE_L2 ? AE_L1 + i - 8 : AE_L1);
-      const unsigned stride = ((ld_rope >> j) & 1u) ? stride2 : stride1;
-#if AE_PAGED
-      g[i] = ld_ptr[j] + (((ld_rope >> j) & 1u) ? tile_off2 : tile_off1);
+    const char* tile1 = (const char*)k1 + ((int64_t)page * p.k_stride_b + (int64_t)in_page * p.k_stride_s) * 2;
+    const char* tile2 = (const char*)k2 + ((int64_t)page * p.k2_stride_b + (int64_t)in_page * p.k2_stride_s) * 2;
 #else
-      g[i] = ld_ptr[j] + (uint64_t)((unsigned)(tt * AE_BN) * (uint64_t)stride);
+    const char* tile1 = (const char*)k1 + (uint64_t)((unsigned)kv0 * (uint64_t)stride1);
+    const char* tile2 = (const char*)k2 + (uint64_t)((unsigned)kv0 * (uint64_t)stride2);
 #endif
+    auto source = [&](int j) -> const void* {
+      const bool rope = (ld_rope >> j) & 1u;
+      int off = ld_off[j];
       if (__builtin_expect(ragged, 0)) {                      // rows past the end re-read the last row
         const int row = ((blk0 + j) * 64 + lane) / AE_CPR;
         int over = kv0 + row - (seqlen_b - 1);
         over = over > 0 ? over : 0;
-        g[i] = (const char*)g[i] - (uint64_t)((unsigned)over * (uint64_t)stride);
+        off -= over * (int)(rope ? stride2 : stride1);
       }
+      return (rope ? tile2 : tile1) + (int64_t)off;
+    };
+    {
+      const void* g[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) g[i] = source(i < AE_L1 ? i : 0);
+      ae_load_lds16_burst<AE_L1>(g, dst + (blk0 + AE_L1 / 2) * 1024);
     }
-    ae_load_lds16_burst<AE_L1>(g, dst + (blk0 + AE_L1 / 2) * 1024);
-    ae_load_lds16_burst<AE_L2>(g + 8, dst + (blk0 + AE_L1 + AE_L2 / 2) * 1024);
+    {
+      const void* g[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) g[i] = source(i < AE_L2 ? AE_L1 + i : AE_L1);
+      ae_load_lds16_burst<AE_L2>(g, dst + (blk0 + AE_L1 + AE_L2 / 2) * 1024);
+    }
   };
   // end of a trip: tile t+2 has landed when only the newest request is outstanding; after the barrier
   // everyone is done with tile t, whose stage takes the next request
   auto end_trip = [&](int t) {
-    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_LOADS));
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT_LGKM0(AE_LOADS));   // ... and this trip's LDS reads have returned
     __syncthreads();
     load_tile(t + AE_NSTAGE);
   };
@@ -346,23 +384,45 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
 
   // V^T fragment (k-step kk, dv block db): A[m = dv][k = kv]: lane i of a 16-lane group supplies the
   // address of row 16*kk + 8*hf + i/4 (+4 for slots 4..7), 8 bytes at value column
-  // 32*db + 16*((lane%32)/16) + 4*(i%4), and receives column i of those four rows.
+  // 32*db + 16*((lane%32)/16) + 4*(i%4), and receives column i of those four rows.  The swizzle of a
+  // row's chunks touches the three low bits of the chunk number only, so a lane has four distinct
+  // offsets (parity of db, first / second group of four rows) and everything else is an immediate.
   const int v_row = 8 * hf + ((lane & 15) >> 2);
   const int v_c0 = 2 * (l32 >> 4) + ((lane & 3) >> 1);
   const int v_half = (lane & 1) * 8;
-  auto read_vfrag = [&](const ae_lds_byte* vt, int kk, int db) -> ae_elem8 {
-    const int r0 = 16 * kk + v_row, r1 = r0 + 4;
-    const int cg = 4 * (dvw * AE_NDB + db) + v_c0;           // global 16-byte chunk
+  int v_base[2][2];     // [db & 1][row group]
+#pragma unroll
+  for (int par = 0; par < 2; par++)
+#pragma unroll
+    for (int rg = 0; rg < 2; rg++) {
+      const int r = v_row + 4 * rg;
+      v_base[par][rg] = r * AE_KSTR + ((((4 * par + v_c0) ^ AE_SWZ(r)) + 4 * AE_NDB * dvw) << 4) + v_half;
+    }
+  static_assert(AE_NDB % 2 == 0, "a value wave's first chunk must be a multiple of eight");
+  auto read_vfrag = [&](const int (&va)[2][2], int kk, int db) -> ae_elem8 {
+    const int imm = 16 * kk * AE_KSTR + (db >> 1) * 128;
     ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)(
-        vt + r0 * AE_KSTR + ((cg ^ AE_SWZ(r0)) << 4) + v_half));
+        lds + va[db & 1][0] + imm));
     ae_s16x4 hi2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)(
-        vt + r1 * AE_KSTR + ((cg ^ AE_SWZ(r1)) << 4) + v_half));
+        lds + va[db & 1][1] + imm));
     return __builtin_bit_cast(ae_elem8, __builtin_shufflevector(lo, hi2, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  for (int t = -1; t < n_tiles; t++) {
-    if (t >= 0) {
-      const ae_lds_byte* vt = lds + (t % AE_NSTAGE) * AE_STAGE_BYTES;
+  // A trip of a value wave: O^T += V^T P^T for tile n - 2 with the V^T fragments it holds in registers (PV),
+  // and the fragments of tile n - 1 read from LDS into those registers as they fall free (RD) - the read
+  // has a whole trip to complete, and tile n - 1's stage can take the next request when the trip ends.
+  ae_elem8 vreg[2 * AE_NDB];     // fragment f = (k-step f / AE_NDB, dv block f % AE_NDB)
+#pragma unroll
+  for (int f = 0; f < 2 * AE_NDB; f++) vreg[f] = (ae_elem8){};
+  auto value_trip = [&](int n, auto with_pv, auto with_rd) {
+    constexpr bool PV = decltype(with_pv)::value;
+    constexpr bool RD = decltype(with_rd)::value;
+    int va[2][2];          // the lane's four fragment offsets inside tile n - 1's stage
+#pragma unroll
+    for (int i = 0; i < 4; i++) va[i >> 1][i & 1] = v_base[i >> 1][i & 1] + ((n - 1) % AE_NSTAGE) * AE_STAGE_BYTES;
+    ae_elem8 pf[2][2];
+    if (PV) {
+      const int t = n - 2;
       const ae_lds_byte* pb = pbuf + (t & 1) * AE_P_BYTES;
       const ae_lds_byte* xb = xbuf + (t & 1) * AE_X_BYTES;
       // rescale O for the heads whose reference moved (rare once the maxima have settled)
@@ -378,32 +438,37 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         }
       }
       // P^T fragments: B[k = kv = 16*kk + 8*hf + j][n = head = 32*hb + l32]
-      ae_elem8 pf[2][2];
 #pragma unroll
       for (int hb = 0; hb < 2; hb++)
 #pragma unroll
         for (int kk = 0; kk < 2; kk++)
           pf[hb][kk] = *(const __attribute__((address_space(3))) ae_elem8*)(
               pb + (hb * 32 + l32) * AE_PSTR + 32 * kk + 16 * hf);
-      // fragment f = (k-step f/NDB, dv block f%NDB), read AE_AHEAD fragments ahead
-      ae_elem8 ring[AE_RING];
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_vfrag(vt, f / AE_NDB, f % AE_NDB);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int f = 0; f < 2 * AE_NDB; f++) {
-        if (f + AE_AHEAD < 2 * AE_NDB)
-          ring[(f + AE_AHEAD) % AE_RING] = read_vfrag(vt, (f + AE_AHEAD) / AE_NDB, (f + AE_AHEAD) % AE_NDB);
+    for (int f = 0; f < 2 * AE_NDB; f++) {
+      if (PV) {
 #pragma unroll
         for (int hb = 0; hb < 2; hb++)
-          oacc[hb][f % AE_NDB] = ae_mfma32(ring[f % AE_RING], pf[hb][f / AE_NDB], oacc[hb][f % AE_NDB]);
-        __builtin_amdgcn_sched_barrier(0);
+          oacc[hb][f % AE_NDB] = ae_mfma32(vreg[f], pf[hb][f / AE_NDB], oacc[hb][f % AE_NDB]);
       }
+      if (RD) vreg[f] = read_vfrag(va, f / AE_NDB, f % AE_NDB);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    end_trip(t);
+  };
+  end_trip(-1);                                                    // trip 0: the score waves multiply tile 0
+  value_trip(1, ae_const_bool<false>(), ae_const_bool<true>());    // trip 1: fragments of tile 0
+  end_trip(0);
+  for (int n = 2; n <= n_tiles; n++) {
+    value_trip(n, ae_const_bool<true>(), ae_const_bool<true>());
+    end_trip(n - 1);
   }
-  __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));
-  __syncthreads();               // final (m, r) of every head are in LDS
+  if (n_tiles > 0) {                                               // trip n_tiles + 1: the last tile's product
+    value_trip(n_tiles + 1, ae_const_bool<true>(), ae_const_bool<false>());
+    end_trip(n_tiles);
+  }
+  __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // (the last barrier also made the final (m, r) of every head visible)
 
   // ---- per-split epilogue: lane owns head 32*hb + l32, value columns AE_DVW*dvw + 32*db + 8*(r/4) + 4*hf + r%4
 #pragma unroll
