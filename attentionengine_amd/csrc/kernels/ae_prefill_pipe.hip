@@ -165,6 +165,17 @@ void ae_prefill_kernel(const ae_attn_params p) {
     j_end = lim < n_kvt ? lim : n_kvt;
   }
 #endif
+  // Under the causal mask a wave's own rows end before the workgroup's: the kv tiles past its diagonal are
+  // invisible to all of its rows.  It does not multiply them (for 256-row q tiles six of the sixteen
+  // (wave, tile) pairs on the diagonal), but keeps requesting its share of every tile and keeps meeting
+  // the others at the barriers.
+  int j_end_w = j_end;
+#if AE_MASK_MODE == 1
+  {
+    int lim = (q0w + AE_WROWS + AE_BN - 1) / AE_BN;
+    j_end_w = lim < j_end ? lim : j_end;
+  }
+#endif
 #if AE_MASK_MODE == 2
   const int8_t* bm_base = p.block_mask +
       ((int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : h)) * p.mask_nq * (int64_t)p.mask_nkv;
@@ -530,11 +541,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #if AE_TOP_PREFETCH
   if (any_tile) prefetch_ring();
 #endif
-  auto iteration = [&](auto has_next_tag) {
+  // HN: the wave multiplies a next tile of its own.  TL (only without HN): it has none, but the other waves
+  // have, so it still requests its share of the tiles they need.
+  auto iteration = [&](auto has_next_tag, auto tail_loads_tag) {
     constexpr bool HN = decltype(has_next_tag)::value;
+    constexpr bool TL = decltype(tail_loads_tag)::value;
     const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
     const ae_lds_byte* vt = lds + 2 * AE_K_BYTES + (n & 1) * AE_V_BYTES;
-    const int j2 = HN ? next_tile(j1 + 1) : j_end;
+    const int j2 = (HN || TL) ? next_tile(j1 + 1) : j_end;
     // Nothing is in flight here on the back edge (the iteration ends with vmcnt(0)); saying so
     // also clears loads still pending on loop ENTRY (Q fragments, spill reloads), which the
     // compiler's wait-count insertion would otherwise wait for after this iteration's tile loads
@@ -573,6 +587,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
         }
       }
     } else {
+      if (TL) {
+        load_k(j2l, n & 1);
+        load_v(j1, (n + 1) & 1);
+      }
       exp_all();
     }
     if (HN) mx[0] = mx[1] = AE_NEG_INF;
@@ -626,17 +644,50 @@ void ae_prefill_kernel(const ae_attn_params p) {
         for (int r = 0; r < 16; r++) oacc[qb][db][r] *= osc[qb];
     rescale = false;
   };
+#if AE_MASK_MODE == 1
+  // an iteration of a wave that is done with its own tiles: its share of the tile loads, and the barrier
+  auto drain = [&]() {
+    const int j2 = next_tile(j1 + 1);
+    const int j2l = j2 < j_end ? j2 : j_end - 1;
+    load_k(j2l, n & 1);
+    load_v(j1, (n + 1) & 1);
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);   // vmcnt(0)
+    __syncthreads();
+    j0 = j1;
+    j1 = j2;
+    n++;
+  };
   if (any_tile) {
     while (true) {
-      while (j1 < j_end && !rescale) iteration(ae_tag_true{});
+      while (j1 < j_end_w && !rescale) iteration(ae_tag_true{}, ae_tag_false{});
       if (rescale) {
         rescale_o();
         continue;
       }
       break;
     }
-    iteration(ae_tag_false{});
+    if (j1 < j_end) {              // the other waves go on: last product of this wave, then only loads
+      iteration(ae_tag_false{}, ae_tag_true{});
+      while (j1 < j_end) drain();
+      __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);
+      __syncthreads();             // the barrier of the other waves' last iteration
+    } else {
+      iteration(ae_tag_false{}, ae_tag_false{});
+    }
   }
+#else
+  if (any_tile) {
+    while (true) {
+      while (j1 < j_end && !rescale) iteration(ae_tag_true{}, ae_tag_false{});
+      if (rescale) {
+        rescale_o();
+        continue;
+      }
+      break;
+    }
+    iteration(ae_tag_false{}, ae_tag_false{});
+  }
+#endif
 
   // ---- epilogue -------------------------------------------------------------------------------
 #pragma unroll
