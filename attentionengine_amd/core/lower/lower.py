@@ -51,6 +51,10 @@ class LoweredFunctors:
     # (scale, max field, sum field) when the graph is the online softmax of `scores * scale`,
     # scale > 0: the case the software-pipelined prefill kernel is written for
     softmax: tuple = None
+    # out = sum_kv f(s) v: no row state, no reduction over the kv tile, no use of the kv index, o_scale = 1,
+    # no final row scales (sigmoid / relu attention) - ae_online_fwd<N> may then be called on any subset
+    # of a tile's scores, which is how the software-pipelined prefill kernel calls it
+    elementwise: bool = False
 
 
 def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
@@ -230,6 +234,22 @@ def _pure_scale(sym, scores):
     return c
 
 
+def _no_tile_reduction(node) -> bool:
+    """True when no node of the graph reduces over the kv-tile axis (a value without the ``block_N``
+    dimension computed from one that has it)."""
+    seen, stack = set(), [node]
+    while stack:
+        n = stack.pop()
+        if id(n) in seen or not isinstance(n, SymbolScalar):
+            continue
+        seen.add(id(n))
+        prev = [q for q in (n.prev or []) if isinstance(q, SymbolScalar)]
+        if "block_N" not in n.shape_idx and any("block_N" in q.shape_idx for q in prev):
+            return False
+        stack.extend(prev)
+    return True
+
+
 def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO, in_dtype,
                    mask_value: str = "-inf") -> LoweredFunctors:
     """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
@@ -306,6 +326,8 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
         if expr != f"st.{k}":
             body.append(f"  st.{k} = {expr};")
     online_fwd_body = "\n".join(body)
+    elementwise = (not rowscales and not new_rowscales and o_scale_one and id(kv_idx) not in em.done
+                   and not any(sid in em.done for sid in cust_preambles) and _no_tile_reduction(new_scores))
     score_mod_body = "  // score_mod is fused into ae_online_fwd"
 
     # ---- epilogue -------------------------------------------------------------------------
@@ -338,6 +360,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     lf.custom_fields = cust_fields
     lf.custom_loads = cust_loads
     lf.softmax = softmax
+    lf.elementwise = bool(elementwise and not fvals)
     return lf
 
 
@@ -408,10 +431,12 @@ class PrefillTiles:
 _MI355X_CUS = 256
 
 
-def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0) -> PrefillTiles:
+def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0,
+                         elementwise: bool = False) -> PrefillTiles:
     """The direct-to-LDS kernels handle 128- and 256-byte K/V rows (head dims 64 and 128): the
     software-pipelined one (64 rows per wave, 256-row q tiles, one wave per SIMD) when the graph is
-    the online softmax of scaled scores and the problem has enough q tiles to occupy the chip
+    the online softmax of scaled scores, or elementwise (out = sum f(s) v: the kernel then calls the
+    generated functor), and the problem has enough q tiles to occupy the chip
     (measured on B2 H32 S4096 D128 fp16: 1.0 against 0.86 PFLOP/s non-causal), otherwise the generic
     one (32 rows per wave, two waves per SIMD, runs any functor).  Other head dims use the
     register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one wave per SIMD and a
@@ -420,7 +445,8 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
     if d in (64, 128) and dv in (64, 128):
         force = os.environ.get("AE_PREFILL_KERNEL", "")
         n_tiles = batch_heads * ((seqlen_q + 255) // 256)
-        if softmax is not None and force != "generic" and (force == "pipelined" or n_tiles >= (3 * _MI355X_CUS) // 4):
+        if (softmax is not None or elementwise) and force != "generic" and (
+                force == "pipelined" or n_tiles >= (3 * _MI355X_CUS) // 4):
             return PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)
         return PrefillTiles()
     t = PrefillTiles(template="ae_prefill_simple.hip", k_pad=16)
@@ -443,9 +469,13 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
 
 
 def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, has_mask_mod: bool,
-                  n_rowscales: int, o_scale_one: bool, even_q: bool, even_kv: bool, softmax=None) -> str:
-    """Text of ae_config.h."""
+                  n_rowscales: int, o_scale_one: bool, even_q: bool, even_kv: bool, softmax=None,
+                  elementwise: bool = False) -> str:
+    """Text of ae_config.h.  ``softmax`` / ``elementwise`` say what the software-pipelined kernel does with a
+    score (AE_PIPE_KIND 0: its built-in online softmax; 1: the generated functor); other kernels ignore them."""
     extra = []
+    if softmax is None and elementwise:
+        extra = ["#define AE_PIPE_KIND 1"]
     if softmax is not None:
         extra = [f"#define AE_SM_SCALE {float_literal(softmax[0])}", f"#define AE_SM_M {softmax[1]}",
                  f"#define AE_SM_R {softmax[2]}"]

@@ -48,9 +48,15 @@ class PrefillOp:
                                          self.dtype, mask_value)
         self._graph = (score_mod, online_func, custom_fwd_inputs)     # the backward traces score_mod again
         self.functor_src = L.render_functors(self.functors)
+        # what the software-pipelined kernel can run: the proven online softmax, or an elementwise graph
+        # (masked scores are -inf before score_mod there, as in the reference: not with mask_value "0")
+        self._pipe_softmax = None if self.mask_value_zero else self.functors.softmax
+        self._pipe_elementwise = (self._pipe_softmax is None and self.functors.elementwise
+                                  and not self.mask_value_zero)
         self.tiles = L.choose_prefill_tiles(self.D, self.DV_launch, _dim(q_meta.shape[2], 0),
-                                            None if self.mask_value_zero else self.functors.softmax,
-                                            _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1))
+                                            self._pipe_softmax,
+                                            _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1),
+                                            elementwise=self._pipe_elementwise)
         # Split-KV ("MHA decode": a few query tokens against a long KV, attn_engine.py:273-290 and
         # core/lower/lower_decode.py:287-313 of the reference): the kv axis is shared out over several
         # workgroups per q tile and the partial results are merged with the user's combine().
@@ -155,7 +161,8 @@ class PrefillOp:
             has_mask_mod = self.elementwise_mask and mask_mode != 1
             cfg_src = L.render_config(self.D, self.DV_launch, self.dtype, self.tiles, mask_mode, has_mask_mod,
                                       self.n_rowscales, self.functors.o_scale_one, even_q, even_kv,
-                                      self.functors.softmax if self.tiles.rows_per_wave == 64 else None)
+                                      self._pipe_softmax if self.tiles.rows_per_wave == 64 else None,
+                                      elementwise=self._pipe_elementwise and self.tiles.rows_per_wave == 64)
             if self.mask_value_zero:
                 cfg_src += "#define AE_MASK_VALUE_ZERO 1\n"
             if n_split > 1:

@@ -1,11 +1,12 @@
-// Software-pipelined flash attention forward (prefill) for gfx950 / CDNA4: online softmax only.
+// Software-pipelined flash attention forward (prefill) for gfx950 / CDNA4: the online softmax, or (AE_PIPE_KIND 1)
+// any elementwise graph out = sum_kv f(s) v through its generated functor.
 //
 // Same role and operation order as ae_prefill.hip (the reference's TileLang prefill template,
 // attention_engine/core/template/tl_template/attn/attn_tl.py:76-174, and its block-sparse sibling
 // blockattn_tl.py:49-160), specialised for the case the lowering has PROVEN to be the online
 // softmax of attn_script/mha.py:47-72 applied to `score * constant`:
 //     m' = max(m, rowmax(s*c)), p = exp(s*c - m'), r' = r*exp(m - m') + rowsum(p), O' = O*exp(m - m') + pV
-// Any other score_mod / OnlineFunc graph uses ae_prefill.hip, which runs the generated functors.
+// Graphs with other row state use ae_prefill.hip, which runs the generated functors on whole tiles.
 //
 // Why a second kernel: with 32 query rows per wave every 32x32x16 MFMA needs a fresh 1 KiB A
 // fragment (K or V^T) from LDS, and four SIMDs issuing MFMAs back to back then ask LDS for exactly
@@ -81,9 +82,16 @@
 #ifndef AE_TOP_PREFETCH
 #define AE_TOP_PREFETCH (AE_MASK_MODE == 0)
 #endif
+// What turns a score into p.  0: the online softmax described above.  1: the generated functor
+// ae_online_fwd itself, two scores at a time, for graphs the lowering has shown to be ELEMENTWISE
+// (out = sum_kv f(s) v, attn_script/sigmoidattn.py, reluattn.py: no row state, no row reduction, no use of
+// the kv index, o_scale = 1): the same pipeline without maxima, sums and the lazy reference.
+#ifndef AE_PIPE_KIND
+#define AE_PIPE_KIND 0
+#endif
 // 1: Q carries c*log2e and the reference is the C operand of the first k-step (see above)
 #ifndef AE_PRESCALE
-#define AE_PRESCALE (!AE_DTYPE_BF16)
+#define AE_PRESCALE (!AE_DTYPE_BF16 && AE_PIPE_KIND == 0)
 #endif
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
@@ -363,7 +371,9 @@ void ae_prefill_kernel(const ae_attn_params p) {
       // allocator keeps the value in the accumulator file and re-reads it at the top of the loop
       asm volatile("" : "+v"(x));
       sv[qb][e] = x;
+#if AE_PIPE_KIND == 0
       mx[qb] = __builtin_fmaxf(mx[qb], x);
+#endif
     }
   };
   // p = exp2(x), two scores at a time ("unit" u: q block u%2, k-step u/8, pair (u/2)%4 of that k-step's 8
@@ -372,11 +382,12 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // sum.  Unit u starts in slot (u * AE_EXP_SPAN) / 32; units are ordered by k-step, the order
   // O^T += V^T P^T needs them.
   float rsum[2];
+  int kv_lim = 0;       // elementwise kind, ragged kv: keys of the tile in sv at offsets >= kv_lim (lane-relative) are past the end
   float xa[32][2];
   float negm2[2] = {0.f, 0.f};
   auto stage_a = [&](int u) {
     const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
-#if AE_PRESCALE
+#if AE_PRESCALE || AE_PIPE_KIND == 1
     xa[u][0] = sv[qb][e];
     xa[u][1] = sv[qb][e + 1];
 #else
@@ -385,8 +396,13 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #endif
   };
   auto stage_b = [&](int u) {
+#if AE_PIPE_KIND == 1
+    // (score_mod is fused into ae_online_fwd; the graph has neither row state nor an o_scale)
+    ae_online_fwd<2>(xa[u], st[u & 1], ctx[u & 1], cust[u & 1]);
+#else
     xa[u][0] = ae_exp2(xa[u][0]);
     xa[u][1] = ae_exp2(xa[u][1]);
+#endif
   };
   auto stage_c = [&](int u) {
     const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
@@ -394,7 +410,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
     const ae_f32x2 x2 = {xa[u][0], xa[u][1]};
     const ae_elem2 hv = __builtin_convertvector(x2, ae_elem2);   // one packed conversion, round to nearest
     pf[qb][e >> 3][(e & 7) >> 1] = __builtin_bit_cast(unsigned, hv);
-#if AE_DTYPE_BF16
+#if AE_PIPE_KIND == 1
+    (void)rsum;
+#if !AE_EVEN_KV
+    // keys past the end: f(-inf) need not be zero
+    if (ae_kv_off(e) >= kv_lim) pf[qb][e >> 3][(e & 7) >> 1] = 0u;
+    else if (ae_kv_off(e + 1) >= kv_lim) pf[qb][e >> 3][(e & 7) >> 1] &= 0xffffu;
+#endif
+#elif AE_DTYPE_BF16
     // bf16 keeps 8 significant bits: summing the rounded values would put ~1e-3 into lse for rows
     // with few visible keys, so the fp32 values are summed (fp16 sums the rounded pairs in one v_dot2)
     rsum[qb] += xa[u][0] + xa[u][1];
@@ -459,6 +482,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
         }
       }
     }
+#if AE_PIPE_KIND == 0
     float tmax[2];
     bool any_need = false;
 #pragma unroll
@@ -492,6 +516,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #endif
       }
     }
+#endif  // AE_PIPE_KIND == 0
   };
 
   // ---- prologue: first tile's scores ------------------------------------------------------------
@@ -570,6 +595,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     // (with AE_TOP_PREFETCH the first AE_AHEAD fragments are already on their way: prefetch_ring at the
     // end of the previous iteration, or of the prologue)
     rsum[0] = rsum[1] = 0.f;
+    kv_lim = p.seqlen_kv - j0 * AE_BN - 4 * hf;
     AE_SB();
 
     // ---- phase 1: x(j1)^T = K Q^T - m2  ||  p(j0) ------------------------------------------------
@@ -700,6 +726,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
     frs[0] = 0.f;
     if (any_tile) {
+#if AE_PIPE_KIND == 0
       st[qb].AE_SM_M = m2[qb] * AE_LN2;
       st[qb].AE_SM_R = ae_group_sum(r_run[qb]);
       ae_epilogue<AE_NO>(o, st[qb], frs, ctx[qb], cust[qb]);
@@ -708,6 +735,9 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
         for (int e = 0; e < AE_NO; e++) o[e] = 0.f;
       }
+#else
+      ae_epilogue<AE_NO>(o, st[qb], frs, ctx[qb], cust[qb]);
+#endif
     } else {
 #pragma unroll
       for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;

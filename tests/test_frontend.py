@@ -427,3 +427,38 @@ def test_symbol_backward_leaves_gradient_expressions_on_the_leaves():
     env = {id(x): xv.detach(), id(y): yv.detach(), id(g): gv}
     assert torch.allclose(evaluate(x.grad, env), gx, atol=1e-12)
     assert torch.allclose(evaluate(y.grad, env), gy, atol=1e-12)
+
+
+def test_elementwise_graphs_are_recognised():
+    """out = sum_kv f(s) v (no row state, no reduction over the tile, no kv index): the functor may be applied
+    to any subset of a tile, which is what lets the software-pipelined kernel call it pairwise."""
+    import attn_script as C
+    from core.lower import lower as L
+    f16 = torch.float16
+    sig = L.trace_functors(C.make_sigmoid_score_mod(0.125), None, C.OnlineIdentity(),
+                           CustomIO({"softmax_bias": (1,)}), f16)
+    relu = L.trace_functors(C.make_relu_score_mod(0.125), C.causal_mask, C.OnlineIdentity(), CustomIO({}), f16)
+    soft = L.trace_functors(C.make_scale_score_mod(0.125), None, C.OnlineSoftmax(), CustomIO({}), f16)
+    assert sig.elementwise and relu.elementwise and not soft.elementwise
+    assert sig.softmax is None and soft.softmax is not None
+
+    def uses_kv(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+        return score * 0.125 + kv_idx
+    assert not L.trace_functors(uses_kv, None, C.OnlineIdentity(), CustomIO({}), f16).elementwise
+
+    class TileNormalised(C.OnlineIdentity):      # no row state, but a reduction over the tile
+        @staticmethod
+        def online_fwd(scores, online_rowscales, b, h, q_idx):
+            return scores / scores.get_reduce("abssum"), online_rowscales, C.OnlineIdentity.online_fwd(
+                scores, online_rowscales, b, h, q_idx)[2]
+    try:
+        lf = L.trace_functors(C.make_scale_score_mod(0.125), None, TileNormalised(), CustomIO({}), f16)
+    except Exception:
+        lf = None
+    assert lf is None or not lf.elementwise
+    # tile choice: a chip-filling elementwise problem takes the pipelined kernel, a small one the generic one
+    big = L.choose_prefill_tiles(128, 128, seqlen_q=4096, softmax=None, batch_heads=64, elementwise=True)
+    small = L.choose_prefill_tiles(128, 128, seqlen_q=512, softmax=None, batch_heads=4, elementwise=True)
+    assert big.template == "ae_prefill_pipe.hip" and small.template == "ae_prefill.hip"
+    cfg = L.render_config(128, 128, f16, big, 0, False, 0, True, True, True, None, elementwise=True)
+    assert "#define AE_PIPE_KIND 1" in cfg

@@ -142,6 +142,48 @@ def test_sigmoid_prefill(cuda_device, B, H, S, D, causal):
     assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
 
 
+@pytest.mark.parametrize("kind,dtype,B,H,Sq,Skv,D,mask", [
+    ("sigmoid", torch.float16, 1, 2, 512, 512, 128, None),
+    ("sigmoid", torch.bfloat16, 2, 2, 300, 427, 64, "causal"),     # ragged q rows and keys, causal tile skip
+    ("relu", torch.float16, 1, 3, 256, 333, 128, "window"),       # ragged keys, tile-class table + mask_mod
+    ("square", torch.float16, 1, 2, 200, 150, 64, None),          # f(-inf) = +inf: keys past the end must give 0
+])
+def test_pipelined_kernel_runs_elementwise_functors(cuda_device, monkeypatch, kind, dtype, B, H, Sq, Skv, D, mask):
+    """Graphs of the form out = sum_kv f(s) v (no row state: sigmoid / relu attention) run in the
+    software-pipelined kernel through their generated functor, two scores at a time (forced here on small
+    shapes; chosen by itself on chip-filling ones).  Checked against the generic kernel's oracle."""
+    print(f"case pipelined elementwise {kind} {dtype} B{B} H{H} Sq{Sq} Skv{Skv} D{D} {mask}", flush=True)
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    scale = 1 / math.sqrt(D)
+    q, k, v = C.make_inputs(B, Sq, Skv, H, H, D, D, dtype)
+    mask_mod = {None: None, "causal": C.causal_mask, "window": C.make_sliding_window_mask(64)}[mask]
+    customs, extra = CustomIO({}), ()
+    if kind == "sigmoid":
+        bias = torch.tensor([-math.log(Skv)], dtype=torch.float32)
+        customs, extra = CustomIO({"softmax_bias": (1,)}), (bias.cuda(),)
+        score_mod = C.make_sigmoid_score_mod(scale)
+    elif kind == "relu":
+        score_mod = C.make_relu_score_mod(scale)
+    else:
+        def score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+            return (score * scale) * (score * scale)
+    meta = (meta_tensor(B, H, Sq, D, dtype=dtype), meta_tensor(B, H, Skv, D, dtype=dtype),
+            meta_tensor(B, H, Skv, D, dtype=dtype))
+    mod = AttentionEngine(meta, customs, score_mod=score_mod, mask_mod=mask_mod, online_func=C.OnlineIdentity())
+    assert mod.attention.tiles.template == "ae_prefill_pipe.hip" and mod.attention.functors.elementwise
+    out = mod(q.cuda(), k.cuda(), v.cuda(), *extra)
+    qf, kf, vf = (t.float().permute(0, 2, 1, 3) for t in (q, k, v))
+    s = qf @ kf.transpose(-1, -2) * scale
+    if mask_mod is not None:
+        qi, ki = torch.arange(Sq)[:, None], torch.arange(Skv)[None, :]
+        s = s.masked_fill(~mask_mod(0, 0, qi, ki), float("-inf"))
+    p = {"sigmoid": lambda x: torch.sigmoid(x - math.log(Skv)), "relu": torch.relu, "square": lambda x: x * x}[kind](s)
+    p = torch.where(torch.isinf(s), torch.zeros_like(p), p) if kind != "square" else p
+    ref = (p @ vf).permute(0, 2, 1, 3)
+    assert torch.isfinite(out).all()
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL * max(1.0, ref.abs().max().item())
+
+
 def test_relu_prefill(cuda_device):
     B, H, S, D = 2, 3, 256, 64
     dtype = torch.float16
