@@ -65,6 +65,7 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
     ``seq_len_kv`` dimension is read per element from global memory in the input dtype
     (lower.py:590-597)."""
     leaves, descs, loads, fields, preambles = {}, [], [], [], {}
+    prefetch = []      # body lines of ae_prefetch_custom (per-kv inputs, kernels that fetch a tile ahead)
     for slot, (name, sym) in enumerate(custom_fwd_inputs.input_tensors.items()):
         slot += slot_offset
         dims = list(sym.shape_idx)
@@ -93,14 +94,39 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
             # one element per score (e.g. the retention decay mask, attn_script/retention.py:14-16):
             # the row's base pointer is kept per lane, elements are read in the input dtype where the
             # scores are modified; kv positions past the end of a ragged tile read the last element
-            fields += [f"const ae_elem* {name}_row;", f"int64_t {name}_kvstride;", f"int {name}_kvlast;"]
+            fields += [f"const ae_elem* {name}_row;", f"int64_t {name}_kvstride;", f"int {name}_kvlast;",
+                       "#if AE_KV_PF_GROUPS > 0",
+                       f"ae_elem4 {name}_pf[AE_KV_PF_GROUPS];   // the lane's elements of the tile fetched ahead",
+                       "#endif"]
             loads += [f"c.{name}_row = (const ae_elem*)p.custom[{slot}] + ({index});",
                       f"c.{name}_kvstride = {kv_stride};", f"c.{name}_kvlast = p.seqlen_kv - 1;"]
             leaves[id(sym)] = (f"cm_{name}", True)
             # a lane's elements come in groups of four consecutive kv positions (ae_kv_off): one 8-byte
             # load per group where the tensor allows it (unit kv stride, aligned, inside the row)
+            # A kernel that defines AE_KV_PF_GROUPS (a lane's groups per tile) calls ae_prefetch_custom for
+            # the NEXT tile once the functors have used the current one: the loads then have a whole tile
+            # of MFMAs to arrive, instead of stalling the functor that issues them.
+            group_load = [
+                "    const int kv = kv_base + ae_kv_off(4 * g);",
+                f"    const ae_elem* src = cust.{name}_row + (int64_t)kv * cust.{name}_kvstride;",
+                f"    if (cust.{name}_kvstride == 1 && kv + 3 <= cust.{name}_kvlast && ((unsigned long)src & 7) == 0) {{",
+                f"      cust.{name}_pf[g] = *(const ae_elem4*)src;",
+                "    } else {",
+                "#pragma unroll",
+                "      for (int i = 0; i < 4; i++) {",
+                f"        const int kvi = kv + i < cust.{name}_kvlast ? kv + i : cust.{name}_kvlast;",
+                f"        cust.{name}_pf[g][i] = cust.{name}_row[(int64_t)kvi * cust.{name}_kvstride];",
+                "      }",
+                "    }"]
+            prefetch += ["#pragma unroll", "  for (int g = 0; g < AE_KV_PF_GROUPS; g++) {", *group_load, "  }"]
             preambles[id(sym)] = [
-                f"  float cm_{name}[N];", "#pragma unroll",
+                f"  float cm_{name}[N];",
+                "#if AE_KV_PF_GROUPS > 0",
+                '  static_assert(N == 4 * AE_KV_PF_GROUPS, "the kernel fetches a whole tile of a lane\'s elements ahead");',
+                "#pragma unroll",
+                f"  for (int e = 0; e < N; e++) cm_{name}[e] = (float)cust.{name}_pf[e >> 2][e & 3];",
+                "#else",
+                "#pragma unroll",
                 "  for (int g = 0; g < N / 4; g++) {",
                 "    const int kv = ctx.kv_base + ae_kv_off(4 * g);",
                 f"    const ae_elem* src = cust.{name}_row + (int64_t)kv * cust.{name}_kvstride;",
@@ -115,7 +141,8 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
                 f"        cm_{name}[4 * g + i] = (float)cust.{name}_row[(int64_t)kvi * cust.{name}_kvstride];",
                 "      }",
                 "    }",
-                "  }"]
+                "  }",
+                "#endif"]
             descs.append(CustomInput(name, dims, per_kv, in_dtype))
             continue
         fields.append(f"float {name};")
@@ -123,6 +150,7 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
         leaves[id(sym)] = (f"cust.{name}", False)
         tdtype = torch.float32
         descs.append(CustomInput(name, dims, per_kv, tdtype))
+    preambles["prefetch"] = prefetch
     return leaves, descs, loads, fields, preambles
 
 
@@ -255,6 +283,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
     custom_fwd_inputs = custom_fwd_inputs if custom_fwd_inputs is not None else CustomIO()
     cust_leaves, customs, cust_loads, cust_fields, cust_preambles = _custom_leaves(custom_fwd_inputs, in_dtype)
+    cust_prefetch = cust_preambles.pop("prefetch")
 
     def index_leaves():
         b = SymbolScalar("b", Var("b"), shape_idx=[])
@@ -359,6 +388,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
                          [k for k, _ in fvals], o_scale_one, customs, lowered_mask)
     lf.custom_fields = cust_fields
     lf.custom_loads = cust_loads
+    lf.custom_prefetch = cust_prefetch
     lf.softmax = softmax
     lf.elementwise = bool(elementwise and not fvals)
     return lf
@@ -372,15 +402,30 @@ def render_functors(lf: LoweredFunctors) -> str:
     cfields = "\n".join("  " + f for f in lf.custom_fields) or "  int ae_unused;"
     cloads = "\n".join("  " + ld for ld in lf.custom_loads) or "  c.ae_unused = 0;"
     mask_body = lf.mask.body if lf.mask is not None else "  return true;"
+    prefetch = ""
+    if getattr(lf, "custom_prefetch", None):
+        body = "\n".join(lf.custom_prefetch)
+        prefetch = f"""#if AE_KV_PF_GROUPS > 0
+// custom inputs with a kv dimension: the lane's elements of the tile whose first kv position (for this lane)
+// is kv_base, fetched into cust for the functors' next call
+#define AE_HAS_KV_PREFETCH 1
+AE_DEV void ae_prefetch_custom(ae_custom& cust, int kv_base) {{
+{body}
+}}
+#endif
+"""
     return f"""// generated by core/lower/lower.py -- do not edit
 {MASK_HELPERS}
+#ifndef AE_KV_PF_GROUPS
+#define AE_KV_PF_GROUPS 0      // kernels that fetch per-score custom inputs a tile ahead define it before this header
+#endif
 struct ae_custom {{
 {cfields}
 }};
 AE_DEV void ae_load_custom(ae_custom& c, const ae_attn_params& p, const ae_ctx& ctx) {{
 {cloads}
 }}
-struct ae_rowstate {{
+{prefetch}struct ae_rowstate {{
 {fields}
 }};
 AE_DEV void ae_rowstate_init(ae_rowstate& st) {{

@@ -38,6 +38,9 @@
 #define AE_NSPLIT 1                // > 1: split-KV, fp32 partial results + the merge kernel of ae_combine.h
 #endif
 #include "ae_device.h"
+// custom inputs with a kv dimension (one element per score) are fetched a tile ahead: a lane's groups of four
+// consecutive kv positions per tile
+#define AE_KV_PF_GROUPS (AE_BN / 8)
 #include "ae_functors.h"  // generated: the functor bodies
 
 // value given to score positions past seqlen_kv before the user functors run: -inf, or 0 for graphs
@@ -281,6 +284,12 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #endif
   bool any_tile = j < j_end;
   if (any_tile) load_tile(j, 0);
+#ifdef AE_HAS_KV_PREFETCH
+  if (any_tile) {
+#pragma unroll
+    for (int rb = 0; rb < AE_RB; rb++) ae_prefetch_custom(cust[rb], j * AE_BN + 4 * hf);
+  }
+#endif
   // Drain every outstanding load (Q fragments, first tile) before the loop: with loads still
   // pending at the loop header the compiler's wait-count insertion makes the QK^T MFMAs of every
   // iteration wait for that iteration's K/V prefetch, which serialises the pipeline.
@@ -352,6 +361,11 @@ void ae_prefill_kernel(const ae_attn_params p) {
       // ---- user functors ----------------------------------------------------------------------
       ae_score_mod<AE_NS>(s, ctx[rb], cust[rb]);
       float o_scale = ae_online_fwd<AE_NS>(s, st[rb], ctx[rb], cust[rb]);
+#ifdef AE_HAS_KV_PREFETCH
+      // the functors are done with this tile's elements of the per-score custom inputs: request the next
+      // tile's, which travel while the second product runs
+      if (jn < j_end) ae_prefetch_custom(cust[rb], jn * AE_BN + 4 * hf);
+#endif
 
 #if !AE_EVEN_KV
       if (kv0 + AE_BN > p.seqlen_kv) {

@@ -39,6 +39,9 @@
 #include "ae_hip.h"
 #include "ae_config.h"    // generated: the AE_* configuration macros
 #include "ae_device.h"
+// custom inputs with a kv dimension (one element per score) are fetched a tile ahead: a lane's groups of four
+// consecutive kv positions per tile
+#define AE_KV_PF_GROUPS (AE_BN / 8)
 #include "ae_functors.h"  // generated: the functor bodies
 
 // value given to score positions past seqlen_kv before the user functors run: -inf, or 0 for graphs
@@ -251,6 +254,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
   if (any_tile) {
     load_tile(j);
     store_tile(0);
+#ifdef AE_HAS_KV_PREFETCH
+#pragma unroll
+    for (int rb = 0; rb < AE_RB; rb++) ae_prefetch_custom(cust[rb], j * AE_BN + 4 * hf);
+#endif
   }
   // Drain every outstanding load (Q fragments, first tile) before the loop: with loads still
   // pending at the loop header the compiler's wait-count insertion makes the QK^T MFMAs of every
@@ -323,6 +330,11 @@ void ae_prefill_kernel(const ae_attn_params p) {
       // ---- user functors ----------------------------------------------------------------------
       ae_score_mod<AE_NS>(s, ctx[rb], cust[rb]);
       float o_scale = ae_online_fwd<AE_NS>(s, st[rb], ctx[rb], cust[rb]);
+#ifdef AE_HAS_KV_PREFETCH
+      // the functors are done with this tile's elements of the per-score custom inputs: request the next
+      // tile's, which travel while the second product runs
+      if (jn < j_end) ae_prefetch_custom(cust[rb], jn * AE_BN + 4 * hf);
+#endif
 
 #if !AE_EVEN_KV
       if (kv0 + AE_BN > p.seqlen_kv) {
