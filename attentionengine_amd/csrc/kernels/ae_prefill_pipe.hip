@@ -667,7 +667,15 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) oacc[qb][db][r] *= osc[qb];
+        for (int r = 0; r < 16; r++) {
+          // one accumulator register at a time through one scratch register: written as plain arithmetic,
+          // the register allocator makes room for all of O in ordinary registers and pays for it with
+          // ~70 registers stored to and reloaded from scratch memory in every workgroup's prologue
+          float o = oacc[qb][db][r], t;
+          asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                       : "+a"(o), "=&v"(t) : "v"(osc[qb]));
+          oacc[qb][db][r] = o;
+        }
     rescale = false;
   };
 #if AE_MASK_MODE == 1
