@@ -170,9 +170,11 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // Q has landed
     __syncthreads();                           // tile 0 has landed
 
-    // K fragment of k-step ks: row lane%32, global chunk 2*ks + lane/32
-    const int k_row_off = l32s * AE_KSTR;
-    const int k_sw = AE_SWZ(l32s);
+    // K fragment of k-step ks: row lane%32, global chunk 2*ks + lane/32.  The swizzle touches the three low
+    // bits of the chunk number only, so a lane has four distinct offsets (ks % 4) and the rest is an immediate.
+    int k_base[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) k_base[i] = l32s * AE_KSTR + (((2 * i + hfs) ^ AE_SWZ(l32s)) << 4);
     // A trip multiplies tile n by Q^T and, in the issue slots between those MFMAs, runs the softmax of tile
     // n - 1 (its raw scores wait in `xs`): the wave's matrix work and its softmax overlap instead of
     // following each other.  P of tile n - 1 is handed over by the barrier that ends trip n.
@@ -180,14 +182,13 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
 #pragma unroll
     for (int r = 0; r < 16; r++) xs[r] = 0.f;
     // lane owns head lane%32 and kv rows 8*(e/4) + 4*(lane/32) + e%4 of a tile
-    float x[16], mx, mn, osc, rs;
+    float mx, mn, osc, rs;
     bool need;
     ae_lds_byte* prow;
     ae_lds_byte* xb;
     // start of the softmax of tile tp: scores beyond the end of the range are taken out (ragged tail only)
     auto soft_begin = [&](int tp) {
-#pragma unroll
-      for (int e = 0; e < 16; e++) x[e] = xs[e];   // raw scores: the scale is folded into the exponent
+      // (xs holds raw scores: the scale is folded into the exponent; the softmax works on it in place)
       const bool tail = kv_begin + tp * AE_BN + AE_BN > kv_end;
       if (__builtin_expect(tail, 0)) {
         // the empty asm keeps this a branch: flattened into selects it costs 5 instructions per score
@@ -195,7 +196,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         asm volatile("" ::: "memory");
         const int kvb = kv_begin + tp * AE_BN + 4 * hfs;
 #pragma unroll
-        for (int e = 0; e < 16; e++) x[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? x[e] : AE_NEG_INF;
+        for (int e = 0; e < 16; e++) xs[e] = (kvb + 8 * (e >> 2) + (e & 3) < kv_end) ? xs[e] : AE_NEG_INF;
       }
       mx = AE_NEG_INF;
       rs = 0.f;
@@ -205,8 +206,8 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     // the softmax of one tile in AE_NKS pieces, piece f issued behind the MFMA of k-step f
     auto soft_slot = [&](int f) {
       if (f < 4) {
-        mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[4 * f]), x[4 * f + 1]);
-        mx = __builtin_fmaxf(__builtin_fmaxf(mx, x[4 * f + 2]), x[4 * f + 3]);
+        mx = __builtin_fmaxf(__builtin_fmaxf(mx, xs[4 * f]), xs[4 * f + 1]);
+        mx = __builtin_fmaxf(__builtin_fmaxf(mx, xs[4 * f + 2]), xs[4 * f + 3]);
       } else if (f == 4) {
         float hi;
         const float lo = ae_swap32_lo_hi(mx, hi);
@@ -218,13 +219,13 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         m2 = mn;
       } else if (f < 22) {
         const int e = f - 6;
-        x[e] = ae_exp2(__builtin_fmaf(x[e], AE_SM_SCALE * AE_LOG2E, -mn));
-        rs += x[e];
+        xs[e] = ae_exp2(__builtin_fmaf(xs[e], AE_SM_SCALE * AE_LOG2E, -mn));
+        rs += xs[e];
       } else if (f < 26) {
         const int rb = f - 22;
         ae_elem4 w;
 #pragma unroll
-        for (int i = 0; i < 4; i++) w[i] = (ae_elem)x[4 * rb + i];
+        for (int i = 0; i < 4; i++) w[i] = (ae_elem)xs[4 * rb + i];
         *(__attribute__((address_space(3))) ae_elem4*)(prow + 16 * rb) = w;
       } else if (f == 26) {
         r_run = r_run * osc + rs;
@@ -237,11 +238,13 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     // S^T of tile tn into xs; with SOFT the softmax of tile tn - 1 rides along
     auto score_trip = [&](int tn, auto with_soft) {
       constexpr bool SOFT = decltype(with_soft)::value;
-      const ae_lds_byte* kt = lds + (tn % AE_NSTAGE) * AE_STAGE_BYTES + k_row_off;
+      int ka[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) ka[i] = k_base[i] + (tn % AE_NSTAGE) * AE_STAGE_BYTES;
       // read AE_AHEAD fragments before the MFMA that uses them (the compiler on its own keeps one read
       // in flight, which leaves the LDS latency exposed)
       auto read_kfrag = [&](int ks) -> ae_elem8 {
-        return *(const __attribute__((address_space(3))) ae_elem8*)(kt + (((2 * ks + hfs) ^ k_sw) << 4));
+        return *(const __attribute__((address_space(3))) ae_elem8*)(lds + ka[ks & 3] + (ks >> 2) * 128);
       };
       ae_elem8 ring[AE_RING];
 #pragma unroll
