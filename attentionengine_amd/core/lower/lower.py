@@ -278,6 +278,41 @@ def _no_tile_reduction(node) -> bool:
     return True
 
 
+def _depends_on(node, target) -> bool:
+    seen, stack = set(), [node]
+    while stack:
+        n = stack.pop()
+        if n is target:
+            return True
+        if id(n) in seen or not isinstance(n, SymbolScalar):
+            continue
+        seen.add(id(n))
+        stack.extend(n.prev or [])
+    return False
+
+
+def find_deferred_norm(rowscales, new_scores, new_rowscales, o_scale):
+    """Online functions that renormalise on every tile: ``scores' = X / r_new`` and
+    ``o_scale = r_old / r_new`` with r a row scale and X free of it (retention's running sum of |s|,
+    attn_script/retention.py:40-60).  The factors telescope: the output equals (sum over tiles of X v) / r_final,
+    so the kernels may accumulate X v unscaled - no rescale of the whole accumulator per tile - and divide
+    once in the epilogue.  Returns (name of r, X) or None."""
+    if not (isinstance(new_scores, SymbolScalar) and isinstance(o_scale, SymbolScalar)):
+        return None
+    if new_scores.code.type != "Div" or o_scale.code.type != "Div":
+        return None
+    x, r_new = new_scores.prev
+    r_old, r_new2 = o_scale.prev
+    if r_new is not r_new2:
+        return None
+    names = [k for k, v in new_rowscales.items() if v is r_new]
+    if len(names) != 1 or rowscales.get(names[0]) is not r_old:
+        return None
+    if _depends_on(x, r_new) or _depends_on(x, r_old):
+        return None
+    return names[0], x
+
+
 def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO, in_dtype,
                    mask_value: str = "-inf") -> LoweredFunctors:
     """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
@@ -315,6 +350,12 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
         fields.append(k)
         inits.append(init_literal(v.code.name))
     new_scores, new_rowscales, o_scale = online_func.online_fwd(scores_mod, rowscales, b, h, q_idx)
+    deferred = find_deferred_norm(rowscales, new_scores, new_rowscales, o_scale)
+    if deferred is not None and os.environ.get("AE_DEFER_NORM", "1") != "0":
+        # accumulate unscaled, divide by the final row scale in the epilogue (see find_deferred_norm)
+        new_scores, o_scale = deferred[1], 1.0
+    else:
+        deferred = None
     em = Emitter(leaves, {}, ["block_N"], n="N", prefix="of")
     lazy = find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale)
     softmax = None
@@ -373,7 +414,12 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     fvals = [(k, em.value(v)) for k, v in final_rowscales.items()]
     if any(sid in em.done for sid in cust_preambles):
         raise NotImplementedError("a custom input with a seq_len_kv dimension cannot be used in the epilogue")
-    body = [em.code()]
+    body = []
+    if deferred is not None:
+        body += [f"  // the accumulator holds the unscaled sum: the per-tile normalisation by st.{deferred[0]} was deferred",
+                 f"  {{ const float ae_inv = 1.0f / st.{deferred[0]};", "#pragma unroll",
+                 "    for (int e = 0; e < N; e++) o[e] *= ae_inv; }"]
+    body.append(em.code())
     if oval[0] != "o":
         src = f"{oval[0]}[e]" if oval[1] else oval[0]
         body += ["#pragma unroll", f"  for (int e = 0; e < N; e++) o[e] = {src};"]
@@ -391,6 +437,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     lf.custom_prefetch = cust_prefetch
     lf.softmax = softmax
     lf.elementwise = bool(elementwise and not fvals)
+    lf.deferred_norm = deferred[0] if deferred is not None else None
     return lf
 
 

@@ -462,3 +462,33 @@ def test_elementwise_graphs_are_recognised():
     assert big.template == "ae_prefill_pipe.hip" and small.template == "ae_prefill.hip"
     cfg = L.render_config(128, 128, f16, big, 0, False, 0, True, True, True, None, elementwise=True)
     assert "#define AE_PIPE_KIND 1" in cfg
+
+
+def test_per_tile_renormalisation_is_deferred_to_the_epilogue(monkeypatch):
+    """scores / r_new with o_scale = r_old / r_new (retention's running sum of |s|): the factors telescope, so
+    the lowering accumulates unscaled and divides once by the final row scale - no rescale of the accumulator
+    per tile.  The row state and the final row scale are untouched; graphs of another form are left alone."""
+    import attn_script as C
+    from core.lower import lower as L
+    f16 = torch.float16
+    lf = L.trace_functors(C.retention_score_mod, C.causal_mask, C.OnlineRetention(), C.retention_custom_inputs(),
+                          f16, "0")
+    assert lf.deferred_norm == "r" and lf.o_scale_one
+    src = L.render_functors(lf)
+    fwd = src[src.index("AE_DEV float ae_online_fwd"):src.index("AE_DEV void ae_epilogue")]
+    assert " / " not in fwd.split("#endif")[-1] and "const float ae_o_scale = 1.0f;" in fwd
+    epi = src[src.index("AE_DEV void ae_epilogue"):]
+    assert "1.0f / st.r" in epi and "frs[0] = st.r;" in epi
+    assert L.trace_functors(C.make_scale_score_mod(0.125), None, C.OnlineSoftmax(), CustomIO({}), f16).deferred_norm is None
+    assert L.trace_functors(C.make_relu_score_mod(0.125), None, C.OnlineIdentity(), CustomIO({}), f16).deferred_norm is None
+
+    class ScaledDifferently(C.OnlineAbsNorm):        # o_scale does not match the normalisation of the scores
+        @staticmethod
+        def online_fwd(scores, online_rowscales, b, h, q_idx):
+            s, rs, o_scale = C.OnlineAbsNorm.online_fwd(scores, online_rowscales, b, h, q_idx)
+            return s, rs, o_scale * 0.5
+    assert L.trace_functors(C.make_scale_score_mod(0.125), None, ScaledDifferently(), CustomIO({}), f16).deferred_norm is None
+    monkeypatch.setenv("AE_DEFER_NORM", "0")
+    lf0 = L.trace_functors(C.retention_score_mod, C.causal_mask, C.OnlineRetention(), C.retention_custom_inputs(),
+                           f16, "0")
+    assert lf0.deferred_norm is None and not lf0.o_scale_one

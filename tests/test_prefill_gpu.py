@@ -363,10 +363,13 @@ def test_pipelined_kernel(cuda_device, monkeypatch, case):
     (2, 3, 200, 128, 128, torch.bfloat16),     # ragged q and kv tiles, batch > 1 against a [1,H,S,S] mask
     (1, 2, 512, 256, 512, torch.float16),      # head dims of attn_script/retention.py
 ])
-def test_retention_with_decay_mask_input(cuda_device, B, H, S, D, DV, dtype):
+@pytest.mark.parametrize("defer", ["1", "0"])
+def test_retention_with_decay_mask_input(cuda_device, monkeypatch, B, H, S, D, DV, dtype, defer):
     """attn_script/retention.py: score * mask with the mask a [1,H,S,S] input tensor (one element
-    per score, read inside the tile loop), abs-sum normalisation clamped at 1, mask_value="0"."""
-    print(f"case retention B{B} H{H} S{S} D{D} DV{DV} {dtype}", flush=True)
+    per score, fetched a tile ahead), abs-sum normalisation clamped at 1, mask_value="0".  With the
+    per-tile renormalisation deferred to the epilogue (the default) and as the script writes it."""
+    print(f"case retention B{B} H{H} S{S} D{D} DV{DV} {dtype} defer={defer}", flush=True)
+    monkeypatch.setenv("AE_DEFER_NORM", defer)
     q, k, v = C.make_inputs(B, S, S, H, H, D, DV, dtype)
     q = (q.float() * (1 / D) ** 0.5).to(dtype)                       # bench_utils.py:1034-1036
     g = torch.Generator().manual_seed(5)
@@ -375,6 +378,7 @@ def test_retention_with_decay_mask_input(cuda_device, B, H, S, D, DV, dtype):
             meta_tensor(B, H, S, DV, dtype=dtype))
     mod = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
                           mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0")
+    assert mod.attention.functors.deferred_norm == ("r" if defer == "1" else None)
     out = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).float().cpu()
     ref, r = R.retention_attention(q, k, v, mask)
     assert (r > 1.0).any()
