@@ -525,7 +525,8 @@ _MI355X_CUS = 256
 
 def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0,
                          elementwise: bool = False) -> PrefillTiles:
-    """The direct-to-LDS kernels handle 128- and 256-byte K/V rows (head dims 64 and 128): the
+    """The direct-to-LDS kernels handle head dims 64 and 128 (and, the generic one, 256 and value head dims
+    up to 512 with one wave per SIMD): the
     software-pipelined one (64 rows per wave, 256-row q tiles, one wave per SIMD) when the graph is
     the online softmax of scaled scores, or elementwise (out = sum f(s) v: the kernel then calls the
     generated functor), and the problem has enough q tiles to occupy the chip
@@ -534,6 +535,11 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
     register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one wave per SIMD and a
     shorter kv tile once the accumulators outgrow 256 registers.  AE_PREFILL_KERNEL=generic|pipelined
     overrides the choice between the first two (tests)."""
+    if d in (64, 128, 256) and dv in (64, 128, 256, 512) and max(d, dv) > 128:
+        # wide heads in the direct-to-LDS kernel: the accumulators of 32 rows (up to 256 registers for 512
+        # value columns) and the Q fragments take one wave per SIMD; 64-key tiles while a wave's share of
+        # a tile fits one burst of eight loads, else 32
+        return PrefillTiles(waves_per_eu=1, block_n=64 if dv <= 256 else 32)
     if d in (64, 128) and dv in (64, 128):
         force = os.environ.get("AE_PREFILL_KERNEL", "")
         n_tiles = batch_heads * ((seqlen_q + 255) // 256)

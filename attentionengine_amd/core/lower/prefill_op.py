@@ -8,6 +8,8 @@ rowscales, launches on torch's current stream, returns ``o``.
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from ..runtime import hip_rt as rt
@@ -32,12 +34,15 @@ class PrefillOp:
             raise ValueError("q and k head dims differ")
         if self.D % 16 or self.DV % 32:
             raise NotImplementedError(f"head dims (D={self.D}, DV={self.DV}) must be multiples of 16 / 32")
-        # Value head dims above 256 (attn_script/retention.py: DV = 512) run as several launches over
-        # column slices of V and of the output: O for 512 columns would need 256 accumulator registers
-        # per lane, which spills (measured 8.0 ms against 2 x 1.2 ms at B1 H32 S4096 D256).  The scores
-        # are recomputed per slice; the row scales of every launch are the same.
+        # Value head dim 512 with head dim 64 / 128 / 256 (attn_script/retention.py: D 256, DV 512) runs in one
+        # launch of the direct-to-LDS kernel: 256 accumulator registers per lane, one wave per SIMD, its
+        # epilogue working block by block.  Other value head dims above 256 run as several launches over
+        # column slices of V and of the output (the scores are recomputed per slice; the row scales of every
+        # launch are the same); AE_DV_SLICE=1 forces that form.
         self.DV_launch = self.DV
-        if self.DV > 256:
+        single_pass = (self.D in (64, 128, 256) and self.DV == 512 and os.environ.get("AE_DV_SLICE", "") != "1"
+                       and not split_kv)
+        if self.DV > 256 and not single_pass:
             self.DV_launch = next(c for c in (256, 192, 128, 96, 64, 32) if self.DV % c == 0)
         self.mask_mod = mask_mod
         self.elementwise_mask = mask_mod is not None and mask_value == "-inf"
@@ -63,7 +68,7 @@ class PrefillOp:
         self.split_kv = bool(split_kv)
         self.target_workgroups = int(target_workgroups)
         if self.split_kv:
-            if self.tiles.template == "ae_prefill_simple.hip":
+            if self.tiles.template == "ae_prefill_simple.hip" or max(self.D, self.DV) > 128:
                 raise NotImplementedError("split-KV prefill needs head dims 64 or 128")
             if self.DV_launch != self.DV:
                 raise NotImplementedError("split-KV prefill with a value head dim above 256")

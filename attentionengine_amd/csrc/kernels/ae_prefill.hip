@@ -7,7 +7,7 @@
 // O += P V, then the epilogue and the final-rowscale store.
 //
 // The user-defined parts arrive in "ae_config.h" / "ae_functors.h", generated from the traced
-// score_mod / mask_mod / OnlineFunc graphs:
+// score_mod / mask_mod / OnlineFunc graphs (head dims 64, 128, 256; value head dims 64 ... 512):
 //   configuration  AE_D AE_DV AE_BN AE_NWAVES AE_DTYPE_BF16 AE_MASK_MODE AE_HAS_MASK_MOD
 //                  AE_N_ROWSCALES AE_O_SCALE_ONE AE_EVEN_Q AE_EVEN_KV AE_WAVES_PER_EU
 //   functors       ae_rowstate, ae_rowstate_init, ae_mask_mod, ae_score_mod, ae_online_fwd,
@@ -73,6 +73,9 @@
 #define AE_K_RPI (64 / AE_KCPR)   // K rows one wave instruction (64 lanes x 16 B) covers
 #define AE_V_RPI (64 / AE_VCPR)
 #define AE_VPPR (AE_VCPR / 2)     // 32-byte pairs per V row
+// the pairs of a V row are exchanged by the row's low bits: at most three of them, so that rows 8 apart (the
+// two halves of a transposed fragment) share one permutation whatever the row length
+#define AE_VSWM ((AE_VPPR < 8 ? AE_VPPR : 8) - 1)
 
 static_assert(AE_D % 16 == 0, "head dim must be a multiple of 16");
 static_assert(AE_DV % 32 == 0, "value head dim must be a multiple of 32");
@@ -80,8 +83,8 @@ static_assert(AE_BN % 32 == 0, "kv tile must be a multiple of 32");
 static_assert((AE_BN * AE_KCPR) % AE_NT == 0, "K tile must split evenly over the workgroup");
 static_assert((AE_BN * AE_VCPR) % AE_NT == 0, "V tile must split evenly over the workgroup");
 static_assert(AE_K_LOADS >= 1 && AE_K_LOADS <= 8 && AE_V_LOADS >= 1 && AE_V_LOADS <= 8, "one burst per tile and wave");
-static_assert(AE_KCPR == 8 || AE_KCPR == 16, "swizzle is written for 128- or 256-byte K rows");
-static_assert(AE_VCPR == 8 || AE_VCPR == 16, "swizzle is written for 128- or 256-byte V rows");
+static_assert(AE_KCPR == 8 || AE_KCPR == 16 || AE_KCPR == 32, "swizzle is written for 128-, 256- or 512-byte K rows");
+static_assert(AE_VCPR == 8 || AE_VCPR == 16 || AE_VCPR == 32 || AE_VCPR == 64, "swizzle is written for 128- to 1024-byte V rows");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 
@@ -203,7 +206,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   auto v_lane_off = [&](int i, int last_row) -> unsigned {
     int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
     const int cp = lane % AE_VCPR;
-    const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
+    const int c = (((cp >> 1) ^ (row & AE_VSWM)) << 1) | (cp & 1);
     row = row < last_row ? row : last_row;
     return (unsigned)((row * (int)p.v_stride_s + c * 8) * 2 + 4096 - (i - AE_V_LOADS / 2) * 1024);
   };
@@ -268,7 +271,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // (2*db + g) ^ (row mod PPR), g = (lane%32)/16; rows of one group differ only in their low bits
   const int v_row = 4 * hf + ((lane & 15) >> 2);
   const int v_row_off = v_row * AE_VSTR + (lane & 3) * 8;
-  const int v_sw = v_row & (AE_VPPR - 1);
+  const int v_sw = v_row & AE_VSWM;
   const int v_g = l32 >> 4;
 
 #if AE_NSPLIT > 1
@@ -386,7 +389,18 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
         for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
-          for (int r = 0; r < 16; r++) oacc[rb][db][r] *= o_scale;
+          for (int r = 0; r < 16; r++) {
+#if AE_NO > 128 && AE_WAVES_PER_EU == 1
+            // wide value heads keep O in the accumulator file: one register at a time through one scratch
+            // register (as plain arithmetic the allocator wants all of O in ordinary registers, and spills)
+            float o = oacc[rb][db][r], t;
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                         : "+a"(o), "=&v"(t) : "v"(o_scale));
+            oacc[rb][db][r] = o;
+#else
+            oacc[rb][db][r] *= o_scale;
+#endif
+          }
       }
 #else
       (void)o_scale;
@@ -400,7 +414,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
       const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
 #pragma unroll
       for (int db = 0; db < AE_NDB; db++) {
-        // (rb0 and +8 are multiples of 8 >= pairs per row, so they do not change the swizzle)
+        // (rb0 and +8 are multiples of 8, so they do not change the swizzle)
         ae_lds_byte* a0 = vs_ + v_row_off + rb0 * AE_VSTR + (((2 * db + v_g) ^ v_sw) << 5);
         ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (__attribute__((address_space(3))) ae_s16x4*)a0);
@@ -421,6 +435,43 @@ void ae_prefill_kernel(const ae_attn_params p) {
   }
 
   // ---- epilogue -------------------------------------------------------------------------------
+#if AE_NO > 128 && AE_NSPLIT == 1
+  // wide value heads: the epilogue functor (elementwise over the value columns) runs one 32-column block at a
+  // time; a copy of all of O next to its accumulators would not fit the register file
+#pragma unroll
+  for (int rb = 0; rb < AE_RB; rb++) {
+    float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+    frs[0] = 0.f;
+    ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow[rb] * p.o_stride_s +
+                    (int64_t)h * p.o_stride_h;
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++) {
+      float o[16];
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[r] = oacc[rb][db][r];
+      if (any_tile) {
+        ae_epilogue<16>(o, st[rb], frs, ctx[rb], cust[rb]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
+      }
+      if (q_ok[rb]) {
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int t = 0; t < 4; t++) w[t] = (ae_elem)o[rg * 4 + t];
+          *(ae_elem4*)(optr + db * 32 + rg * 8 + hf * 4) = w;
+        }
+      }
+    }
+    if (q_ok[rb] && hf == 0) {
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+        p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[rb]] = frs[i];
+    }
+  }
+#else
 #pragma unroll
   for (int rb = 0; rb < AE_RB; rb++) {
     float o[AE_NO];
@@ -477,6 +528,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     }
 #endif
   }
+#endif  // wide value heads
 }
 
 #if AE_NSPLIT > 1

@@ -431,6 +431,41 @@ def test_small_and_odd_shapes_against_oracle(cuda_device):
         assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL, (B, H, Hkv, S, D)
 
 
+@pytest.mark.parametrize("B,H,Hkv,Sq,Skv,D,DV,dtype,mask,slice_dv", [
+    (1, 2, 2, 300, 300, 256, 256, torch.float16, "causal", False),     # 512-byte K and V rows, ragged tiles
+    (2, 4, 2, 257, 257, 256, 512, torch.bfloat16, None, False),        # retention's head dims in ONE launch, grouped heads
+    (1, 2, 2, 384, 384, 128, 512, torch.float16, "window", False),     # tile-class table + mask_mod, 32-key tiles
+    (1, 2, 1, 200, 200, 64, 256, torch.float16, "causal", False),
+    (1, 2, 2, 320, 320, 256, 512, torch.float16, "causal", True),      # the sliced form (two launches of 256 columns)
+])
+def test_wide_head_dims_in_the_direct_to_lds_kernel(cuda_device, monkeypatch, B, H, Hkv, Sq, Skv, D, DV, dtype, mask,
+                                                    slice_dv):
+    """Head dim 256 and value head dims 256 / 512 (attn_script/retention.py: D 256, DV 512; the reference's
+    `shared_fuse` case, core/lower/lower.py:648-654) run in the generic direct-to-LDS kernel with one wave per
+    SIMD; DV 512 in a single launch unless AE_DV_SLICE=1 asks for the sliced form."""
+    print(f"case wide heads B{B} H{H}/{Hkv} Sq{Sq} Skv{Skv} D{D} DV{DV} {dtype} {mask} slice={slice_dv}", flush=True)
+    if slice_dv:
+        monkeypatch.setenv("AE_DV_SLICE", "1")
+    q, k, v = C.make_inputs(B, Sq, Skv, H, Hkv, D, DV, dtype, seed=7)
+    mask_mod = {None: None, "causal": C.causal_mask, "window": C.make_sliding_window_mask(100)}[mask]
+    meta = (meta_tensor(B, H, Sq, D, dtype=dtype), meta_tensor(B, Hkv, Skv, D, dtype=dtype),
+            meta_tensor(B, Hkv, Skv, DV, dtype=dtype))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod=mask_mod,
+                          online_func=C.OnlineSoftmax())
+    op = mod.attention
+    assert op.DV_launch == (256 if slice_dv else DV)
+    assert op.tiles.template == "ae_prefill.hip" and op.tiles.waves_per_eu == 1
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    if mask_mod is None:
+        mk = None
+    else:
+        mk = mask_mod(0, 0, torch.arange(Sq)[:, None], torch.arange(Skv)[None, :])[None, None]
+    ref, lse = R.softmax_attention(q, k, v, mask=mk)
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
 def test_pipelined_kernel_exact_scale_switch(cuda_device, monkeypatch):
     """AE_PREFILL_PRESCALE=0: the pipelined kernel leaves Q alone and scales every score in fp32; lse then
     holds 1e-3 (+ fp32 rounding) also for scores of size 60."""
