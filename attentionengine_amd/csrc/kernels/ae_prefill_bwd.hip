@@ -92,6 +92,13 @@ static_assert(AE_BWD_ROLE == 0 || AE_BWD_ROLE == 1, "role");
 #ifndef AE_BWD_KIND
 #define AE_BWD_KIND 0
 #endif
+// 1: at the top of every tile the output accumulators are named as accumulator-file values (an empty asm).
+// Launches with one wave per SIMD use both register files; without the hint the register allocator keeps a
+// quarter of the output accumulators in ordinary registers and moves them in and out around the p / ds
+// arithmetic: 64 moves per tile.
+#ifndef AE_BWD_PIN_ACC
+#define AE_BWD_PIN_ACC (AE_BWD_WAVES_PER_EU == 1)
+#endif
 static_assert(AE_MASK_MODE >= 0 && AE_MASK_MODE <= 2, "none, causal, or tile-class tables");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
@@ -360,6 +367,14 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     const ae_lds_byte* t1 = lds + (n % AE_NSTAGE) * AE_STAGE_BYTES;
     const ae_lds_byte* t2 = t1 + AE_T1_BYTES;
     const int s0 = item_tile(it) * AE_BS;
+#if AE_BWD_PIN_ACC
+#pragma unroll
+    for (int db = 0; db < AE_NDB1; db++) asm volatile("" : "+a"(acc1[db]));
+#if AE_BWD_ROLE == 1
+#pragma unroll
+    for (int db = 0; db < AE_NDB2; db++) asm volatile("" : "+a"(acc2[db]));
+#endif
+#endif
 
     // S = X1 R1^T and dP = X2 R2^T, [streamed row][resident row], one 32-row block of the tile at a
     // time; p and ds are packed as B operands: k-step kk holds the lane's elements 8*kk .. 8*kk+7
