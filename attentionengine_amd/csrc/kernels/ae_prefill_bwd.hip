@@ -378,7 +378,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 
     // S = X1 R1^T and dP = X2 R2^T, [streamed row][resident row], one 32-row block of the tile at a
     // time; p and ds are packed as B operands: k-step kk holds the lane's elements 8*kk .. 8*kk+7
-    ae_elem8 pf[4], dsf[4];
+    ae_u32x4 pf[4], dsf[4];       // as packed pairs: two scores are converted by ONE packed conversion
 #if AE_BWD_ROLE == 1
     const ae_lds_f32* rs_l = (const ae_lds_f32*)(t2 + AE_T2_BYTES);
     const int hq = item_head(it);
@@ -424,9 +424,9 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
         else pacc = ae_mfma32(ring[f % AE_RING], rf2[ks], pacc);
         __builtin_amdgcn_sched_barrier(0);
       }
+      float pvs[16], dss[16];
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int e = nb * 16 + r;
         const int sl = nb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);     // streamed row inside the tile
         const int srow = s0 + sl;
 #if AE_BWD_ROLE == 0
@@ -466,8 +466,16 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #else
         const float dsv = vis ? dfac : 0.f;                    // an invisible score contributes nothing and moves nothing
 #endif
-        pf[e >> 3][e & 7] = (ae_elem)pv;
-        dsf[e >> 3][e & 7] = (ae_elem)dsv;
+        pvs[r] = pv;
+        dss[r] = dsv;
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        typedef float ae_f32x2 __attribute__((ext_vector_type(2)));
+        const int e = nb * 16 + r;
+        const ae_f32x2 p2 = {pvs[r], pvs[r + 1]}, d2 = {dss[r], dss[r + 1]};
+        pf[e >> 3][(e & 7) >> 1] = __builtin_bit_cast(unsigned, __builtin_convertvector(p2, ae_elem2));
+        dsf[e >> 3][(e & 7) >> 1] = __builtin_bit_cast(unsigned, __builtin_convertvector(d2, ae_elem2));
       }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -497,10 +505,10 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
         if (f + AE_AHEAD < NF) ring[(f + AE_AHEAD) % AE_RING] = frag(f + AE_AHEAD);
         const int kk = f / NB_OUT, j = f % NB_OUT;
         if (j < AE_NDB1) {
-          acc1[j] = ae_mfma32(ring[f % AE_RING], dsf[kk], acc1[j]);
+          acc1[j] = ae_mfma32(ring[f % AE_RING], __builtin_bit_cast(ae_elem8, dsf[kk]), acc1[j]);
         } else {
 #if AE_BWD_ROLE == 1
-          acc2[j - AE_NDB1] = ae_mfma32(ring[f % AE_RING], pf[kk], acc2[j - AE_NDB1]);
+          acc2[j - AE_NDB1] = ae_mfma32(ring[f % AE_RING], __builtin_bit_cast(ae_elem8, pf[kk]), acc2[j - AE_NDB1]);
 #endif
         }
         __builtin_amdgcn_sched_barrier(0);
