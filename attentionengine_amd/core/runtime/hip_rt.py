@@ -246,6 +246,32 @@ class Module:
         _check(lib().ae_module_code(self.handle, C.byref(data), C.byref(size)))
         return C.string_at(data, size.value)
 
+    def kernel_info(self) -> dict:
+        """{kernel name: its metadata from the code object's AMDGPU note (register counts, ``.vgpr_spill_count``,
+        scratch and LDS bytes, ...)}.  What the compiler that built THIS code object did - hipRTC's, which need not
+        agree with an offline hipcc of another ROCm release about how many registers it spills."""
+        import struct
+        import msgpack
+        f = self.code()
+        if f[:4] != b"\x7fELF" or f[4] != 2:
+            raise AEError("not a 64-bit ELF code object")
+        shoff = struct.unpack_from("<Q", f, 0x28)[0]
+        shentsize, shnum, _ = struct.unpack_from("<HHH", f, 0x3A)
+        for i in range(shnum):
+            _, typ, _, _, offset, size = struct.unpack_from("<IIQQQQ", f, shoff + i * shentsize)
+            if typ != 7:                                   # SHT_NOTE
+                continue
+            pos = offset
+            while pos < offset + size:
+                namesz, descsz, ntype = struct.unpack_from("<III", f, pos)
+                pos += 12 + ((namesz + 3) & ~3)
+                desc = f[pos:pos + descsz]
+                pos += (descsz + 3) & ~3
+                if ntype == 32:                            # NT_AMDGPU_METADATA (msgpack)
+                    md = msgpack.unpackb(desc, raw=False, strict_map_key=False)
+                    return {k[".name"]: k for k in md.get("amdhsa.kernels", [])}
+        raise AEError("code object without an AMDGPU metadata note")
+
     def kernel(self, name: str) -> Kernel:
         k = self._kernels.get(name)
         if k is None:

@@ -193,3 +193,26 @@ def test_code_object_cache_is_keyed_by_content(tmp_path, monkeypatch):
     m3 = rt.compile_module(template, headers2)
     assert not m3.from_cache and m3.key != m1.key
     rt._modules.clear()
+
+
+def test_benchmarked_kernels_do_not_spill_registers():
+    """The code objects hipRTC builds for the benchmark configurations (and the backward of the causal one) keep
+    every value in registers: a kernel that spills pays for it with scratch-memory traffic in every workgroup, and
+    an offline hipcc of another ROCm release does not show what this compiler does."""
+    import __graft_entry__ as G
+    engines = G.benchmark_engines()
+    mods = {}
+    for name, eng in engines.items():
+        op = eng._op
+        for key, v in op._variants.items():
+            mods[f"{name}{key}"] = v[0]
+    bwd = engines["c2_softmax_causal"]._op.backward_op()
+    m_dq, m_dkv, _ = bwd._variant(1, False)
+    mods["c2_bwd_dq"], mods["c2_bwd_dkv"] = m_dq, m_dkv
+    assert len(mods) >= 8
+    for name, m in mods.items():
+        info = m.kernel_info()
+        assert info, name
+        for kname, k in info.items():
+            assert k[".vgpr_spill_count"] == 0 and k[".sgpr_spill_count"] == 0, (name, kname, k[".vgpr_spill_count"])
+            assert k[".private_segment_fixed_size"] == 0, (name, kname)
