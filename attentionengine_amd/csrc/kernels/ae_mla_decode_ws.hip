@@ -250,18 +250,22 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f);
       if (SOFT) soft_begin(tn - 1);
-      ae_f32x16 sacc;
+      // even / odd k-steps accumulate separately (two independent MFMA chains)
+      ae_f32x16 sacc[2];
 #pragma unroll
-      for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+      for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[c][r] = 0.f;
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int f = 0; f < AE_NKS; f++) {
         if (f + AE_AHEAD < AE_NKS) ring[(f + AE_AHEAD) % AE_RING] = read_kfrag(f + AE_AHEAD);
-        sacc = ae_mfma32(ring[f % AE_RING], qf[f], sacc);
+        sacc[f & 1] = ae_mfma32(ring[f % AE_RING], qf[f], sacc[f & 1]);
         if (SOFT) soft_slot(f);
         __builtin_amdgcn_sched_barrier(0);
       }
-      xs = sacc;
+#pragma unroll
+      for (int r = 0; r < 16; r++) xs[r] = sacc[0][r] + sacc[1][r];
     };
     if (n_tiles > 0) score_trip(0, ae_const_bool<false>());
     __syncthreads();                             // end of trip 0: tile 1 has landed
@@ -319,6 +323,23 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     // immediate offset of load i inside its burst
     ld_off[i] -= i < AE_L1 ? (i - AE_L1 / 2) * 1024 : (i - AE_L1 - AE_L2 / 2) * 1024;
   }
+#if !AE_PAGED
+  // Dense cache: the requests go tile by tile, so a lane keeps the source address of each of its loads for the
+  // NEXT tile to request and adds the tile pitch after every request - two instructions per load and tile.
+  // (Two waves share a SIMD here: address arithmetic of ~140 instructions per tile and wave, as a base + offset
+  // form needs, made these waves, not the matrix pipe, set the pace of the whole workgroup.)
+  const char* ld_ptr[AE_LOADS];
+  unsigned ld_adv[AE_LOADS];
+#pragma unroll
+  for (int i = 0; i < AE_LOADS; i++) {
+    const bool rope = (ld_rope >> i) & 1u;
+    const unsigned stride = rope ? stride2 : stride1;
+    ld_ptr[i] = (const char*)(rope ? (const void*)k2 : (const void*)k1) + (uint64_t)((unsigned)kv_begin * (uint64_t)stride) +
+                (int64_t)ld_off[i];
+    ld_adv[i] = AE_BN * stride;
+  }
+#endif
+  // requests are made for t = 0, 1, 2, ... in this order
   auto load_tile = [&](int t_) {
     const int t = __builtin_amdgcn_readfirstlane(t_);
     int tt = t < n_tiles ? t : n_tiles - 1;
@@ -335,33 +356,43 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     const int in_page = kv0 - slot * p.page_block_size;
     const char* tile1 = (const char*)k1 + ((int64_t)page * p.k_stride_b + (int64_t)in_page * p.k_stride_s) * 2;
     const char* tile2 = (const char*)k2 + ((int64_t)page * p.k2_stride_b + (int64_t)in_page * p.k2_stride_s) * 2;
-#else
-    const char* tile1 = (const char*)k1 + (uint64_t)((unsigned)kv0 * (uint64_t)stride1);
-    const char* tile2 = (const char*)k2 + (uint64_t)((unsigned)kv0 * (uint64_t)stride2);
 #endif
-    auto source = [&](int j) -> const void* {
-      const bool rope = (ld_rope >> j) & 1u;
-      int off = ld_off[j];
-      if (__builtin_expect(ragged, 0)) {                      // rows past the end re-read the last row
+    // the lane's source of load j in this tile
+    auto source = [&](int j) -> const char* {
+#if AE_PAGED
+      return (((ld_rope >> j) & 1u) ? tile2 : tile1) + (int64_t)ld_off[j];
+#else
+      return ld_ptr[j];
+#endif
+    };
+    const char* g1[8];
+    const char* g2[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      g1[i] = source(i < AE_L1 ? i : 0);
+      g2[i] = source(i < AE_L2 ? AE_L1 + i : AE_L1);
+    }
+    if (__builtin_expect(ragged, 0)) {                        // rows past the end re-read the last row
+      asm volatile("" ::: "memory");                          // (keeps this ONE branch, out of the common path)
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int j = i < 8 ? (i < AE_L1 ? i : 0) : (i - 8 < AE_L2 ? AE_L1 + i - 8 : AE_L1);
         const int row = ((blk0 + j) * 64 + lane) / AE_CPR;
         int over = kv0 + row - (seqlen_b - 1);
         over = over > 0 ? over : 0;
-        off -= over * (int)(rope ? stride2 : stride1);
+        const int back = over * (int)(((ld_rope >> j) & 1u) ? stride2 : stride1);
+        if (i < 8) g1[i] -= back;
+        else g2[i - 8] -= back;
       }
-      return (rope ? tile2 : tile1) + (int64_t)off;
-    };
-    {
-      const void* g[8];
-#pragma unroll
-      for (int i = 0; i < 8; i++) g[i] = source(i < AE_L1 ? i : 0);
-      ae_load_lds16_burst<AE_L1>(g, dst + (blk0 + AE_L1 / 2) * 1024);
     }
-    {
-      const void* g[8];
+    ae_load_lds16_burst<AE_L1>((const void* const*)g1, dst + (blk0 + AE_L1 / 2) * 1024);
+    ae_load_lds16_burst<AE_L2>((const void* const*)g2, dst + (blk0 + AE_L1 + AE_L2 / 2) * 1024);
+#if !AE_PAGED
+    if (t + 1 < n_tiles) {                                    // (requests past the end repeat the last tile)
 #pragma unroll
-      for (int i = 0; i < 8; i++) g[i] = source(i < AE_L2 ? AE_L1 + i : AE_L1);
-      ae_load_lds16_burst<AE_L2>(g, dst + (blk0 + AE_L1 + AE_L2 / 2) * 1024);
+      for (int i = 0; i < AE_LOADS; i++) ld_ptr[i] += ld_adv[i];
     }
+#endif
   };
   // end of a trip: tile t+2 has landed when only the newest request is outstanding; after the barrier
   // everyone is done with tile t, whose stage takes the next request
