@@ -263,8 +263,8 @@ def _pure_scale(sym, scores):
 
 
 def _no_tile_reduction(node) -> bool:
-    """True when no node of the graph reduces over the kv-tile axis (a value without the ``block_N``
-    dimension computed from one that has it)."""
+    """True when no node of the graph reduces over the kv-tile axis (a reduction node, or a value without the
+    ``block_N`` dimension computed from one that has it)."""
     seen, stack = set(), [node]
     while stack:
         n = stack.pop()
@@ -272,6 +272,8 @@ def _no_tile_reduction(node) -> bool:
             continue
         seen.add(id(n))
         prev = [q for q in (n.prev or []) if isinstance(q, SymbolScalar)]
+        if "Reduce" in str(getattr(n.code, "type", "")):
+            return False
         if "block_N" not in n.shape_idx and any("block_N" in q.shape_idx for q in prev):
             return False
         stack.extend(prev)
