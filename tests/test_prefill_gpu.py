@@ -362,6 +362,7 @@ def test_pipelined_kernel(cuda_device, monkeypatch, case):
     (1, 2, 256, 64, 64, torch.float16),
     (2, 3, 200, 128, 128, torch.bfloat16),     # ragged q and kv tiles, batch > 1 against a [1,H,S,S] mask
     (1, 2, 512, 256, 512, torch.float16),      # head dims of attn_script/retention.py
+    (1, 2, 200, 96, 160, torch.float16),       # head dims only the register-staged kernel takes
 ])
 @pytest.mark.parametrize("defer", ["1", "0"])
 def test_retention_with_decay_mask_input(cuda_device, monkeypatch, B, H, S, D, DV, dtype, defer):
