@@ -75,11 +75,16 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
         extents = {"batch": "p.batch", "heads": "p.heads_q", "seq_len": "p.seqlen_q",
                    _KV_DIM: "p.seqlen_kv"}
         kv_stride = None
+        base_terms, q_stride = [], "0"      # the same index without its query-row term, and that term's stride
         for d in reversed(dims):
             if d in _DIM_INDEX:
                 # rows past seqlen_q (a ragged last q tile) compute on the last row and are never stored
                 ix = "(ctx.q_idx < p.seqlen_q ? ctx.q_idx : p.seqlen_q - 1)" if d == "seq_len" else _DIM_INDEX[d]
                 idx_terms.append(f"(int64_t)({ix}) * ({stride})")
+                if d == "seq_len":
+                    q_stride = stride
+                else:
+                    base_terms.append(idx_terms[-1])
                 stride = f"{stride} * (int64_t){extents[d]}"
             elif d == _KV_DIM:
                 kv_stride = stride          # the kv term is added per element inside the tile loop
@@ -94,12 +99,23 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
             # one element per score (e.g. the retention decay mask, attn_script/retention.py:14-16):
             # the row's base pointer is kept per lane, elements are read in the input dtype where the
             # scores are modified; kv positions past the end of a ragged tile read the last element
+            base_index = " + ".join(base_terms) if base_terms else "0"
             fields += [f"const ae_elem* {name}_row;", f"int64_t {name}_kvstride;", f"int {name}_kvlast;",
                        "#if AE_KV_PF_GROUPS > 0",
                        f"ae_elem4 {name}_pf[AE_KV_PF_GROUPS];   // the lane's elements of the tile fetched ahead",
+                       "#endif",
+                       "#if AE_KV_COALESCED",
+                       f"const ae_elem* {name}_base;            // element (b, h, row 0, kv 0)",
+                       f"int64_t {name}_qstride;                // elements between query rows",
+                       f"ae_elem8 {name}_raw[AE_KV_PF_GROUPS / 2];   // the tile fetched ahead, 16 bytes of a row per lane",
+                       f"bool {name}_staged;                    // raw holds the tile (else pf does)",
                        "#endif"]
             loads += [f"c.{name}_row = (const ae_elem*)p.custom[{slot}] + ({index});",
-                      f"c.{name}_kvstride = {kv_stride};", f"c.{name}_kvlast = p.seqlen_kv - 1;"]
+                      f"c.{name}_kvstride = {kv_stride};", f"c.{name}_kvlast = p.seqlen_kv - 1;",
+                      "#if AE_KV_COALESCED",
+                      f"c.{name}_base = (const ae_elem*)p.custom[{slot}] + ({base_index});",
+                      f"c.{name}_qstride = {q_stride};", f"c.{name}_staged = false;",
+                      "#endif"]
             leaves[id(sym)] = (f"cm_{name}", True)
             # a lane's elements come in groups of four consecutive kv positions (ae_kv_off): one 8-byte
             # load per group where the tensor allows it (unit kv stride, aligned, inside the row)
@@ -118,7 +134,44 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
                 f"        cust.{name}_pf[g][i] = cust.{name}_row[(int64_t)kvi * cust.{name}_kvstride];",
                 "      }",
                 "    }"]
-            prefetch += ["#pragma unroll", "  for (int g = 0; g < AE_KV_PF_GROUPS; g++) {", *group_load, "  }"]
+            # Coalesced form (kernels that define AE_KV_COALESCED and hand a wave-private LDS scratch to
+            # ae_stage_custom): a lane's own elements are 8-byte pieces of 32 different rows per load
+            # instruction, which the texture path serves one cache line at a time; instead instruction
+            # (half h, row group rg) fetches 64 contiguous bytes of each of 16 rows (row 16*rg + lane/4,
+            # 16 bytes at kv 32*h + 8*(lane%4)) and the wave redistributes the tile through LDS.
+            coalesced = [
+                "#if AE_KV_COALESCED",
+                f"  cust.{name}_staged = cust.{name}_kvstride == 1 && kv0 + 8 * AE_KV_PF_GROUPS <= p.seqlen_kv && "
+                f"(cust.{name}_qstride & 7) == 0 && (((unsigned long)cust.{name}_base) & 15) == 0;",
+                f"  if (cust.{name}_staged) {{",
+                "#pragma unroll",
+                "    for (int i = 0; i < AE_KV_PF_GROUPS / 2; i++) {",
+                "      int row = row0 + 16 * (i & 1) + (lane >> 2);",
+                "      row = row < p.seqlen_q ? row : p.seqlen_q - 1;",
+                f"      cust.{name}_raw[i] = *(const ae_elem8*)(cust.{name}_base + (int64_t)row * cust.{name}_qstride + "
+                "kv0 + 32 * (i >> 1) + 8 * (lane & 3));",
+                "    }",
+                "  } else",
+                "#endif",
+                "  {"]
+            prefetch += [*coalesced, "#pragma unroll", "  for (int g = 0; g < AE_KV_PF_GROUPS; g++) {", *group_load,
+                         "  }", "  }"]
+            stage = preambles.setdefault("stage", [])
+            stage += [
+                f"  if (cust.{name}_staged) {{",
+                "#pragma unroll",
+                "    for (int h = 0; h < AE_KV_PF_GROUPS / 4; h++) {",
+                "      // rows of 64 bytes (32 kv positions) at a pitch of 80 (16-byte aligned for the 128-bit writes)",
+                "#pragma unroll",
+                "      for (int rg = 0; rg < 2; rg++)",
+                "        *(__attribute__((address_space(3))) ae_elem8*)(scratch + (16 * rg + (lane >> 2)) * 80 + (lane & 3) * 16) = "
+                f"cust.{name}_raw[2 * h + rg];",
+                "#pragma unroll",
+                "      for (int g = 0; g < 4; g++)",
+                f"        cust.{name}_pf[4 * h + g] = *(const __attribute__((address_space(3))) ae_elem4*)"
+                "(scratch + (lane & 31) * 80 + 16 * g + 8 * (lane >> 5));",
+                "    }",
+                "  }"]
             preambles[id(sym)] = [
                 f"  float cm_{name}[N];",
                 "#if AE_KV_PF_GROUPS > 0",
@@ -151,6 +204,7 @@ def _custom_leaves(custom_fwd_inputs: CustomIO, in_dtype, slot_offset: int = 0):
         tdtype = torch.float32
         descs.append(CustomInput(name, dims, per_kv, tdtype))
     preambles["prefetch"] = prefetch
+    preambles.setdefault("stage", [])
     return leaves, descs, loads, fields, preambles
 
 
@@ -321,6 +375,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     custom_fwd_inputs = custom_fwd_inputs if custom_fwd_inputs is not None else CustomIO()
     cust_leaves, customs, cust_loads, cust_fields, cust_preambles = _custom_leaves(custom_fwd_inputs, in_dtype)
     cust_prefetch = cust_preambles.pop("prefetch")
+    cust_stage = cust_preambles.pop("stage")
 
     def index_leaves():
         b = SymbolScalar("b", Var("b"), shape_idx=[])
@@ -437,6 +492,7 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
     lf.custom_fields = cust_fields
     lf.custom_loads = cust_loads
     lf.custom_prefetch = cust_prefetch
+    lf.custom_stage = cust_stage
     lf.softmax = softmax
     lf.elementwise = bool(elementwise and not fvals)
     lf.deferred_norm = deferred[0] if deferred is not None else None
@@ -454,19 +510,34 @@ def render_functors(lf: LoweredFunctors) -> str:
     prefetch = ""
     if getattr(lf, "custom_prefetch", None):
         body = "\n".join(lf.custom_prefetch)
+        stage_body = "\n".join(getattr(lf, "custom_stage", []))
         prefetch = f"""#if AE_KV_PF_GROUPS > 0
 // custom inputs with a kv dimension: the lane's elements of the tile whose first kv position (for this lane)
 // is kv_base, fetched into cust for the functors' next call
 #define AE_HAS_KV_PREFETCH 1
-AE_DEV void ae_prefetch_custom(ae_custom& cust, int kv_base) {{
+// kv_base: the lane's first kv position of the tile (its own elements); row0 / kv0: first query row of the wave's
+// 32-row block and first kv position of the tile (the coalesced form)
+AE_DEV void ae_prefetch_custom(ae_custom& cust, int kv_base, int row0, int kv0, const ae_attn_params& p) {{
+  const int lane = threadIdx.x & 63; (void)lane; (void)row0; (void)kv0;
 {body}
 }}
+#if AE_KV_COALESCED
+// the tile fetched ahead goes from the coalesced layout to the lanes that own its elements, through 2560 bytes of
+// LDS that belong to this wave alone (a wave's LDS operations complete in order: no wait between its writes and reads)
+AE_DEV void ae_stage_custom(ae_custom& cust, __attribute__((address_space(3))) unsigned char* scratch) {{
+  const int lane = threadIdx.x & 63;
+{stage_body}
+}}
+#endif
 #endif
 """
     return f"""// generated by core/lower/lower.py -- do not edit
 {MASK_HELPERS}
 #ifndef AE_KV_PF_GROUPS
 #define AE_KV_PF_GROUPS 0      // kernels that fetch per-score custom inputs a tile ahead define it before this header
+#endif
+#ifndef AE_KV_COALESCED
+#define AE_KV_COALESCED 0      // ... and 1 if they also hand ae_stage_custom a wave-private LDS scratch
 #endif
 struct ae_custom {{
 {cfields}

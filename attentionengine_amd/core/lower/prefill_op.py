@@ -159,6 +159,15 @@ class PrefillOp:
         per = -(-kv_tiles // want)
         return -(-kv_tiles // per), per * bn
 
+    def _kv_custom_scratch(self) -> int:
+        """LDS a launch needs beyond its K / V stages: the direct-to-LDS kernel redistributes the tiles of custom
+        inputs with a kv dimension (fetched in a coalesced layout) through 2560 bytes per wave and 32-row block
+        (AE_KV_SCRATCH of ae_prefill.hip; its builds with two waves per SIMD)."""
+        if (self.tiles.template != "ae_prefill.hip" or self.tiles.waves_per_eu < 2
+                or not any(c.per_kv for c in self.functors.customs)):
+            return 0
+        return self.tiles.n_waves * (self.tiles.rows_per_wave // 32) * 2560
+
     def _variant(self, mask_mode, even_q, even_kv, n_split=1):
         key = (mask_mode, even_q, even_kv, n_split)
         v = self._variants.get(key)
@@ -176,7 +185,7 @@ class PrefillOp:
                                                           "ae_functors.h": self.functor_src})
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
                              threads=64 * self.tiles.n_waves,
-                             lds_bytes=self.tiles.lds_bytes(self.D, self.DV_launch), head_dim=self.D,
+                             lds_bytes=self.tiles.lds_bytes(self.D, self.DV_launch) + self._kv_custom_scratch(), head_dim=self.D,
                              head_dim_v=self.DV_launch, elem_bytes=2, n_rowscales=self.n_rowscales,
                              mask_mode=mask_mode)
             v = self._variants[key] = (module, cfg, cfg_src)

@@ -256,7 +256,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     store_tile(0);
 #ifdef AE_HAS_KV_PREFETCH
 #pragma unroll
-    for (int rb = 0; rb < AE_RB; rb++) ae_prefetch_custom(cust[rb], j * AE_BN + 4 * hf);
+    for (int rb = 0; rb < AE_RB; rb++) ae_prefetch_custom(cust[rb], j * AE_BN + 4 * hf, q0w + rb * 32, j * AE_BN, p);
 #endif
   }
   // Drain every outstanding load (Q fragments, first tile) before the loop: with loads still
@@ -333,7 +333,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #ifdef AE_HAS_KV_PREFETCH
       // the functors are done with this tile's elements of the per-score custom inputs: request the next
       // tile's, which travel while the second product runs
-      if (jn < j_end) ae_prefetch_custom(cust[rb], jn * AE_BN + 4 * hf);
+      if (jn < j_end) ae_prefetch_custom(cust[rb], jn * AE_BN + 4 * hf, q0w + rb * 32, jn * AE_BN, p);
 #endif
 
 #if !AE_EVEN_KV
