@@ -340,3 +340,44 @@ def test_mla_odd_shapes_against_oracle(cuda_device):
         assert torch.isfinite(out).all()
         assert (out[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL, (B, H, G, S)
         assert (mod.final_rowscales["lse"][:, :, 0].cpu() - lse).abs().max().item() <= LSE_TOL, (B, H, G, S)
+
+
+def test_decode_and_prefill_replay_from_a_hip_graph(cuda_device):
+    """The launches go to the caller's stream and nothing but torch allocates, so a call can be captured into
+    a HIP graph (serving loops do that for their decode step) and replayed on new contents of the same buffers.
+    Every replay is checked against the eager result, with eager work between the replays."""
+    B, Hq, Hkv, Skv, D = 4, 32, 8, 2048, 128
+    dtype = torch.float16
+    meta = (meta_tensor(B, Hq, 1, D, dtype=dtype), meta_tensor(B, Hkv, Skv, D, dtype=dtype),
+            meta_tensor(B, Hkv, Skv, D, dtype=dtype))
+    dec = AttentionEngine(meta, CustomIO({}), C.make_scale_score_mod(1 / math.sqrt(D)), None, C.OnlineSoftmax())
+    S = 512
+    pre = AttentionEngine((meta_tensor(1, 4, S, D, dtype=dtype),) * 3, CustomIO({}),
+                          C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask, C.OnlineSoftmax())
+    q, k, v = (t.cuda() for t in C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, dtype, seed=1))
+    pq, pk, pv = (t.cuda() for t in C.make_inputs(1, S, S, 4, 4, D, D, dtype, seed=2))
+    dec(q, k, v), pre(pq, pk, pv)                      # compile and warm up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        dec(q, k, v), pre(pq, pk, pv)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_d = dec(q, k, v)
+        out_p = pre(pq, pk, pv)
+    for step in range(3):
+        g = torch.Generator().manual_seed(10 + step)
+        q.copy_(torch.randn(q.shape, generator=g).to(dtype))
+        k.copy_(torch.randn(k.shape, generator=g).to(dtype))
+        pq.copy_(torch.randn(pq.shape, generator=g).to(dtype))
+        graph.replay()
+        torch.cuda.synchronize()
+        got_d, got_p = out_d.clone(), out_p.clone()
+        ref_d, ref_p = dec(q, k, v), pre(pq, pk, pv)   # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got_d, ref_d), step
+        assert torch.equal(got_p, ref_p), step
+    ref, _ = R.softmax_attention(q.cpu(), k.cpu(), v.cpu(), causal=False)
+    assert (got_d.float().cpu() - ref).abs().max().item() <= OUT_TOL
