@@ -352,7 +352,9 @@ def find_deferred_norm(rowscales, new_scores, new_rowscales, o_scale):
     ``o_scale = r_old / r_new`` with r a row scale and X free of it (retention's running sum of |s|,
     attn_script/retention.py:40-60).  The factors telescope: the output equals (sum over tiles of X v) / r_final,
     so the kernels may accumulate X v unscaled - no rescale of the whole accumulator per tile - and divide
-    once in the epilogue.  Returns (name of r, X) or None."""
+    once in the epilogue.  What changes is the range of P, the operand of the second product: |X / r| <= 1 in
+    the script's form, |X| itself here, so scores of size 65504 and more overflow an fp16 P (bf16 has the
+    range of fp32); AE_DEFER_NORM=0 in the environment keeps the script's form.  Returns (name of r, X) or None."""
     if not (isinstance(new_scores, SymbolScalar) and isinstance(o_scale, SymbolScalar)):
         return None
     if new_scores.code.type != "Div" or o_scale.code.type != "Div":
