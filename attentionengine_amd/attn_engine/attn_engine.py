@@ -88,7 +88,8 @@ class AttentionEngine:
             qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
             infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
             infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
-            kv_shared=kv_shared)
+            kv_shared=kv_shared,
+            tune=dict(tune=bool(tune), tune_file=tune_file, tune_bwd=bool(tune_bwd), tune_file_bwd=tune_file_bwd))
         # generated device source, under the attribute name scripts read
         # (attn_script/reluattn.py:75-76)
         self.tl_code = self._op.source
@@ -99,7 +100,7 @@ class AttentionEngine:
     # same dispatch order as attn_engine.py:218-332
     def _select_lower_template(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
                                mask_value, infer_mask, infer_mask_block_M, infer_mask_block_N,
-                               extern_block_mask, kv_shared):
+                               extern_block_mask, kv_shared, tune=None):
         dtype_map = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
         q_meta, k_meta, v_meta = qkv_meta
         dtype_map[q_meta.dtype]  # KeyError for unsupported dtypes, as in the reference (225-228, 304)
@@ -129,7 +130,7 @@ class AttentionEngine:
         return PrefillOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                          infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
                          infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
-                         split_kv=split_kv)
+                         split_kv=split_kv, **(tune or {}))
 
     def __call__(self, *args, **kargs):
         if kargs.get("block_mask") is not None:

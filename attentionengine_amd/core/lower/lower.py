@@ -575,8 +575,8 @@ AE_DEV void ae_epilogue(float (&o)[N], ae_rowstate& st, float (&frs)[{nrs}], con
 
 @dataclass
 class PrefillTiles:
-    """Tile configuration of a prefill template (fixed per head dim; chosen from rocprof
-    measurements rather than tuned at run time)."""
+    """Tile configuration of a prefill template: ``choose_prefill_tiles`` fixes it per head dim and problem size
+    from measurements; engines built with ``tune=True`` measure the candidates of core/lower/tuner.py instead."""
     template: str = "ae_prefill.hip"   # direct-to-LDS kernel
     n_waves: int = 4
     block_n: int = 64
@@ -618,8 +618,11 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
     if d in (64, 128) and dv in (64, 128):
         force = os.environ.get("AE_PREFILL_KERNEL", "")
         n_tiles = batch_heads * ((seqlen_q + 255) // 256)
+        # (elementwise graphs at head dim 64 have too little matrix work per score for the pipelined kernel's
+        # one wave per SIMD to pay: relu attention B64 H6 S2048 D64 0.48 ms against 0.45 ms in the generic one)
+        fits = softmax is not None or (elementwise and max(d, dv) > 64)
         if (softmax is not None or elementwise) and force != "generic" and (
-                force == "pipelined" or n_tiles >= (3 * _MI355X_CUS) // 4):
+                force == "pipelined" or (fits and n_tiles >= (3 * _MI355X_CUS) // 4)):
             return PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)
         return PrefillTiles()
     t = PrefillTiles(template="ae_prefill_simple.hip", k_pad=16)

@@ -25,7 +25,12 @@ def _dim(x, default):
 class PrefillOp:
     def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
-                 extern_block_mask=False, split_kv=False, target_workgroups=512):
+                 extern_block_mask=False, split_kv=False, target_workgroups=512,
+                 tiles=None, tune=False, tune_file="", tune_bwd=False, tune_file_bwd=""):
+        self._ctor = ((qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value),
+                      dict(infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
+                           infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
+                           split_kv=split_kv, target_workgroups=target_workgroups))
         q_meta, k_meta, v_meta = qkv_meta
         self.dtype = q_meta.dtype
         self.D = int(q_meta.shape[3])
@@ -62,6 +67,22 @@ class PrefillOp:
                                             self._pipe_softmax,
                                             _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1),
                                             elementwise=self._pipe_elementwise)
+        # tune=True (attn_tl.py:465-521 of the reference): the tile configuration comes from the record of
+        # this problem in tune_file, or is measured at the first call and recorded there.  Launches whose
+        # tiles are bound to something else (split-KV, an external block mask) keep the fixed choice.
+        self._tune_file, self._tune_pending, self.tune_times = "", False, None
+        self._tune_bwd = (bool(tune_bwd), tune_file_bwd)
+        if tiles is not None:
+            self.tiles = tiles
+        elif tune and tune_file and not split_kv and not extern_block_mask:
+            from . import tuner
+            self._tune_file = tune_file
+            self._tune_keys = tuner.problem_keys(q_meta.shape, self.D, self.DV)
+            found = tuner.decode_tiles(tuner.lookup(tune_file, self._tune_keys), self._tune_candidates())
+            if found is not None:
+                self.tiles = found
+            else:
+                self._tune_pending = True
         # Split-KV ("MHA decode": a few query tokens against a long KV, attn_engine.py:273-290 and
         # core/lower/lower_decode.py:287-313 of the reference): the kv axis is shared out over several
         # workgroups per q tile and the partial results are merged with the user's combine().
@@ -109,6 +130,34 @@ class PrefillOp:
             self.source = cfg_src + "\n" + self.functor_src
             if infer_mask and mask_mod is not None and not self.extern_block_mask:
                 self.block_mask = self._reference_block_mask(B, H, Sq, Skv)
+
+    # ---- tuning ------------------------------------------------------------------------
+    def _tune_candidates(self):
+        from . import tuner
+        return tuner.prefill_candidates(self.D, self.DV_launch, self._pipe_softmax, self._pipe_elementwise)
+
+    def _tune(self, q, k, v, *extra):
+        """Measures every candidate tile configuration on the caller's tensors, becomes the fastest one and
+        records it under this engine's problem keys (AE_TUNE_VERBOSE=1 prints the measurements)."""
+        from . import tuner
+        self._tune_pending = False
+        args, kw = self._ctor
+        log = print if os.environ.get("AE_TUNE_VERBOSE", "") == "1" else None
+        cands = self._tune_candidates()
+        mine = self.block_mask      # the engine appends this very object to every call: see _forward
+
+        def run(o):
+            return o._forward(q, k, v, *[o.block_mask if (mine is not None and x is mine) else x for x in extra])
+        best, op, times = tuner.pick(
+            cands, lambda t: self if t == self.tiles else PrefillOp(*args, **kw, tiles=t), run, log)
+        if op is not self:
+            keep = (self._ctor, self._tune_file, self._tune_keys, self._tune_bwd, mine)
+            self.__dict__.update(op.__dict__)
+            self._ctor, self._tune_file, self._tune_keys, self._tune_bwd, self.block_mask = keep
+            self._bwd = None        # the backward reads this operator's mask plans: built again on demand
+        self._tune_pending = False
+        self.tune_times = {tuple(tuner.encode_tiles(cands[i])): ms for i, ms in times.items()}
+        tuner.store(self._tune_file, self._tune_keys, tuner.encode_tiles(best))
 
     # ---- mask --------------------------------------------------------------------------
     def _plan(self, B, H, Sq, Skv, device):
@@ -202,10 +251,12 @@ class PrefillOp:
     def backward_op(self):
         if getattr(self, "_bwd", None) is None:
             from .prefill_bwd_op import PrefillBwdOp
-            self._bwd = PrefillBwdOp(self, *self._graph)
+            self._bwd = PrefillBwdOp(self, *self._graph, tune=self._tune_bwd[0], tune_file=self._tune_bwd[1])
         return self._bwd
 
     def _forward(self, q, k, v, *extra):
+        if self._tune_pending:
+            self._tune(q, k, v, *extra)
         n_custom = len(self.functors.customs)
         extern_mask = None
         if len(extra) == n_custom + 1:

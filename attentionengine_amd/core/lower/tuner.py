@@ -1,0 +1,138 @@
+"""Measured choice between the tile configurations of the prefill kernels, with the reference's json cache.
+
+The reference tunes (block_M, block_N, num_stages, thread_num, shared_fuse) of its TileLang kernel when an
+engine is built with ``tune=True`` and keeps the winner in ``tune_file``: a json list of
+``{"batch", "heads", "seq_len", "dim", "dimv", "tuned_config": [...]}`` records, looked up by the five
+problem keys before anything is measured
+(attention_engine/core/template/tl_template/attn/attn_tl.py:33-48 candidates, 465-500 cache, 503-521 use;
+backward 538-552).  Here the candidates are the tile configurations the HIP templates can be compiled with
+for the head dims at hand, the measurement is HIP events around back-to-back launches on the caller's own
+tensors at the first call, and the file keeps the same records; ``tuned_config`` is
+``[block_M, block_N, LDS stages, threads, waves per SIMD, template]`` for the forward and
+``[q rows of a dq workgroup]`` for the backward.  A record whose configuration is not among the candidates
+(e.g. written by the reference for another GPU) is ignored and measured again.
+"""
+from __future__ import annotations
+
+import json
+import os
+
+import torch
+
+from . import lower as L
+
+# extents the reference assumes for dynamic (string) dims when it looks a problem up (attn_tl.py:465-472)
+_DYNAMIC_DEFAULT = {"batch": 4, "heads": 32, "seq_len": 2048}
+
+
+def problem_keys(q_shape, dim, dimv):
+    """The five keys of a cache record from the declared q shape [batch, heads, seq_len, dim]."""
+    def ext(x, name):
+        return _DYNAMIC_DEFAULT[name] if isinstance(x, str) else int(x)
+    return {"batch": ext(q_shape[0], "batch"), "heads": ext(q_shape[1], "heads"),
+            "seq_len": ext(q_shape[2], "seq_len"), "dim": int(dim), "dimv": int(dimv)}
+
+
+def _records(tune_file):
+    if not tune_file or not os.path.exists(tune_file):
+        return []
+    try:
+        with open(tune_file) as f:
+            recs = json.load(f)
+    except (OSError, ValueError):
+        return []
+    return recs if isinstance(recs, list) else []
+
+
+def lookup(tune_file, pk):
+    """tuned_config of the record with these problem keys, or None."""
+    for rec in _records(tune_file):
+        if isinstance(rec, dict) and all(rec.get(k) == v for k, v in pk.items()):
+            return rec.get("tuned_config")
+    return None
+
+
+def store(tune_file, pk, tuned_config):
+    """Adds (or replaces) the record of this problem; the other records of the file are kept."""
+    recs = [r for r in _records(tune_file)
+            if not (isinstance(r, dict) and all(r.get(k) == v for k, v in pk.items()))]
+    recs.append({**pk, "tuned_config": list(tuned_config)})
+    with open(tune_file, "w") as f:
+        json.dump(recs, f, indent=4)
+
+
+def prefill_candidates(d, dv, softmax, elementwise):
+    """Every tile configuration the forward templates are built for at these head dims; the first one is
+    what ``choose_prefill_tiles`` picks for a problem large enough to fill the chip."""
+    if d in (64, 128, 256) and dv in (64, 128, 256, 512) and max(d, dv) > 128:
+        c = [L.PrefillTiles(waves_per_eu=1, block_n=32)]
+        if dv <= 256:
+            c.insert(0, L.PrefillTiles(waves_per_eu=1, block_n=64))
+        return c
+    if d in (64, 128) and dv in (64, 128):
+        c = [L.PrefillTiles(), L.PrefillTiles(block_n=32), L.PrefillTiles(waves_per_eu=1)]
+        if softmax is not None or elementwise:
+            c.insert(0, L.PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64))
+        return c
+    base = L.choose_prefill_tiles(d, dv)
+    c = [base]
+    other, nt = 96 - base.block_n, 64 * base.n_waves          # the kv tile is 32 or 64 keys
+    if (other * d // 8) % nt == 0 and (other * dv // 8) % nt == 0:
+        c.append(L.PrefillTiles(template=base.template, n_waves=base.n_waves, block_n=other,
+                                waves_per_eu=base.waves_per_eu, k_pad=base.k_pad, v_pad=base.v_pad))
+    return c
+
+
+def encode_tiles(t):
+    return [t.block_m, t.block_n, 2, 64 * t.n_waves, t.waves_per_eu, t.template]
+
+
+def decode_tiles(tuned_config, candidates):
+    """The candidate a cache record names, or None."""
+    if not isinstance(tuned_config, (list, tuple)):
+        return None
+    for t in candidates:
+        if list(tuned_config) == encode_tiles(t):
+            return t
+    return None
+
+
+def time_call(fn, budget_ms=30.0, min_calls=3, max_calls=200):
+    """Mean milliseconds of ``fn()`` on torch's current stream: two warm-up calls, a one-call estimate, then
+    as many back-to-back calls as fit ``budget_ms`` between two events."""
+    fn()
+    fn()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    fn()
+    end.record()
+    end.synchronize()
+    n = int(max(min_calls, min(max_calls, budget_ms / max(start.elapsed_time(end), 1e-3))))
+    start.record()
+    for _ in range(n):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / n
+
+
+def pick(candidates, build, run, log=None):
+    """Measures ``run(build(c))`` for every candidate; candidates that cannot be built or launched for this
+    problem are passed over.  Returns (best candidate, what build() made of it, {candidate index: ms})."""
+    best, times = None, {}
+    for i, c in enumerate(candidates):
+        try:
+            made = build(c)
+            ms = time_call(lambda: run(made))
+        except (NotImplementedError, ValueError, RuntimeError) as e:
+            if log is not None:
+                log(f"tune: {c} not usable here ({e})")
+            continue
+        times[i] = ms
+        if log is not None:
+            log(f"tune: {c} {ms:.4f} ms")
+        if best is None or ms < best[2]:
+            best = (c, made, ms)
+    if best is None:
+        raise RuntimeError("no tile configuration could be launched for this problem")
+    return best[0], best[1], times

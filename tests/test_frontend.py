@@ -492,3 +492,42 @@ def test_per_tile_renormalisation_is_deferred_to_the_epilogue(monkeypatch):
     lf0 = L.trace_functors(C.retention_score_mod, C.causal_mask, C.OnlineRetention(), C.retention_custom_inputs(),
                            f16, "0")
     assert lf0.deferred_norm is None and not lf0.o_scale_one
+
+
+def test_tuner_cache_records(tmp_path):
+    """tune=True / tune_file: the json records of the reference's tuner (attn_tl.py:465-500: a list of the five
+    problem keys plus ``tuned_config``), looked up at construction; nothing is measured or written without a GPU
+    call."""
+    import json
+    from core.lower import tuner
+    f = str(tmp_path / "tuned.json")
+    pk = tuner.problem_keys((2, "heads", 1024, 128), 128, 128)
+    assert pk == {"batch": 2, "heads": 32, "seq_len": 1024, "dim": 128, "dimv": 128}   # dynamic dims: attn_tl.py:465-472
+    assert tuner.lookup(f, pk) is None
+    cands = tuner.prefill_candidates(128, 128, softmax=(0.1, "m", "r"), elementwise=False)
+    assert len(cands) == 4 and cands[0].template == "ae_prefill_pipe.hip"
+    assert len(tuner.prefill_candidates(128, 128, None, False)) == 3
+    assert [c.block_n for c in tuner.prefill_candidates(256, 512, None, False)] == [32]
+    assert [c.block_n for c in tuner.prefill_candidates(192, 128, None, False)] == [32, 64]
+    tuner.store(f, pk, tuner.encode_tiles(cands[2]))
+    tuner.store(f, {**pk, "batch": 4}, [128, 128, 2, 256, False])     # a record as the reference writes it
+    recs = json.load(open(f))
+    assert [sorted(r) for r in recs] == [sorted(list(pk) + ["tuned_config"])] * 2
+    assert recs[0]["tuned_config"] == [128, 32, 2, 256, 2, "ae_prefill.hip"]
+    assert tuner.decode_tiles(tuner.lookup(f, pk), cands) == cands[2]
+    assert tuner.decode_tiles(tuner.lookup(f, {**pk, "batch": 4}), cands) is None   # not one of this build's tiles
+
+    sm = C.make_scale_score_mod(0.1)
+    hit = AttentionEngine(_meta(2, 32, 32, 1024, 1024, 128, 128, torch.float16), CustomIO({}), sm, C.causal_mask,
+                          C.OnlineSoftmax(), tune=True, tune_file=f)
+    assert hit._op.tiles == cands[2] and not hit._op._tune_pending
+    assert "#define AE_BN 32" in hit.tl_code
+    miss = AttentionEngine(_meta(4, 32, 32, 1024, 1024, 128, 128, torch.float16), CustomIO({}), sm, C.causal_mask,
+                           C.OnlineSoftmax(), tune=True, tune_file=f)
+    assert miss._op._tune_pending and miss._op.tiles == cands[0]      # measured at the first call on a GPU
+    plain = AttentionEngine(_meta(2, 32, 32, 1024, 1024, 128, 128, torch.float16), CustomIO({}), sm, C.causal_mask,
+                            C.OnlineSoftmax(), tune_file=f)
+    assert plain._op.tiles == cands[0] and not plain._op._tune_pending
+    tuner.store(f, pk, tuner.encode_tiles(cands[1]))                  # replaces the record of that problem
+    assert len(json.load(open(f))) == 2 and tuner.decode_tiles(tuner.lookup(f, pk), cands) == cands[1]
+    assert json.load(open(f)) == recs[1:] + [{**pk, "tuned_config": tuner.encode_tiles(cands[1])}]

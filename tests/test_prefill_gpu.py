@@ -564,3 +564,113 @@ def test_pipelined_kernel_scores_far_above_the_first_tiles(cuda_device, monkeypa
                         sc = sc.masked_fill(~dense, 0.0)
                     tol = tol + 2.0 ** -11 * sc.amax(-1)
                 assert ((got - lse).abs() <= tol).all(), (dtype, case, causal)
+
+
+def _tuner_case(kind):
+    """(engine, GPU call arguments, check(out, rowscales)) for one graph family the tuner covers."""
+    if kind in ("softmax_d128", "softmax_d192", "softmax_d256"):
+        D, DV, dtype = {"softmax_d128": (128, 128, torch.float16), "softmax_d192": (192, 128, torch.bfloat16),
+                        "softmax_d256": (256, 256, torch.float16)}[kind]
+        B, H, S = 1, 3, 576                     # whole 64-row tiles, a ragged 256-row tile
+        q, k, v = C.make_inputs(B, S, S, H, H, D, DV, dtype)
+        mod = _engine(B, H, S, D, DV, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask, C.OnlineSoftmax())
+        ref, lse = R.softmax_attention(q, k, v, causal=True)
+        extra = ()
+
+        def check(out, rs):
+            assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+            assert (rs["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+    elif kind == "sigmoid_d64":
+        B, H, S, D, dtype = 2, 2, 300, 64, torch.bfloat16
+        q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+        bias = torch.tensor([-math.log(S)], dtype=torch.float32)
+        mod = _engine(B, H, S, D, D, dtype, C.make_sigmoid_score_mod(1 / math.sqrt(D)), None, C.OnlineIdentity(),
+                      customs=CustomIO({"softmax_bias": (1,)}))
+        ref = R.sigmoid_attention(q, k, v, bias=bias.item())
+        extra = (bias.cuda(),)
+
+        def check(out, rs):
+            assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    else:
+        assert kind == "retention_d128"
+        B, H, S, D, dtype = 2, 2, 328, 128, torch.float16
+        q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+        q = (q.float() * (1 / D) ** 0.5).to(dtype)
+        g = torch.Generator().manual_seed(5)
+        mask = (torch.rand(1, H, S, S, generator=g) * 4.0).tril().to(dtype).contiguous()
+        meta = (meta_tensor(B, H, S, D, dtype=dtype),) * 3
+        mod = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
+                              mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0")
+        ref, r = R.retention_attention(q, k, v, mask)
+        extra = (mask.cuda(),)
+
+        def check(out, rs):
+            assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+            assert (rs["r"].cpu() - r).abs().max().item() <= 2e-3 * r.max().item()
+    return mod, (q.cuda(), k.cuda(), v.cuda()) + extra, check
+
+
+@pytest.mark.parametrize("kind", ["softmax_d128", "sigmoid_d64", "retention_d128", "softmax_d192", "softmax_d256"])
+def test_every_tile_configuration_the_tuner_may_pick(cuda_device, kind):
+    """tune=True chooses among these by time alone, so each of them must compute the same thing: every candidate
+    of core/lower/tuner.py against the oracle, on shapes with ragged q and kv tiles."""
+    from core.lower.prefill_op import PrefillOp
+    mod, args, check = _tuner_case(kind)
+    base = mod.attention
+    cands = base._tune_candidates()
+    assert len(cands) >= 2 and base.tiles in cands
+    for t in cands:
+        print(f"case {kind} tiles {t}", flush=True)
+        op = PrefillOp(*base._ctor[0], **base._ctor[1], tiles=t)
+        assert op.tiles == t
+        out = op(*args, *([op.block_mask] if op.block_mask is not None else []))
+        check(out, op.final_rowscales)
+
+
+def test_tune_measures_at_the_first_call_and_records(cuda_device, tmp_path):
+    """tune=True with an empty tune_file (attn_script/mha.py:100-104 passes tune, tune_file, tune_bwd): the first
+    forward measures every candidate and records the winner, the first backward does the same for the dq launch's
+    shape; an engine built afterwards from the same files measures nothing and computes the same results."""
+    import json
+    from core.lower import tuner
+    B, H, S, D, dtype = 2, 4, 1024, 128, torch.float16
+    f, fb = str(tmp_path / "fwd.json"), str(tmp_path / "bwd.json")
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    g = torch.Generator().manual_seed(11)
+    do = torch.randn(B, S, H, D, generator=g).to(dtype)
+    ref, lse = R.softmax_attention(q, k, v, causal=True)
+    dq, dk, dv = R.softmax_attention_grads(q, k, v, do, scale=1 / math.sqrt(D), causal=True)
+
+    def run(mod):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        out = mod(qd, kd, vd)
+        out.backward(do.cuda())
+        assert (out.detach().float().cpu() - ref).abs().max().item() <= OUT_TOL
+        assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+        for got, want in ((qd.grad, dq), (kd.grad, dk), (vd.grad, dv)):
+            assert (got.float().cpu() - want).abs().max().item() <= 2e-2 + 1e-2 * want.abs().max().item()
+        return out.detach(), qd.grad
+
+    kw = dict(tune=True, tune_file=f, tune_bwd=True, tune_file_bwd=fb)
+    first = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask, C.OnlineSoftmax(), **kw)
+    assert first.attention._tune_pending
+    out1, dq1 = run(first)
+    op = first.attention
+    cands = op._tune_candidates()
+    assert not op._tune_pending and len(op.tune_times) == len(cands) and all(ms > 0 for ms in op.tune_times.values())
+    (rec,) = json.load(open(f))
+    assert {k_: rec[k_] for k_ in ("batch", "heads", "seq_len", "dim", "dimv")} == \
+        {"batch": B, "heads": H, "seq_len": S, "dim": D, "dimv": D}
+    assert rec["tuned_config"] == tuner.encode_tiles(op.tiles)
+    assert op.tune_times[tuple(rec["tuned_config"])] == min(op.tune_times.values())
+    (recb,) = json.load(open(fb))
+    bwd = op.backward_op()
+    assert recb["tuned_config"] == [bwd.dq_rows] and set(bwd.tune_times) == {256, 128}
+    run(first)                                  # later calls measure nothing
+    assert len(json.load(open(f))) == 1
+
+    second = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask, C.OnlineSoftmax(), **kw)
+    assert not second.attention._tune_pending and second.attention.tiles == op.tiles
+    out2, dq2 = run(second)
+    assert second.attention.tune_times is None and second.attention.backward_op().dq_rows == bwd.dq_rows
+    assert torch.equal(out1, out2) and torch.equal(dq1, dq2)
