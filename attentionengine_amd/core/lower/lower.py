@@ -598,10 +598,23 @@ class PrefillTiles:
 _MI355X_CUS = 256
 
 
+# Head dims the direct-to-LDS kernel (ae_prefill.hip) is written for: its K rows are swizzled for lengths of
+# 2^n, 4*odd or 8*odd 16-byte chunks, its V rows for powers of two.
+DIRECT_D = (64, 96, 128, 160, 192, 256)
+DIRECT_DV = (64, 128, 256, 512)
+
+
+def direct_tile_ok(d: int, dv: int, block_n: int, n_waves: int = 4) -> bool:
+    """A K / V tile of block_n rows is fetched as whole 16-byte chunks, the same number per lane, at most eight
+    a wave and tile (one burst of direct loads)."""
+    nt = 64 * n_waves
+    return all((block_n * x // 8) % nt == 0 and (block_n * x // 8) // nt <= 8 for x in (d, dv))
+
+
 def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0,
                          elementwise: bool = False) -> PrefillTiles:
-    """The direct-to-LDS kernels handle head dims 64 and 128 (and, the generic one, 256 and value head dims
-    up to 512 with one wave per SIMD): the
+    """The direct-to-LDS kernels handle head dims 64 and 128 (and, the generic one, 96, 160, 192, 256 and value
+    head dims up to 512, with one wave per SIMD where the accumulators need it): the
     software-pipelined one (64 rows per wave, 256-row q tiles, one wave per SIMD) when the graph is
     the online softmax of scaled scores, or elementwise (out = sum f(s) v: the kernel then calls the
     generated functor), and the problem has enough q tiles to occupy the chip
@@ -610,18 +623,23 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
     register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one wave per SIMD and a
     shorter kv tile once the accumulators outgrow 256 registers.  AE_PREFILL_KERNEL=generic|pipelined
     overrides the choice between the first two (tests)."""
-    if d in (64, 128, 256) and dv in (64, 128, 256, 512) and max(d, dv) > 128:
+    if d in DIRECT_D and dv in DIRECT_DV and (d > 128 or dv > 128):
+        if d <= 192 and dv <= 128:
+            # head dims 160 / 192 with up to 128 value columns (192 / 128: multi-head latent attention before its
+            # absorption): the wave still fits 256 registers, two waves per SIMD; 32-key tiles where two workgroups
+            # with 64-key tiles would not fit the LDS of a compute unit
+            return PrefillTiles(block_n=64 if direct_tile_ok(d, dv, 64) and d <= 160 else 32)
         # wide heads in the direct-to-LDS kernel: the accumulators of 32 rows (up to 256 registers for 512
         # value columns) and the Q fragments take one wave per SIMD; 64-key tiles while a wave's share of
         # a tile fits one burst of eight loads, else 32
-        return PrefillTiles(waves_per_eu=1, block_n=64 if dv <= 256 else 32)
-    if d in (64, 128) and dv in (64, 128):
+        return PrefillTiles(waves_per_eu=1, block_n=64 if dv <= 256 and direct_tile_ok(d, dv, 64) else 32)
+    if d in DIRECT_D and dv in DIRECT_DV:
         force = os.environ.get("AE_PREFILL_KERNEL", "")
         n_tiles = batch_heads * ((seqlen_q + 255) // 256)
         # (elementwise graphs at head dim 64 have too little matrix work per score for the pipelined kernel's
         # one wave per SIMD to pay: relu attention B64 H6 S2048 D64 0.48 ms against 0.45 ms in the generic one)
         fits = softmax is not None or (elementwise and max(d, dv) > 64)
-        if (softmax is not None or elementwise) and force != "generic" and (
+        if d in (64, 128) and (softmax is not None or elementwise) and force != "generic" and (
                 force == "pipelined" or (fits and n_tiles >= (3 * _MI355X_CUS) // 4)):
             return PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)
         return PrefillTiles()

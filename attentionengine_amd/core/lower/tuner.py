@@ -64,15 +64,17 @@ def store(tune_file, pk, tuned_config):
 def prefill_candidates(d, dv, softmax, elementwise):
     """Every tile configuration the forward templates are built for at these head dims; the first one is
     what ``choose_prefill_tiles`` picks for a problem large enough to fill the chip."""
-    if d in (64, 128, 256) and dv in (64, 128, 256, 512) and max(d, dv) > 128:
-        c = [L.PrefillTiles(waves_per_eu=1, block_n=32)]
-        if dv <= 256:
-            c.insert(0, L.PrefillTiles(waves_per_eu=1, block_n=64))
-        return c
-    if d in (64, 128) and dv in (64, 128):
-        c = [L.PrefillTiles(), L.PrefillTiles(block_n=32), L.PrefillTiles(waves_per_eu=1)]
-        if softmax is not None or elementwise:
-            c.insert(0, L.PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64))
+    if d in L.DIRECT_D and dv in L.DIRECT_DV:
+        c = []
+        if d in (64, 128) and dv in (64, 128) and (softmax is not None or elementwise):
+            c.append(L.PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64))
+        # two waves per SIMD while a wave may fit 256 registers (Q fragments of up to 192 columns, 128 value columns)
+        shapes = [(2, 64), (2, 32), (1, 64)] if d <= 192 and dv <= 128 else [(1, 64), (1, 32)]
+        if d > 128 and dv <= 128:
+            shapes.append((1, 32))
+        for wpe, bn in shapes:
+            if L.direct_tile_ok(d, dv, bn) and not (bn == 64 and dv > 256):
+                c.append(L.PrefillTiles(waves_per_eu=wpe, block_n=bn))
         return c
     base = L.choose_prefill_tiles(d, dv)
     c = [base]

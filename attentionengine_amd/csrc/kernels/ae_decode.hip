@@ -85,15 +85,15 @@ void ae_decode_split_kernel(const ae_attn_params p) {
   ae_elem8 kf_next[2][AE_NKS];
   ae_u32x4 vreg[AE_V_LOADS];
 
-  auto tile_kv0 = [&](int i) { return wg_base + (wave + i * AE_NWAVES) * AE_TILE; };
-  auto clamp_kv = [&](int kv) {
+  auto tile_kv0 = [&](int i) AE_LAMBDA { return wg_base + (wave + i * AE_NWAVES) * AE_TILE; };
+  auto clamp_kv = [&](int kv) AE_LAMBDA {
 #if AE_EVEN_KV
     return kv;
 #else
     return kv < p.seqlen_kv ? kv : p.seqlen_kv - 1;
 #endif
   };
-  auto load_k = [&](int kv0, ae_elem8 (&dst)[2][AE_NKS]) {
+  auto load_k = [&](int kv0, ae_elem8 (&dst)[2][AE_NKS]) AE_LAMBDA {
 #pragma unroll
     for (int rb = 0; rb < 2; rb++) {
       const ae_elem* row = kbase + (int64_t)clamp_kv(kv0 + rb * 16 + l16) * p.k_stride_s + g4 * 8;
@@ -101,7 +101,7 @@ void ae_decode_split_kernel(const ae_attn_params p) {
       for (int ks = 0; ks < AE_NKS; ks++) dst[rb][ks] = *(const ae_elem8*)(row + ks * 32);
     }
   };
-  auto load_v = [&](int kv0) {
+  auto load_v = [&](int kv0) AE_LAMBDA {
 #pragma unroll
     for (int i = 0; i < AE_V_LOADS; i++) {
       int c = lane + i * 64;
@@ -109,7 +109,7 @@ void ae_decode_split_kernel(const ae_attn_params p) {
       vreg[i] = *(const ae_u32x4*)(vbase + (int64_t)clamp_kv(kv0 + row) * p.v_stride_s + col * 8);
     }
   };
-  auto store_v = [&]() {
+  auto store_v = [&]() AE_LAMBDA {
 #pragma unroll
     for (int i = 0; i < AE_V_LOADS; i++) {
       int c = lane + i * 64;

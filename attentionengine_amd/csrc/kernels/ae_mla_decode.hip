@@ -135,7 +135,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   // (w*AE_LOADS + i) mod AE_BLOCKS (a few blocks are fetched twice so every wave issues the same
   // number of loads); LDS slot s = 64*block + lane is chunk c' = s % CPR of row s / CPR and
   // receives global chunk c' ^ f(row).
-  auto load_tile = [&](int t, int stage) {
+  auto load_tile = [&](int t, int stage) AE_LAMBDA {
     const int kv0 = kv_begin + t * AE_BN;
     ae_lds_byte* dst = lds + stage * AE_STAGE_BYTES;
 #if AE_PAGED

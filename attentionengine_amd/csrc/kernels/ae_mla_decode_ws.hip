@@ -187,7 +187,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     ae_lds_byte* prow;
     ae_lds_byte* xb;
     // start of the softmax of tile tp: scores beyond the end of the range are taken out (ragged tail only)
-    auto soft_begin = [&](int tp) {
+    auto soft_begin = [&](int tp) AE_LAMBDA {
       // (xs holds raw scores: the scale is folded into the exponent; the softmax works on it in place)
       const bool tail = kv_begin + tp * AE_BN + AE_BN > kv_end;
       if (__builtin_expect(tail, 0)) {
@@ -204,7 +204,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
       xb = xbuf + (tp & 1) * AE_X_BYTES;
     };
     // the softmax of one tile in AE_NKS pieces, piece f issued behind the MFMA of k-step f
-    auto soft_slot = [&](int f) {
+    auto soft_slot = [&](int f) AE_LAMBDA {
       if (f < 4) {
         mx = __builtin_fmaxf(__builtin_fmaxf(mx, xs[4 * f]), xs[4 * f + 1]);
         mx = __builtin_fmaxf(__builtin_fmaxf(mx, xs[4 * f + 2]), xs[4 * f + 3]);
@@ -236,14 +236,14 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     };
     static_assert(AE_NKS >= 27, "the softmax of a tile is spread over 27 k-steps");
     // S^T of tile tn into xs; with SOFT the softmax of tile tn - 1 rides along
-    auto score_trip = [&](int tn, auto with_soft) {
+    auto score_trip = [&](int tn, auto with_soft) AE_LAMBDA {
       constexpr bool SOFT = decltype(with_soft)::value;
       int ka[4];
 #pragma unroll
       for (int i = 0; i < 4; i++) ka[i] = k_base[i] + (tn % AE_NSTAGE) * AE_STAGE_BYTES;
       // read AE_AHEAD fragments before the MFMA that uses them (the compiler on its own keeps one read
       // in flight, which leaves the LDS latency exposed)
-      auto read_kfrag = [&](int ks) -> ae_elem8 {
+      auto read_kfrag = [&](int ks) AE_LAMBDA -> ae_elem8 {
         return *(const __attribute__((address_space(3))) ae_elem8*)(lds + ka[ks & 3] + (ks >> 2) * 128);
       };
       ae_elem8 ring[AE_RING];
@@ -340,7 +340,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   }
 #endif
   // requests are made for t = 0, 1, 2, ... in this order
-  auto load_tile = [&](int t_) {
+  auto load_tile = [&](int t_) AE_LAMBDA {
     const int t = __builtin_amdgcn_readfirstlane(t_);
     int tt = t < n_tiles ? t : n_tiles - 1;
     tt = tt < 0 ? 0 : tt;
@@ -358,7 +358,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     const char* tile2 = (const char*)k2 + ((int64_t)page * p.k2_stride_b + (int64_t)in_page * p.k2_stride_s) * 2;
 #endif
     // the lane's source of load j in this tile
-    auto source = [&](int j) -> const char* {
+    auto source = [&](int j) AE_LAMBDA -> const char* {
 #if AE_PAGED
       return (((ld_rope >> j) & 1u) ? tile2 : tile1) + (int64_t)ld_off[j];
 #else
@@ -396,7 +396,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   };
   // end of a trip: tile t+2 has landed when only the newest request is outstanding; after the barrier
   // everyone is done with tile t, whose stage takes the next request
-  auto end_trip = [&](int t) {
+  auto end_trip = [&](int t) AE_LAMBDA {
     __builtin_amdgcn_s_waitcnt(AE_VMCNT_LGKM0(AE_LOADS));   // ... and this trip's LDS reads have returned
     __syncthreads();
     load_tile(t + AE_NSTAGE);
@@ -433,7 +433,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
       v_base[par][rg] = r * AE_KSTR + ((((4 * par + v_c0) ^ AE_SWZ(r)) + 4 * AE_NDB * dvw) << 4) + v_half;
     }
   static_assert(AE_NDB % 2 == 0, "a value wave's first chunk must be a multiple of eight");
-  auto read_vfrag = [&](const int (&va)[2][2], int kk, int db) -> ae_elem8 {
+  auto read_vfrag = [&](const int (&va)[2][2], int kk, int db) AE_LAMBDA -> ae_elem8 {
     const int imm = 16 * kk * AE_KSTR + (db >> 1) * 128;
     ae_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) ae_s16x4*)(
         lds + va[db & 1][0] + imm));
@@ -448,7 +448,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   ae_elem8 vreg[2 * AE_NDB];     // fragment f = (k-step f / AE_NDB, dv block f % AE_NDB)
 #pragma unroll
   for (int f = 0; f < 2 * AE_NDB; f++) vreg[f] = (ae_elem8){};
-  auto value_trip = [&](int n, auto with_pv, auto with_rd) {
+  auto value_trip = [&](int n, auto with_pv, auto with_rd) AE_LAMBDA {
     constexpr bool PV = decltype(with_pv)::value;
     constexpr bool RD = decltype(with_rd)::value;
     int va[2][2];          // the lane's four fragment offsets inside tile n - 1's stage

@@ -75,7 +75,6 @@
 #define AE_VCPR (AE_DV / 8)
 #define AE_K_LOADS ((AE_BN * AE_KCPR) / AE_NT)   // direct loads per lane per K tile
 #define AE_V_LOADS ((AE_BN * AE_VCPR) / AE_NT)
-#define AE_K_RPI (64 / AE_KCPR)   // K rows one wave instruction (64 lanes x 16 B) covers
 #define AE_V_RPI (64 / AE_VCPR)
 #define AE_VPPR (AE_VCPR / 2)     // 32-byte pairs per V row
 // the pairs of a V row are exchanged by the row's low bits: at most three of them, so that rows 8 apart (the
@@ -88,10 +87,27 @@ static_assert(AE_BN % 32 == 0, "kv tile must be a multiple of 32");
 static_assert((AE_BN * AE_KCPR) % AE_NT == 0, "K tile must split evenly over the workgroup");
 static_assert((AE_BN * AE_VCPR) % AE_NT == 0, "V tile must split evenly over the workgroup");
 static_assert(AE_K_LOADS >= 1 && AE_K_LOADS <= 8 && AE_V_LOADS >= 1 && AE_V_LOADS <= 8, "one burst per tile and wave");
-static_assert(AE_KCPR == 8 || AE_KCPR == 16 || AE_KCPR == 32, "swizzle is written for 128-, 256- or 512-byte K rows");
+static_assert(AE_KCPR == 8 || AE_KCPR == 16 || AE_KCPR == 32 || AE_KCPR % 8 == 4 || AE_KCPR % 16 == 8,
+              "swizzle is written for K rows of 128, 256 or 512 bytes, or an odd multiple of 64 or 128 bytes");
 static_assert(AE_VCPR == 8 || AE_VCPR == 16 || AE_VCPR == 32 || AE_VCPR == 64, "swizzle is written for 128- to 1024-byte V rows");
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
+
+// LDS chunk of K row `row` that holds global chunk c (and the other way round: an involution).  A fragment read
+// (ds_read_b128) takes one chunk index of 16 consecutive rows; they must fall into 16 different groups of four
+// banks.  Rows of a power-of-two length all start in the same group, so the chunk index is exchanged by the row
+// number.  Rows of 8*odd chunks (head dim 192: 384 bytes) start in two alternating groups and rows of 4*odd
+// chunks (head dims 96, 160) in four, so only the low three (two) bits of the chunk index are exchanged, by the
+// row number without the bits that the row pitch already spreads.
+AE_DEV int ae_k_swz(int c, int row) {
+#if (AE_KCPR & (AE_KCPR - 1)) == 0
+  return c ^ (row & (AE_KCPR - 1));
+#elif AE_KCPR % 16 == 8
+  return c ^ ((row >> 1) & 7);
+#else
+  return c ^ ((row >> 2) & 3);
+#endif
+}
 
 extern "C" __global__ __launch_bounds__(AE_NT)
 __attribute__((amdgpu_waves_per_eu(AE_WAVES_PER_EU, AE_WAVES_PER_EU)))
@@ -180,7 +196,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int bm_r0 = q0 / p.mask_block_m;
   int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
   bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
-  auto tile_class = [&](int j) -> int {
+  auto tile_class = [&](int j) AE_LAMBDA -> int {
     const int col = (j * AE_BN) / p.mask_block_n;
     int any = 0, all = 2;
     for (int r = bm_r0; r <= bm_r1; r++) {
@@ -196,19 +212,21 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
   const ae_elem* vbase = (const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)hk * p.v_stride_h;
 
-  // Direct HBM -> LDS tile load.  Wave w, instruction i covers rows (w*LOADS + i)*RPI ...+RPI-1;
-  // lane L lands in LDS chunk c' = L % CPR of row (L / CPR) and fetches the permuted global chunk.
+  // Direct HBM -> LDS tile load.  Wave w, instruction i covers the 64 consecutive 16-byte chunks
+  // (w*LOADS + i)*64 ... of the tile (whole rows when the row length is a power of two); lane L lands in LDS
+  // chunk c' of row r, (w*LOADS + i)*64 + L = r*CPR + c', and fetches the permuted global chunk.
   // A lane's byte offset inside a tile never changes, so it is computed once; per tile only a
   // wave-uniform base moves.  The K loads and the V loads of a wave each go out as one burst behind a
   // single write of M0 (see ae_load_lds16_burst_base: bases are passed 4 KiB low and the offsets 4 KiB
   // high, so that the offsets, which carry the compensation for the immediate offsets, stay >= 0).
-  auto k_lane_off = [&](int i, int last_row) -> unsigned {
-    int row = (wave * AE_K_LOADS + i) * AE_K_RPI + lane / AE_KCPR;
-    const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
+  auto k_lane_off = [&](int i, int last_row) AE_LAMBDA -> unsigned {
+    const int chunk = (wave * AE_K_LOADS + i) * 64 + lane;     // of the tile, in LDS order
+    int row = chunk / AE_KCPR;
+    const int c = ae_k_swz(chunk % AE_KCPR, row);
     row = row < last_row ? row : last_row;
     return (unsigned)((row * (int)p.k_stride_s + c * 8) * 2 + 4096 - (i - AE_K_LOADS / 2) * 1024);
   };
-  auto v_lane_off = [&](int i, int last_row) -> unsigned {
+  auto v_lane_off = [&](int i, int last_row) AE_LAMBDA -> unsigned {
     int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
     const int cp = lane % AE_VCPR;
     const int c = (((cp >> 1) ^ (row & AE_VSWM)) << 1) | (cp & 1);
@@ -220,7 +238,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   for (int i = 0; i < AE_K_LOADS; i++) koff[i] = k_lane_off(i, AE_BN);
 #pragma unroll
   for (int i = 0; i < AE_V_LOADS; i++) voff[i] = v_lane_off(i, AE_BN);
-  auto load_tile = [&](int j, int stage) {
+  auto load_tile = [&](int j, int stage) AE_LAMBDA {
     ae_lds_byte* ks = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* vs = ks + AE_K_BYTES;
     const char* gk = (const char*)kbase + (int64_t)j * AE_BN * p.k_stride_s * 2 - 4096;
@@ -242,7 +260,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     ae_load_lds16_burst_base<AE_V_LOADS>(gv, vo, vs + (wave * AE_V_LOADS + AE_V_LOADS / 2) * 1024);
   };
   // next tile index >= j that has work (block table) or j itself
-  auto next_tile = [&](int j) {
+  auto next_tile = [&](int j) AE_LAMBDA {
 #if AE_MASK_MODE == 2
     while (j < j_end && AE_TILE_CLASS(j) == 0) j++;
 #endif
@@ -271,7 +289,6 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // lane-constant pieces of the swizzled LDS read addresses
   // K fragment (row l32 of a 32-row block, d chunk 2*ks+hf): chunk' = (2*ks+hf) ^ (l32 mod CPR)
   const int k_row_off = l32 * AE_KSTR;
-  const int k_sw = l32 & (AE_KCPR - 1);
   // V transpose read: lane i of a 16-lane group reads row 4*hf + i/4 (+8), 8 bytes at pair
   // (2*db + g) ^ (row mod PPR), g = (lane%32)/16; rows of one group differ only in their low bits
   const int v_row = 4 * hf + ((lane & 15) >> 2);
@@ -337,7 +354,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int nb = 0; nb < AE_NB; nb++) {
         ae_elem8 kf = *(__attribute__((address_space(3))) ae_elem8*)(
-            ks_ + k_row_off + nb * 32 * AE_KSTR + (((2 * ks + hf) ^ k_sw) << 4));
+            ks_ + k_row_off + nb * 32 * AE_KSTR + (ae_k_swz(2 * ks + hf, l32) << 4));
 #pragma unroll
         for (int rb = 0; rb < AE_RB; rb++) sacc[rb][nb] = ae_mfma32(kf, qf[rb][ks], sacc[rb][nb]);
       }

@@ -217,11 +217,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #else
   const int n_items = n_t * group;
 #endif
-  auto item_tile = [&](int x) { return t_lo + (AE_BWD_ROLE == 0 ? x : x % n_t); };
-  auto item_head = [&](int x) { return AE_BWD_ROLE == 0 ? h : h * group + x / n_t; };   // q head of the item
+  auto item_tile = [&](int x) AE_LAMBDA { return t_lo + (AE_BWD_ROLE == 0 ? x : x % n_t); };
+  auto item_head = [&](int x) AE_LAMBDA { return AE_BWD_ROLE == 0 ? h : h * group + x / n_t; };   // q head of the item
 #if AE_MASK_MODE == 2
   // class of item x for this workgroup's resident tile
-  auto item_class = [&](int x) -> int {
+  auto item_class = [&](int x) AE_LAMBDA -> int {
     const int hq = item_head(x), t = item_tile(x);
     const int64_t mbh = (int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : hq);
 #if AE_BWD_ROLE == 0
@@ -232,7 +232,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   };
 #endif
   // first item at or after x that has anything visible (n_items if none)
-  auto next_item = [&](int x) {
+  auto next_item = [&](int x) AE_LAMBDA {
 #if AE_MASK_MODE == 2
     while (x < n_items && item_class(x) == 0) x++;
 #endif
@@ -245,14 +245,14 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   // one burst behind a single write of M0 (wave-uniform base + per-lane offset + immediate, see
   // ae_load_lds16_burst_base: bases are passed 4 KiB low and offsets 4 KiB high).  Rows past the end of
   // the sequence re-read its last row (they are masked).
-  auto lane_off1 = [&](int i, int last_row, int64_t st) -> unsigned {
+  auto lane_off1 = [&](int i, int last_row, int64_t st) AE_LAMBDA -> unsigned {
     const int sidx = (wave * AE_L1 + i) * 64 + lane;
     int r = sidx / AE_CPR1;
     const int c = ae_bwd_chunk_pos<AE_CPR1>(r, sidx % AE_CPR1);
     r = r < last_row ? r : last_row;
     return (unsigned)((r * (int)st + c * 8) * 2 + 4096 - (i - AE_L1 / 2) * 1024);
   };
-  auto lane_off2 = [&](int i, int last_row, int64_t st) -> unsigned {
+  auto lane_off2 = [&](int i, int last_row, int64_t st) AE_LAMBDA -> unsigned {
     const int sidx = (wave * AE_L2 + i) * 64 + lane;
     int r = sidx / AE_CPR2;
     const int c = ae_bwd_chunk_pos<AE_CPR2>(r, sidx % AE_CPR2);
@@ -270,7 +270,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #pragma unroll
   for (int i = 0; i < AE_L2; i++) off2[i] = lane_off2(i, AE_BS, st2);
   // request item x (past the end: the last item again, so that every call issues AE_NLOADS loads) into `stage`
-  auto request_item = [&](int x, int stage) {
+  auto request_item = [&](int x, int stage) AE_LAMBDA {
     const int itc = x < n_items ? x : n_items - 1;
     const int s0 = item_tile(itc) * AE_BS;
     ae_lds_byte* t1 = lds + stage * AE_STAGE_BYTES;
@@ -314,11 +314,11 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   };
 
   // A operands out of a staged tile.  Row fragment: A[m = row 32*nb + lane%32][k = 16*ks + 8*hf + j].
-  auto row_frag1 = [&](const ae_lds_byte* t, int nb, int ks) -> ae_elem8 {
+  auto row_frag1 = [&](const ae_lds_byte* t, int nb, int ks) AE_LAMBDA -> ae_elem8 {
     const int r = nb * 32 + l32;
     return *(const __attribute__((address_space(3))) ae_elem8*)(t + r * AE_STR1 + ae_bwd_chunk_pos<AE_CPR1>(r, 2 * ks + hf) * 16);
   };
-  auto row_frag2 = [&](const ae_lds_byte* t, int nb, int ks) -> ae_elem8 {
+  auto row_frag2 = [&](const ae_lds_byte* t, int nb, int ks) AE_LAMBDA -> ae_elem8 {
     const int r = nb * 32 + l32;
     return *(const __attribute__((address_space(3))) ae_elem8*)(t + r * AE_STR2 + ae_bwd_chunk_pos<AE_CPR2>(r, 2 * ks + hf) * 16);
   };
@@ -326,7 +326,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   // a lane's accumulator registers hold the rows (see the forward kernels' V^T fragment).
   const int t_row = 4 * hf + ((lane & 15) >> 2);
   const int t_g = l32 >> 4;
-  auto tr_frag = [&](const ae_lds_byte* t, int str, int cpr, int kk, int db) -> ae_elem8 {
+  auto tr_frag = [&](const ae_lds_byte* t, int str, int cpr, int kk, int db) AE_LAMBDA -> ae_elem8 {
     const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
     const int r_lo = rb0 + t_row, r_hi = r_lo + 8;
     const int sh = cpr == 16 ? 3 : 2;
@@ -396,7 +396,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #if AE_MASK_MODE == 1
     need_vis = need_vis || (AE_BWD_ROLE == 0 ? s0 + AE_BS - 1 > r0w : s0 < r0w + 31);
 #endif
-    auto block = [&](int nb, auto masked) {
+    auto block = [&](int nb, auto masked) AE_LAMBDA {
       ae_f32x16 sacc, pacc;
 #pragma unroll
       for (int r = 0; r < 16; r++) sacc[r] = pacc[r] = 0.f;
@@ -404,7 +404,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       // fragments are read AE_AHEAD MFMAs ahead of their use into a small ring, one fence per MFMA (left to
       // itself the scheduler either exposes the LDS latency or hoists every read and spills)
       constexpr int NF = AE_NKS1 + AE_NKS2;
-      auto frag = [&](int f) -> ae_elem8 {
+      auto frag = [&](int f) AE_LAMBDA -> ae_elem8 {
         // f even and S still has k-steps: S; else dP (the dims may differ)
         const int pairs = AE_NKS1 < AE_NKS2 ? AE_NKS1 : AE_NKS2;
         if (f < 2 * pairs) return (f & 1) ? row_frag2(t2, nb, f >> 1) : row_frag1(t1, nb, f >> 1);
@@ -492,7 +492,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     {
       constexpr int NB_OUT = AE_NDB1 + (AE_BWD_ROLE == 1 ? AE_NDB2 : 0);
       constexpr int NF = 4 * NB_OUT;
-      auto frag = [&](int f) -> ae_elem8 {
+      auto frag = [&](int f) AE_LAMBDA -> ae_elem8 {
         const int kk = f / NB_OUT, j = f % NB_OUT;
         return j < AE_NDB1 ? tr_frag(t1, AE_STR1, AE_CPR1, kk, j) : tr_frag(t2, AE_STR2, AE_CPR2, kk, j - AE_NDB1);
       };

@@ -190,7 +190,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int bm_r0 = q0 / p.mask_block_m;
   int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
   bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
-  auto tile_class = [&](int j) -> int {   // 0 skip, 1 elementwise mask, 2 fully visible
+  auto tile_class = [&](int j) AE_LAMBDA -> int {   // 0 skip, 1 elementwise mask, 2 fully visible
     const int col = (j * AE_BN) / p.mask_block_n;
     int any = 0, all = 2;
     for (int r = bm_r0; r <= bm_r1; r++) {
@@ -201,14 +201,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
     return any == 0 ? 0 : (all == 2 ? 2 : 1);
   };
 #endif
-  auto next_tile = [&](int j) {
+  auto next_tile = [&](int j) AE_LAMBDA {
 #if AE_MASK_MODE == 2
     while (j < j_end && tile_class(j) == 0) j++;
 #endif
     return j < j_end ? j : j_end;
   };
   // does tile j need the elementwise mask for this wave's rows?
-  auto needs_mask = [&](int j) -> bool {
+  auto needs_mask = [&](int j) AE_LAMBDA -> bool {
     bool nm = false;
 #if AE_MASK_MODE == 1
     nm = j * AE_BN + AE_BN - 1 > q0w;
@@ -240,13 +240,13 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // A tile's loads go out as one burst behind a single write of M0 (see ae_load_lds16_burst; the offsets
   // carry the compensation for its immediate offsets).
   // (bases are passed 4 KiB low and the offsets 4 KiB high, so that the compensated offsets stay >= 0)
-  auto k_lane_off = [&](int i, int last_row) -> unsigned {
+  auto k_lane_off = [&](int i, int last_row) AE_LAMBDA -> unsigned {
     int row = (wave * AE_K_LOADS + i) * AE_K_RPI + lane / AE_KCPR;
     const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
     row = row < last_row ? row : last_row;
     return (unsigned)((row * (int)p.k_stride_s + c * 8) * 2 + 4096 - (i - AE_K_LOADS / 2) * 1024);
   };
-  auto v_lane_off = [&](int i, int last_row) -> unsigned {
+  auto v_lane_off = [&](int i, int last_row) AE_LAMBDA -> unsigned {
     int row = (wave * AE_V_LOADS + i) * AE_V_RPI + lane / AE_VCPR;
     const int cp = lane % AE_VCPR;
     const int c = (((cp >> 1) ^ (row & (AE_VPPR - 1))) << 1) | (cp & 1);
@@ -258,7 +258,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   for (int i = 0; i < AE_K_LOADS; i++) koff[i] = k_lane_off(i, AE_BN);
 #pragma unroll
   for (int i = 0; i < AE_V_LOADS; i++) voff[i] = v_lane_off(i, AE_BN);
-  auto load_k = [&](int j, int stage) {
+  auto load_k = [&](int j, int stage) AE_LAMBDA {
     const char* g = (const char*)kbase + (int64_t)j * AE_BN * p.k_stride_s * 2 - 4096;
     unsigned gp[8];
 #pragma unroll
@@ -273,7 +273,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     }
     ae_load_lds16_burst_base<AE_K_LOADS>(g, gp, lds + stage * AE_K_BYTES + (wave * AE_K_LOADS + AE_K_LOADS / 2) * 1024);
   };
-  auto load_v = [&](int j, int stage) {
+  auto load_v = [&](int j, int stage) AE_LAMBDA {
     const char* g = (const char*)vbase + (int64_t)j * AE_BN * p.v_stride_s * 2 - 4096;
     unsigned gp[8];
 #pragma unroll
@@ -306,7 +306,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
   for (int i = 0; i < 8; i++) zero8[i] = (ae_elem)0.f;
   // a value DEFINED by an MFMA lives in the accumulator file: splat(v) + 0*0
-  auto acc_splat = [&](float v) -> ae_f32x16 {
+  auto acc_splat = [&](float v) AE_LAMBDA -> ae_f32x16 {
     ae_f32x16 t;
 #pragma unroll
     for (int r = 0; r < 16; r++) t[r] = v;
@@ -339,12 +339,12 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int v_g = l32 >> 4;
 
   // K fragment f = (k-step f/2, kv block f%2); V^T fragment f = (k-step f/NDB, dv block f%NDB)
-  auto read_kfrag = [&](int f, const ae_lds_byte* kt) -> ae_elem8 {
+  auto read_kfrag = [&](int f, const ae_lds_byte* kt) AE_LAMBDA -> ae_elem8 {
     const int ks = f >> 1, nb = f & 1;
     return *(const __attribute__((address_space(3))) ae_elem8*)(
         kt + k_row_off + nb * 32 * AE_KSTR + (((2 * ks + hf) ^ k_sw) << 4));
   };
-  auto read_vfrag = [&](int f, const ae_lds_byte* vt) -> ae_elem8 {
+  auto read_vfrag = [&](int f, const ae_lds_byte* vt) AE_LAMBDA -> ae_elem8 {
     const int kk = f / AE_NDB, db = f % AE_NDB;
     const int rb0 = (kk >> 1) * 32 + (kk & 1) * 16;
     const ae_lds_byte* a0 = vt + v_row_off + rb0 * AE_VSTR + (((2 * db + v_g) ^ v_sw) << 5);
@@ -363,7 +363,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   float osc[2];             // factors of a pending rescale of O
 
   // read x out of its accumulators (q block qb, scores e0 .. e0+n-1) and track the maximum
-  auto read_scores = [&](int qb, int e0, int n) {
+  auto read_scores = [&](int qb, int e0, int n) AE_LAMBDA {
 #pragma unroll
     for (int e = e0; e < e0 + n; e++) {
       float x = sacc[e >> 4][qb][e & 15];
@@ -385,7 +385,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   int kv_lim = 0;       // elementwise kind, ragged kv: keys of the tile in sv at offsets >= kv_lim (lane-relative) are past the end
   float xa[32][2];
   float negm2[2] = {0.f, 0.f};
-  auto stage_a = [&](int u) {
+  auto stage_a = [&](int u) AE_LAMBDA {
     const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
 #if AE_PRESCALE || AE_PIPE_KIND == 1
     xa[u][0] = sv[qb][e];
@@ -395,7 +395,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     xa[u][1] = __builtin_fmaf(sv[qb][e + 1], AE_SM_SCALE * AE_LOG2E, negm2[qb]);
 #endif
   };
-  auto stage_b = [&](int u) {
+  auto stage_b = [&](int u) AE_LAMBDA {
 #if AE_PIPE_KIND == 1
     // (score_mod is fused into ae_online_fwd; the graph has neither row state nor an o_scale)
     ae_online_fwd<2>(xa[u], st[u & 1], ctx[u & 1], cust[u & 1]);
@@ -404,7 +404,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     xa[u][1] = ae_exp2(xa[u][1]);
 #endif
   };
-  auto stage_c = [&](int u) {
+  auto stage_c = [&](int u) AE_LAMBDA {
     const int qb = u & 1, e = (u >> 3) * 8 + ((u >> 1) & 3) * 2;
     typedef float ae_f32x2 __attribute__((ext_vector_type(2)));
     const ae_f32x2 x2 = {xa[u][0], xa[u][1]};
@@ -426,7 +426,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     rsum[qb] = __builtin_amdgcn_fdot2(hv, one, rsum[qb], false);
 #endif
   };
-  auto exp_slot = [&](int g) {      // the stages that belong to MFMA slot g of an iteration
+  auto exp_slot = [&](int g) AE_LAMBDA {      // the stages that belong to MFMA slot g of an iteration
 #pragma unroll
     for (int u = 0; u < 32; u++) {
       const int a = (u * AE_EXP_SPAN) / 32;
@@ -435,7 +435,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
       if (a == g) stage_a(u);
     }
   };
-  auto exp_all = [&]() {            // all stages back to back (no MFMA to hide behind)
+  auto exp_all = [&]() AE_LAMBDA {            // all stages back to back (no MFMA to hide behind)
 #pragma unroll
     for (int u = 0; u < 32; u++) stage_a(u);
 #pragma unroll
@@ -447,7 +447,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // row maxima against the (lazy) reference.  The common case ends after two exchanges and a ballot; a
   // row whose maximum exceeds its threshold moves its reference (cold path): sv is shifted, the
   // running sum rescaled here, O before the next iteration (rescale_o, outside the hot loop).
-  auto finish_scores = [&](int j) {
+  auto finish_scores = [&](int j) AE_LAMBDA {
     const int kvb = j * AE_BN + 4 * hf;
     if (needs_mask(j)) {
 #pragma unroll
@@ -552,7 +552,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   //              phase 1 multiplies K(n+1) (K stage (n+1)%2), phase 2 multiplies V(n) (V stage n%2).
   int n = 0;
   // first AE_AHEAD fragments of iteration n's stream: K(j1) if it has a next tile, else V(j0)
-  auto prefetch_ring = [&]() {
+  auto prefetch_ring = [&]() AE_LAMBDA {
     if (j1 < j_end) {
       const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
 #pragma unroll
@@ -568,7 +568,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #endif
   // HN: the wave multiplies a next tile of its own.  TL (only without HN): it has none, but the other waves
   // have, so it still requests its share of the tiles they need.
-  auto iteration = [&](auto has_next_tag, auto tail_loads_tag) {
+  auto iteration = [&](auto has_next_tag, auto tail_loads_tag) AE_LAMBDA {
     constexpr bool HN = decltype(has_next_tag)::value;
     constexpr bool TL = decltype(tail_loads_tag)::value;
     const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
@@ -585,7 +585,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     // fragment stream of this iteration: K fragments 0..NKF-1 (if HN) then V fragments
     constexpr int NF1 = HN ? AE_NKF : 0;
     constexpr int NF = NF1 + AE_NVF;
-    auto read_frag = [&](int f) -> ae_elem8 {
+    auto read_frag = [&](int f) AE_LAMBDA -> ae_elem8 {
       return f < NF1 ? read_kfrag(f, kt) : read_vfrag(f - NF1, vt);
     };
 #if !AE_TOP_PREFETCH
@@ -661,7 +661,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // The rescale of O (rare once the reference has settled) stays OUTSIDE the hot loop: inside it, O
   // would have to be reachable by VALU instructions on every iteration and the register allocator
   // then shuttles all 128 accumulator registers between the two register files per tile.
-  auto rescale_o = [&]() {
+  auto rescale_o = [&]() AE_LAMBDA {
 #pragma unroll
     for (int qb = 0; qb < 2; qb++)
 #pragma unroll
@@ -680,7 +680,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   };
 #if AE_MASK_MODE == 1
   // an iteration of a wave that is done with its own tiles: its share of the tile loads, and the barrier
-  auto drain = [&]() {
+  auto drain = [&]() AE_LAMBDA {
     const int j2 = next_tile(j1 + 1);
     const int j2l = j2 < j_end ? j2 : j_end - 1;
     load_k(j2l, n & 1);

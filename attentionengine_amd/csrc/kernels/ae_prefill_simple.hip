@@ -159,7 +159,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int bm_r0 = q0 / p.mask_block_m;
   int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
   bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
-  auto tile_class = [&](int j) -> int {
+  auto tile_class = [&](int j) AE_LAMBDA -> int {
     const int col = (j * AE_BN) / p.mask_block_n;
     int any = 0, all = 2;
     for (int r = bm_r0; r <= bm_r1; r++) {
@@ -178,7 +178,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   ae_u32x4 kreg[AE_K_LOADS];
   ae_u32x4 vreg[AE_V_LOADS];
 
-  auto load_tile = [&](int j) {
+  auto load_tile = [&](int j) AE_LAMBDA {
     const int kv0 = j * AE_BN;
 #pragma unroll
     for (int i = 0; i < AE_K_LOADS; i++) {
@@ -201,7 +201,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
       vreg[i] = *(const ae_u32x4*)(vbase + (int64_t)kv * p.v_stride_s + col * 8);
     }
   };
-  auto store_tile = [&](int stage) {
+  auto store_tile = [&](int stage) AE_LAMBDA {
     ae_lds_byte* ks = lds + stage * AE_STAGE_BYTES;
     ae_lds_byte* vs = ks + AE_K_BYTES;
 #pragma unroll
@@ -218,7 +218,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     }
   };
   // next tile index >= j that has work (block table) or j itself
-  auto next_tile = [&](int j) {
+  auto next_tile = [&](int j) AE_LAMBDA {
 #if AE_MASK_MODE == 2
     while (j < j_end && AE_TILE_CLASS(j) == 0) j++;
 #endif

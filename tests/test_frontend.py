@@ -508,7 +508,10 @@ def test_tuner_cache_records(tmp_path):
     assert len(cands) == 4 and cands[0].template == "ae_prefill_pipe.hip"
     assert len(tuner.prefill_candidates(128, 128, None, False)) == 3
     assert [c.block_n for c in tuner.prefill_candidates(256, 512, None, False)] == [32]
-    assert [c.block_n for c in tuner.prefill_candidates(192, 128, None, False)] == [32, 64]
+    assert [(c.waves_per_eu, c.block_n) for c in tuner.prefill_candidates(192, 128, None, False)] == \
+        [(2, 64), (2, 32), (1, 64), (1, 32)]
+    assert [(c.template, c.block_n) for c in tuner.prefill_candidates(192, 192, None, False)] == \
+        [("ae_prefill_simple.hip", 32), ("ae_prefill_simple.hip", 64)]
     tuner.store(f, pk, tuner.encode_tiles(cands[2]))
     tuner.store(f, {**pk, "batch": 4}, [128, 128, 2, 256, False])     # a record as the reference writes it
     recs = json.load(open(f))

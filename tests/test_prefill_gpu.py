@@ -467,6 +467,37 @@ def test_wide_head_dims_in_the_direct_to_lds_kernel(cuda_device, monkeypatch, B,
     assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
+@pytest.mark.parametrize("B,H,Hkv,Sq,Skv,D,DV,dtype,mask,waves", [
+    (1, 4, 4, 333, 333, 192, 128, torch.bfloat16, "causal", 2),    # 384-byte K rows: multi-head latent attention, prefill
+    (2, 4, 4, 456, 456, 192, 128, torch.float16, None, 2),
+    (1, 4, 2, 264, 264, 192, 128, torch.float16, "causal", 2),     # grouped heads
+    (1, 2, 2, 300, 300, 160, 128, torch.float16, "causal", 2),     # 320-byte K rows
+    (1, 2, 2, 257, 257, 96, 64, torch.bfloat16, "window", 2),      # 192-byte K rows, tile-class table + mask_mod
+    (1, 2, 2, 192, 192, 96, 128, torch.float16, "causal", 2),
+    (1, 2, 1, 200, 200, 192, 256, torch.float16, "causal", 1),     # with a wide value head: one wave per SIMD
+    (1, 2, 2, 130, 130, 160, 512, torch.bfloat16, None, 1),
+])
+def test_head_dims_whose_rows_are_not_a_power_of_two(cuda_device, B, H, Hkv, Sq, Skv, D, DV, dtype, mask, waves):
+    """Head dims 96, 160 and 192 in the direct-to-LDS kernel: K rows of 4*odd or 8*odd 16-byte chunks, fetched as
+    64 consecutive chunks per instruction whatever the row boundaries, swizzled by the row bits their pitch does
+    not already spread."""
+    print(f"case K rows B{B} H{H}/{Hkv} Sq{Sq} Skv{Skv} D{D} DV{DV} {dtype} {mask}", flush=True)
+    q, k, v = C.make_inputs(B, Sq, Skv, H, Hkv, D, DV, dtype, seed=9)
+    mask_mod = {None: None, "causal": C.causal_mask, "window": C.make_sliding_window_mask(100)}[mask]
+    meta = (meta_tensor(B, H, Sq, D, dtype=dtype), meta_tensor(B, Hkv, Skv, D, dtype=dtype),
+            meta_tensor(B, Hkv, Skv, DV, dtype=dtype))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod=mask_mod,
+                          online_func=C.OnlineSoftmax())
+    op = mod.attention
+    assert op.tiles.template == "ae_prefill.hip" and op.tiles.waves_per_eu == waves
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    mk = None if mask_mod is None else mask_mod(0, 0, torch.arange(Sq)[:, None], torch.arange(Skv)[None, :])[None, None]
+    ref, lse = R.softmax_attention(q, k, v, mask=mk)
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
 def test_pipelined_kernel_exact_scale_switch(cuda_device, monkeypatch):
     """AE_PREFILL_PRESCALE=0: the pipelined kernel leaves Q alone and scales every score in fp32; lse then
     holds 1e-3 (+ fp32 rounding) also for scores of size 60."""
