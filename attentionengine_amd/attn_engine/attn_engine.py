@@ -109,16 +109,18 @@ class AttentionEngine:
         # dynamic (string) extents are runtime parameters of the kernels; they only rule out the
         # shape-dependent dispatch to the decode templates
         dynamic = any(isinstance(d, str) for m in qkv_meta for d in m.shape)
+        decode_tune = {k: v for k, v in (tune or {}).items() if k in ("tune", "tune_file")}
 
         if kv_shared:
             from core.lower.lower_decode import MLADecodeOp
             return MLADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
-                               mask_value, cute_convention=(self.backend == "cute"))
+                               mask_value, cute_convention=(self.backend == "cute"), **decode_tune)
         if not dynamic and q_seqlen != kv_len and head > head_kv:
             assert q_seqlen < kv_len
             assert q_seqlen == 1
             from core.lower.lower_decode import GQADecodeOp
-            return GQADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value)
+            return GQADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
+                               **decode_tune)
         # MHA decode (attn_engine.py:273-290 of the reference): a few query tokens against a long KV,
         # split over the kv axis and merged with the user's combine()
         # (an online function that does not override combine() cannot merge splits: it runs unsplit)

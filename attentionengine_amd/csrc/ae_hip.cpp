@@ -477,6 +477,15 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
     if (p->kv_per_split % cfg->block_n != 0)
       return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: kv_per_split=%d is not a multiple of the %d-token kv tile",
                   p->kv_per_split, cfg->block_n);
+    // (the wave-specialised kernel keeps a split's part of the block table in LDS: AE_PTAB = 1024 entries)
+    if (p->kv_per_split / p->page_block_size + 2 > 1024)
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: a split of %d tokens spans more than 1022 pages of %d tokens "
+                                      "(use more splits)", p->kv_per_split, p->page_block_size);
+    // the paged kernels address the rope columns as an offset from the latent ones inside one cache tensor
+    if (p->k2 && (p->k2_stride_b != p->k_stride_b || p->k2_stride_s != p->k_stride_s || p->k2_stride_h != p->k_stride_h ||
+                  (const char*)p->k2 < (const char*)p->k || (const char*)p->k2 - (const char*)p->k > (1 << 20)))
+      return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: in a paged cache k2 must be a column range of the tensor k "
+                                      "(equal strides, at most 1 MiB behind it)");
   } else if (p->block_table || p->seqlens_k) {
     return fail(AE_ERR_INVALID_ARG, "ae_mla_decode_fwd: block_table / seqlens_k passed to a kernel built for a dense cache");
   }

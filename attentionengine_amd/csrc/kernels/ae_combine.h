@@ -11,12 +11,22 @@ void ae_decode_combine_kernel(const ae_attn_params p) {
   const int h = blockIdx.x;
   const int b = blockIdx.y;
   const int64_t row = ((int64_t)b * p.heads_q + h) * AE_NSPLIT;
+  // Paged cache (per-entry lengths): only the first ceil(length / kv_per_split) splits of an entry hold keys and
+  // wrote partial results; an entry with at most one wrote `out` itself.
+  int n_used = AE_NSPLIT;
+  if (p.seqlens_k != nullptr) {
+    int len = p.seqlens_k[b];
+    len = len < p.seqlen_kv ? len : p.seqlen_kv;
+    const int n = ((len > 0 ? len : 0) + p.kv_per_split - 1) / p.kv_per_split;
+    n_used = n < AE_NSPLIT ? n : AE_NSPLIT;
+    if (n_used <= 1) return;
+  }
   float rs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1][AE_NSPLIT];
 #pragma unroll
   for (int i = 0; i < AE_N_ROWSCALES; i++)
 #pragma unroll
     for (int k = 0; k < AE_NSPLIT; k++)
-      rs[i][k] = p.partial_rs[(int64_t)i * p.batch * p.heads_q * AE_NSPLIT + row + k];
+      rs[i][k] = k < n_used ? p.partial_rs[(int64_t)i * p.batch * p.heads_q * AE_NSPLIT + row + k] : AE_NEG_INF;
   float w[AE_NSPLIT];
   float merged[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
   ae_combine(rs, w, merged);
@@ -24,7 +34,8 @@ void ae_decode_combine_kernel(const ae_attn_params p) {
   for (int dv = threadIdx.x; dv < AE_DV; dv += AE_COMBINE_THREADS) {
     float acc = 0.f;
 #pragma unroll
-    for (int k = 0; k < AE_NSPLIT; k++) acc += p.partial_o[(row + k) * AE_DV + dv] * w[k];
+    for (int k = 0; k < AE_NSPLIT; k++)
+      if (k < n_used) acc += p.partial_o[(row + k) * AE_DV + dv] * w[k];
     optr[dv] = (ae_elem)acc;
   }
   if (threadIdx.x == 0) {

@@ -125,10 +125,21 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   kv_end = kv_end < seqlen_b ? kv_end : seqlen_b;
   const int n_tiles = kv_end > kv_begin ? (kv_end - kv_begin + AE_BN - 1) / AE_BN : 0;
 #if AE_PAGED
-  if (n_tiles == 0) {       // a split beyond this entry's length
-    ae_mla_write_no_keys(p, b, hk, ht, split, group, tid);
+  // a split beyond this entry's length writes nothing (the merge passes it over); split 0 of an entry of
+  // length 0 writes that entry's "no keys" result
+  if (n_tiles == 0) {
+    if (split == 0) ae_mla_write_no_keys(p, b, hk, ht, group, tid);
     return;
   }
+#endif
+  // who writes `out`: this workgroup (a launch without splits; a paged entry whose keys all lie in split 0), or the
+  // merge kernel from the splits' partial results
+#if AE_NSPLIT == 1
+  constexpr bool direct = true;
+#elif AE_PAGED
+  const bool direct = ae_mla_splits_used(p, seqlen_b) <= 1;
+#else
+  constexpr bool direct = false;
 #endif
 
   // Direct HBM -> LDS tile load.  Instruction i of wave w fills the 1 KiB block
@@ -295,9 +306,8 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
 #pragma unroll
     for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
   }
-#if AE_NSPLIT == 1
-  // a single split needs no merge: write the output row and its rowscales directly
-  if (head_ok) {
+  // no merge needed: write the output row and its rowscales directly
+  if (head_ok && direct) {
     ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)hq * p.o_stride_h +
                     dvh * (AE_DV / 2);
 #pragma unroll
@@ -313,8 +323,7 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         if (p.rowscale_out[i]) p.rowscale_out[i][(int64_t)b * p.heads_q + hq] = frs[i];
     }
   }
-#else
-  if (head_ok) {
+  if (head_ok && !direct) {
     const int64_t row = ((int64_t)b * p.heads_q + hq) * p.num_splits + split;
     float* po = p.partial_o + row * AE_DV + dvh * (AE_DV / 2);
 #pragma unroll
@@ -328,7 +337,6 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         p.partial_rs[(int64_t)i * p.batch * p.heads_q * p.num_splits + row] = frs[i];
     }
   }
-#endif
 }
 
 #include "ae_combine.h"

@@ -203,6 +203,8 @@ def test_mla_decode_cute_convention(cuda_device):
     (torch.bfloat16, 3, 128, 64, [1000, 37, 640], 256),    # split launch; entry 1 leaves most splits without a key
     (torch.float16, 2, 16, 32, [513, 2048], 1),            # one split, long loop, ragged tails, 16 of 64 head rows
     (torch.bfloat16, 2, 64, 128, [128, 1], 8),             # pages larger than a tile, a one-token entry
+    (torch.float16, 4, 64, 64, [700, 0, 64, 257], 64),     # split launch with an empty entry, entries of one split
+                                                           # (they write `out` themselves) and merged ones
 ])
 def test_mla_decode_paged_cache(cuda_device, monkeypatch, kernel, dtype, B, H, page, lens, target):
     """mod(q, kv_cache, block_table=..., cache_seqlens=...): pages in a shuffled order, every batch entry
@@ -237,6 +239,9 @@ def test_mla_decode_paged_cache(cuda_device, monkeypatch, kernel, dtype, B, H, p
     assert out.shape == (B, 1, H, DV) and lse.shape == (B, H, 1)
     for b in range(B):
         n = lens[b]
+        if n == 0:      # no key at all: zeros, lse -inf (cute_template/flash_fwd_kernel.h:180-183 of the reference)
+            assert (out[b] == 0).all() and (lse[b] == float("-inf")).all()
+            continue
         ref, lref = R.mla_decode(q[b:b + 1, 0], q_pe[b:b + 1, 0], kv[b:b + 1, :n], k_pe[b:b + 1, :n], scale=scale)
         assert (out[b:b + 1, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL, b
         assert (lse[b:b + 1, :, 0].cpu() - lref).abs().max().item() <= LSE_TOL, b
@@ -245,6 +250,56 @@ def test_mla_decode_paged_cache(cuda_device, monkeypatch, kernel, dtype, B, H, p
     out2, _ = mod(torch.cat([q, q_pe], -1).cuda(), dense[:, :n0].reshape(-1, page, G, D).contiguous().cuda())
     ref, _ = R.mla_decode(q[:, 0], q_pe[:, 0], kv[:, :n0], k_pe[:, :n0], scale=scale)
     assert (out2[:, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL
+
+
+def test_decode_split_counts_are_tuned_and_recorded(cuda_device, tmp_path):
+    """tune=True for the decode engines (the reference tunes num_split whenever it builds the MLA decode kernel,
+    mla_decode_tl.py:13-24, 308-319): the first call of a shape measures the planned split count, its half and its
+    multiples on the caller's tensors, records the fastest under the problem keys and uses it from then on; every
+    candidate computes the same result (checked here through the oracle on the winner and through the records)."""
+    import json
+    f = str(tmp_path / "splits.json")
+    # MLA, paged cache with very different lengths
+    B, H, G, D, DV, page, dtype = 8, 128, 1, 576, 512, 64, torch.bfloat16
+    lens = [2048, 64, 300, 1, 1024, 77, 512, 1999]
+    scale = 1 / math.sqrt(D)
+    max_pages = -(-max(lens) // page)
+    q, q_pe, kv, k_pe = _mla_inputs(B, H, G, max_pages * page, DV, D - DV, dtype, seed=9)
+    cache = torch.cat([kv, k_pe], -1).reshape(B * max_pages, page, G, D).contiguous()
+    table = torch.arange(B * max_pages, dtype=torch.int32).reshape(B, max_pages)
+    args = (torch.cat([q, q_pe], -1).cuda(), cache.cuda())
+    kw = dict(block_table=table.cuda(), cache_seqlens=torch.tensor(lens, dtype=torch.int32).cuda())
+    mod = _mla_engine(B, H, G, max_pages * page, D, DV, dtype, scale, backend="cute", tune=True, tune_file=f)
+    out, lse = mod(*args, **kw)
+    op = mod.attention
+    key = (B, H, G, max_pages * page)
+    assert len(op.tune_times) >= 3 and op._tuned[key] in op.tune_times
+    assert op.tune_times[op._tuned[key]] == min(op.tune_times.values())
+    (rec,) = json.load(open(f))
+    assert rec == {"batch": B, "heads": H, "seq_len": max_pages * page, "dim": D, "dimv": DV,
+                   "tuned_config": [op._tuned[key]]}
+    for b in range(B):
+        n = lens[b]
+        ref, lref = R.mla_decode(q[b:b + 1, 0], q_pe[b:b + 1, 0], kv[b:b + 1, :n], k_pe[b:b + 1, :n], scale=scale)
+        assert (out[b:b + 1, 0].float().cpu() - ref).abs().max().item() <= OUT_TOL, b
+        assert (lse[b:b + 1, :, 0].cpu() - lref).abs().max().item() <= LSE_TOL, b
+    again = _mla_engine(B, H, G, max_pages * page, D, DV, dtype, scale, backend="cute", tune=True, tune_file=f)
+    out2, lse2 = again(*args, **kw)
+    assert again.attention.tune_times is None and again.attention._tuned[key] == op._tuned[key]
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+    # GQA decode: same file, another problem
+    B, Hq, Hkv, Skv, D = 4, 32, 8, 4096, 128
+    qg, kg, vg = C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, torch.float16)
+    gqa = _decode_engine(B, Hq, Hkv, Skv, D, D, torch.float16, C.make_scale_score_mod(1 / math.sqrt(D)),
+                         C.OnlineSoftmax(), tune=True, tune_file=f)
+    og = gqa(qg.cuda(), kg.cuda(), vg.cuda())
+    ref, lref = R.softmax_attention(qg, kg, vg, causal=False)
+    assert (og.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    assert (gqa.final_rowscales["lse"].cpu() - lref).abs().max().item() <= LSE_TOL
+    assert len(gqa.attention.tune_times) >= 2
+    recs = json.load(open(f))
+    assert len(recs) == 2 and recs[1]["tuned_config"] == [gqa.attention._tuned[(B, Hq, Hkv, Skv)]]
 
 
 def _mha_decode_engine(B, H, Sq, Skv, D, dtype, online, mask_mod=None):
