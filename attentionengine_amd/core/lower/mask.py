@@ -114,6 +114,13 @@ class MaskPlan:
         self.block_m = block_m
         self.block_n = block_n
         self.elementwise = elementwise
+        # late q tiles visit clearly more kv tiles than early ones (causal variants, long sliding windows): the
+        # kernels then start the long q tiles first
+        self.heavy_last = False
+        if table is not None and table.shape[2] >= 4:
+            work = (table > 0).sum(dim=-1).to(torch.float32).mean(dim=(0, 1))
+            third = table.shape[2] // 3
+            self.heavy_last = bool(work[-third:].mean() >= 1.25 * work[:third].mean())
 
 
 def plan_mask(mask_mod, lowered: LoweredMask, B: int, H: int, Sq: int, Skv: int, tile_m: int,

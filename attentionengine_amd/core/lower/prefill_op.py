@@ -23,6 +23,8 @@ def _dim(x, default):
 
 
 class PrefillOp:
+    MASK_ROWS_PER_TILE = 8      # block-mask rows one q tile may span (AE_TT_ROWS of csrc/kernels/ae_tile_table.h)
+
     def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
                  extern_block_mask=False, split_kv=False, target_workgroups=512,
@@ -67,6 +69,13 @@ class PrefillOp:
                                             self._pipe_softmax,
                                             _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1),
                                             elementwise=self._pipe_elementwise)
+        # Masks that reach the kernel as a tile table (anything but none / exactly causal) go to the generic
+        # kernel: with its 128-row q tiles fewer tiles are partly visible, and its masked path costs less than
+        # the pipelined kernel's (B2 H32 S4096 D128, sliding window of 256: 0.13 against 0.31 ms; a random block
+        # mask that keeps 27 %: 0.22 against 0.35 ms).  tune=True still measures both.
+        if self.tiles.rows_per_wave == 64 and os.environ.get("AE_PREFILL_KERNEL", "") != "pipelined" and (
+                self.extern_block_mask or (mask_mod is not None and self._probe_mask_mode(q_meta, v_meta) == 2)):
+            self.tiles = L.PrefillTiles()
         # tune=True (attn_tl.py:465-521 of the reference): the tile configuration comes from the record of
         # this problem in tune_file, or is measured at the first call and recorded there.  Launches whose
         # tiles are bound to something else (split-KV, an external block mask) keep the fixed choice.
@@ -106,8 +115,11 @@ class PrefillOp:
             # a q tile covers whole block-mask rows, a kv tile sits inside one block-mask column
             while self.tiles.block_n > self.mask_block[1] and self.tiles.block_n > 32:
                 self.tiles.block_n //= 2
+            if self.tiles.block_m > self.MASK_ROWS_PER_TILE * self.mask_block[0]:
+                self.tiles = L.PrefillTiles(block_n=self.tiles.block_n)   # 128-row q tiles span fewer table rows
             if (self.tiles.block_m % self.mask_block[0] and self.mask_block[0] % self.tiles.block_m) or \
-                    self.mask_block[1] % self.tiles.block_n:
+                    self.mask_block[1] % self.tiles.block_n or \
+                    self.tiles.block_m > self.MASK_ROWS_PER_TILE * self.mask_block[0]:
                 raise NotImplementedError(f"block mask granularity {self.mask_block} does not fit the tiles")
         self.n_rowscales = len(self.functors.final_rowscale_names)
         if self.n_rowscales > rt.AE_MAX_ROWSCALES or len(self.functors.customs) > rt.AE_MAX_CUSTOM:
@@ -126,10 +138,19 @@ class PrefillOp:
             plan = self._plan(B, H, Sq, Skv, device=None)
             mode = 2 if self.extern_block_mask else plan.mode
             n_split, _ = self.plan_splits(B, H, Sq, Skv)
-            _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split)
+            _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split,
+                                          self._table_rows(self.mask_block[0] if self.extern_block_mask else plan.block_m),
+                                          plan.heavy_last and not self.extern_block_mask)
             self.source = cfg_src + "\n" + self.functor_src
             if infer_mask and mask_mod is not None and not self.extern_block_mask:
                 self.block_mask = self._reference_block_mask(B, H, Sq, Skv)
+
+    def _probe_mask_mode(self, q_meta, v_meta):
+        """Mode of the mask plan at the declared sequence lengths (4096 where they are dynamic), for batch entry
+        and head 0: 2 = the mask needs a tile table."""
+        sq, skv = _dim(q_meta.shape[2], 4096), _dim(v_meta.shape[2], 4096)
+        return plan_mask(self.mask_mod, self.functors.mask, 1, 1, sq, skv, 128, 64,
+                         elementwise=self.elementwise_mask).mode
 
     # ---- tuning ------------------------------------------------------------------------
     def _tune_candidates(self):
@@ -217,8 +238,17 @@ class PrefillOp:
             return 0
         return self.tiles.n_waves * (self.tiles.rows_per_wave // 32) * 2560
 
-    def _variant(self, mask_mode, even_q, even_kv, n_split=1):
-        key = (mask_mode, even_q, even_kv, n_split)
+    def _table_rows(self, mask_block_m):
+        """Block-table rows a q tile spans (1, 2, 4 or 8): the kernels keep that many pairs of 64-bit masks."""
+        if not mask_block_m:
+            return 1
+        rows = max(1, -(-self.tiles.block_m // int(mask_block_m)))
+        return next(r for r in (1, 2, 4, 8) if r >= min(rows, 8))
+
+    def _variant(self, mask_mode, even_q, even_kv, n_split=1, table_rows=1, heavy_last=False):
+        if mask_mode != 2:
+            table_rows, heavy_last = 1, False
+        key = (mask_mode, even_q, even_kv, n_split, table_rows, bool(heavy_last))
         v = self._variants.get(key)
         if v is None:
             has_mask_mod = self.elementwise_mask and mask_mode != 1
@@ -228,6 +258,8 @@ class PrefillOp:
                                       elementwise=self._pipe_elementwise and self.tiles.rows_per_wave == 64)
             if self.mask_value_zero:
                 cfg_src += "#define AE_MASK_VALUE_ZERO 1\n"
+            if mask_mode == 2:
+                cfg_src += f"#define AE_TT_ROWS {table_rows}\n#define AE_HEAVY_LAST {1 if heavy_last else 0}\n"
             if n_split > 1:
                 cfg_src += f"#define AE_NSPLIT {n_split}\n#define AE_COMBINE_THREADS {self.COMBINE_THREADS}\n"
             module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,
@@ -287,7 +319,8 @@ class PrefillOp:
             extern_mask = None
         if extern_mask is not None:
             bm, bn = self.mask_block
-            if bn % self.tiles.block_n or (self.tiles.block_m % bm and bm % self.tiles.block_m):
+            if bn % self.tiles.block_n or (self.tiles.block_m % bm and bm % self.tiles.block_m) or \
+                    self.tiles.block_m > self.MASK_ROWS_PER_TILE * bm:
                 raise NotImplementedError(
                     f"a block mask of {bm}x{bn} blocks does not fit the kernel's {self.tiles.block_m}x"
                     f"{self.tiles.block_n} tiles (construct the engine with extern_block_mask=True)")
@@ -302,7 +335,9 @@ class PrefillOp:
             plan = self._plan(B, Hq, Sq, Skv, dev)
             mode, table, mbm, mbn = plan.mode, plan.table, plan.block_m, plan.block_n
         n_split, kv_per_split = self.plan_splits(B, Hq, Sq, Skv)
-        module, cfg, _ = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split)
+        module, cfg, _ = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split,
+                                       self._table_rows(mbm) if mode == 2 else 1,
+                                       extern_mask is None and plan.heavy_last)
         kern = module.kernel("ae_prefill_kernel")
 
         out = torch.empty((B, Sq, Hq, self.DV), dtype=self.dtype, device=dev)

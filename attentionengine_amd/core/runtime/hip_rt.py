@@ -305,6 +305,7 @@ def compile_module(template: str, headers: dict, arch: str = None, use_cache: bo
         "ae_device.h": _read(osp.join(KERNEL_DIR, "ae_device.h")),
         "ae_combine.h": _read(osp.join(KERNEL_DIR, "ae_combine.h")),
         "ae_mla_paged.h": _read(osp.join(KERNEL_DIR, "ae_mla_paged.h")),
+        "ae_tile_table.h": _read(osp.join(KERNEL_DIR, "ae_tile_table.h")),
     }
     all_headers.update(headers)
     hsh = hashlib.sha256()

@@ -52,6 +52,9 @@
 #include "ae_config.h"
 #include "ae_device.h"
 #include "ae_functors.h"
+#ifndef AE_HEAVY_LAST
+#define AE_HEAVY_LAST 0
+#endif
 
 #ifndef AE_BWD_NWAVES
 #define AE_BWD_NWAVES 4             // waves per workgroup, 32 resident rows each
@@ -150,7 +153,9 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   const int n_bg = (n_bh + 7) >> 3;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int bh = (slot % n_bg) * 8 + xcd;
-#if AE_BWD_ROLE == 0 && AE_MASK_MODE == 1
+#if AE_BWD_ROLE == 0 && (AE_MASK_MODE == 1 || (AE_MASK_MODE == 2 && AE_HEAVY_LAST))
+  // (the q tiles with the most visible keys first: the last ones under a causal mask, and under a tile table
+  // that the host found to be heavier towards the end - AE_HEAVY_LAST)
   const int rt = n_rt - 1 - slot / n_bg;
 #else
   const int rt = slot / n_bg;
@@ -220,21 +225,44 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   auto item_tile = [&](int x) AE_LAMBDA { return t_lo + (AE_BWD_ROLE == 0 ? x : x % n_t); };
   auto item_head = [&](int x) AE_LAMBDA { return AE_BWD_ROLE == 0 ? h : h * group + x / n_t; };   // q head of the item
 #if AE_MASK_MODE == 2
-  // class of item x for this workgroup's resident tile
-  auto item_class = [&](int x) AE_LAMBDA -> int {
-    const int hq = item_head(x), t = item_tile(x);
-    const int64_t mbh = (int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : hq);
+  // Classes of the items from the tile table of this launch (0 = nothing visible, 1 = test every element,
+  // 2 = all visible), 64 items at a time: lane l reads the class of item c0 + l and two ballots keep "visible"
+  // and "fully visible" as 64-bit masks in scalar registers.  Reading the table item by item inside the loop
+  // would cost a dependent memory access per skipped item, and, behind the tile requests' asm statements, a
+  // vector load whose wait (vmcnt(0)) also waits for every tile in flight.
+  int im_c0 = -64;
+  unsigned long im_vis = 0, im_full = 0;
+  auto item_masks = [&](int c0) AE_LAMBDA {
+    const int x = c0 + lane;
+    int c = 0;
+    if (x < n_items) {
+      const int hq = item_head(x), t = item_tile(x);
+      const int64_t mbh = (int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : hq);
 #if AE_BWD_ROLE == 0
-    return p.mask_dq[(mbh * n_rt + rt) * n_st + t];            // [q tiles of 128][kv tiles of 64]
+      c = p.mask_dq[(mbh * n_rt + rt) * n_st + t];            // [q tiles of 128][kv tiles of 64]
 #else
-    return p.mask_dkv[(mbh * n_st + t) * n_rt + rt];           // [q tiles of 64][kv tiles of 128]
+      c = p.mask_dkv[(mbh * n_st + t) * n_rt + rt];           // [q tiles of 64][kv tiles of 128]
 #endif
+    }
+    im_vis = __builtin_amdgcn_ballot_w64(c != 0);
+    im_full = __builtin_amdgcn_ballot_w64(c == 2);
+    im_c0 = c0;
   };
 #endif
-  // first item at or after x that has anything visible (n_items if none)
-  auto next_item = [&](int x) AE_LAMBDA {
+  // first item at or after x that has anything visible (n_items if none), and its class
+  auto next_item = [&](int x, int& cls) AE_LAMBDA {
+    cls = 2;
 #if AE_MASK_MODE == 2
-    while (x < n_items && item_class(x) == 0) x++;
+    while (x < n_items) {
+      if (x < im_c0 || x >= im_c0 + 64) item_masks(x & ~63);
+      const unsigned long m = im_vis >> (x - im_c0);
+      if (m != 0) {
+        x += __builtin_ctzl(m);
+        cls = ((im_full >> (x - im_c0)) & 1ul) ? 2 : 1;
+        break;
+      }
+      x = im_c0 + 64;
+    }
 #endif
     return x < n_items ? x : n_items;
   };
@@ -352,7 +380,8 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #endif
 
   // the n-th visited item is multiplied out of stage n % NSTAGE while the next two are on their way
-  int x0 = next_item(0), x1 = next_item(x0 + 1), x2 = next_item(x1 + 1);
+  int cls0, cls1, cls2;                 // ... and the classes of those three items
+  int x0 = next_item(0, cls0), x1 = next_item(x0 + 1, cls1), x2 = next_item(x1 + 1, cls2);
   if (x0 < n_items) {
     request_item(x0, 0);
     if (AE_NSTAGE == 3) request_item(x1, 1);
@@ -389,7 +418,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     // only tiles that touch the diagonal, the end of a sequence or an elementwise mask test visibility
     const int r0w = r0 + wave * 32;
 #if AE_MASK_MODE == 2
-    bool need_vis = item_class(it) != 2 || s0 + AE_BS > n_str || r0w + 32 > n_res;
+    bool need_vis = cls0 != 2 || s0 + AE_BS > n_str || r0w + 32 > n_res;
 #else
     bool need_vis = (AE_HAS_MASK_MOD != 0) || s0 + AE_BS > n_str || r0w + 32 > n_res;
 #endif
@@ -519,9 +548,9 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     // the next item has landed (with three stages the one after it is still outstanding)
     __builtin_amdgcn_s_waitcnt(AE_VMCNT((AE_NSTAGE - 2) * AE_NLOADS));
     __syncthreads();
-    x0 = x1;
-    x1 = x2;
-    x2 = next_item(x2 + 1);
+    x0 = x1, cls0 = cls1;
+    x1 = x2, cls1 = cls2;
+    x2 = next_item(x2 + 1, cls2);
   }
   __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));             // nothing may land in LDS after the workgroup has gone
 

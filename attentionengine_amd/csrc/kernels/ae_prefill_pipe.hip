@@ -42,6 +42,10 @@
 #include "ae_config.h"
 #include "ae_device.h"
 #include "ae_functors.h"
+#include "ae_tile_table.h"
+#ifndef AE_HEAVY_LAST
+#define AE_HEAVY_LAST 0      // 1: the tile table gives late q tiles more work than early ones
+#endif
 
 #define AE_WROWS 64                // query rows per wave (two 32-row blocks)
 #define AE_BM (AE_NWAVES * AE_WROWS)
@@ -118,9 +122,11 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int wg = blockIdx.x;
   const int xcd = wg & 7;
   const int slot = wg >> 3;
-#if AE_MASK_MODE == 1
+#if AE_MASK_MODE == 1 || (AE_MASK_MODE == 2 && AE_HEAVY_LAST)
   // causal: q tiles differ in work by up to n_qt : 1, so ids go heaviest tile first across ALL heads
-  // (longest-job-first keeps the tail short); the heads of one XCD still meet in its L2
+  // (longest-job-first keeps the tail short); the heads of one XCD still meet in its L2.  A tile table whose
+  // late q tiles are the long ones (AE_HEAVY_LAST, found on the host: causal variants, long sliding windows)
+  // takes the same order: B2 H32 S4096, "kv <= q + 1": 0.40 -> 0.35 ms.
   const int n_bg = (n_bh + 7) >> 3;
   const int qt = n_qt - 1 - slot / n_bg;
   const int bh = (slot % n_bg) * 8 + xcd;
@@ -185,50 +191,37 @@ void ae_prefill_kernel(const ae_attn_params p) {
   }
 #endif
 #if AE_MASK_MODE == 2
-  const int8_t* bm_base = p.block_mask +
-      ((int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : h)) * p.mask_nq * (int64_t)p.mask_nkv;
-  const int bm_r0 = q0 / p.mask_block_m;
-  int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
-  bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
-  auto tile_class = [&](int j) AE_LAMBDA -> int {   // 0 skip, 1 elementwise mask, 2 fully visible
-    const int col = (j * AE_BN) / p.mask_block_n;
-    int any = 0, all = 2;
-    for (int r = bm_r0; r <= bm_r1; r++) {
-      int c = bm_base[(int64_t)r * p.mask_nkv + col];
-      any |= c;
-      all = c < all ? c : all;
-    }
-    return any == 0 ? 0 : (all == 2 ? 2 : 1);
-  };
+  // tile classes from the block table, 64 kv tiles at a time (ae_tile_table.h): 0 skip, 1 elementwise mask,
+  // 2 fully visible
+  ae_tile_table tt;
+  ae_tt_init(tt, p, b, h, q0, AE_BM);
 #endif
   auto next_tile = [&](int j) AE_LAMBDA {
 #if AE_MASK_MODE == 2
-    while (j < j_end && tile_class(j) == 0) j++;
+    j = ae_tt_next(tt, p, j, j_end, AE_BN, n_kvt);
 #endif
     return j < j_end ? j : j_end;
   };
-  // does tile j need the elementwise mask for this wave's rows?
-  auto needs_mask = [&](int j) AE_LAMBDA -> bool {
-    bool nm = false;
+  // What tile j (just found by next_tile) means to this wave: the class of each lane's two rows (the table may
+  // be finer than the 256-row q tile - user block masks -, so rows of one workgroup, even of one wave, can
+  // differ), and whether the wave takes the masked path for it: anything but "every row of this wave sees the
+  // whole tile".
+  auto tile_info = [&](int j, int (&c)[2], bool& nm) AE_LAMBDA {
+    nm = false;
+    c[0] = c[1] = 2;
+    if (j >= j_end) return;
 #if AE_MASK_MODE == 1
     nm = j * AE_BN + AE_BN - 1 > q0w;
 #elif AE_MASK_MODE == 2
-    // the table may be finer than the 256-row q tile (user block masks): rows of one workgroup, even of
-    // one wave, can differ in class, so anything but "every table row of this wave says fully visible"
-    // takes the masked path, which looks the class up per row
-    {
-      const int col = (j * AE_BN) / p.mask_block_n;
-      int r1 = (q0w + AE_WROWS - 1) / p.mask_block_m;
-      r1 = r1 < p.mask_nq ? r1 : p.mask_nq - 1;
-      for (int r = q0w / p.mask_block_m; r <= r1; r++) nm = nm || (bm_base[(int64_t)r * p.mask_nkv + col] != 2);
-    }
+    c[0] = ae_tt_class(tt, p, j, qrow[0]);
+    c[1] = ae_tt_class(tt, p, j, qrow[1]);
+    nm = __builtin_amdgcn_ballot_w64(c[0] != 2 || c[1] != 2) != 0;
 #elif AE_HAS_MASK_MOD
     nm = true;
 #endif
 #if !AE_EVEN_KV
     nm = nm || (j * AE_BN + AE_BN > p.seqlen_kv);
 #endif
-    return nm;
   };
 
   const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
@@ -447,16 +440,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // row maxima against the (lazy) reference.  The common case ends after two exchanges and a ballot; a
   // row whose maximum exceeds its threshold moves its reference (cold path): sv is shifted, the
   // running sum rescaled here, O before the next iteration (rescale_o, outside the hot loop).
-  auto finish_scores = [&](int j) AE_LAMBDA {
+  auto finish_scores = [&](int j, const int (&tcls)[2], bool masked) AE_LAMBDA {
     const int kvb = j * AE_BN + 4 * hf;
-    if (needs_mask(j)) {
+    if (masked) {
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
         mx[qb] = AE_NEG_INF;
 #if AE_MASK_MODE == 2
-        int rr = qrow[qb] / p.mask_block_m;
-        rr = rr < p.mask_nq ? rr : p.mask_nq - 1;
-        const int cls = bm_base[(int64_t)rr * p.mask_nkv + (j * AE_BN) / p.mask_block_n];   // this row's class
+        const int cls = tcls[qb];   // this row's class
 #endif
 #pragma unroll
         for (int e = 0; e < 32; e++) {
@@ -521,8 +512,13 @@ void ae_prefill_kernel(const ae_attn_params p) {
 
   // ---- prologue: first tile's scores ------------------------------------------------------------
   int j0 = next_tile(0);                  // tile whose scores are in sv (exp + PV next)
+  int tc0[2], tc1[2], tc2[2];             // ... and what tiles j0, j1, j2 mean to this wave (tile_info)
+  bool tnm0, tnm1, tnm2 = false;
+  tile_info(j0, tc0, tnm0);
+  tc2[0] = tc2[1] = 2;
   const bool any_tile = j0 < j_end;
   int j1 = any_tile ? next_tile(j0 + 1) : j_end;   // tile multiplied by Q next
+  tile_info(j1, tc1, tnm1);
   if (any_tile) {
     load_k(j0, 0);
     load_v(j0, 0);
@@ -542,7 +538,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     mx[0] = mx[1] = AE_NEG_INF;
     read_scores(0, 0, 32);
     read_scores(1, 0, 32);
-    finish_scores(j0);
+    finish_scores(j0, tc0, tnm0);
     rescale = false;                       // O is still zero
   }
   __syncthreads();                         // everyone is done with K stage 0 before it is refilled
@@ -574,6 +570,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
     const ae_lds_byte* vt = lds + 2 * AE_K_BYTES + (n & 1) * AE_V_BYTES;
     const int j2 = (HN || TL) ? next_tile(j1 + 1) : j_end;
+    tile_info(j2, tc2, tnm2);
     // Nothing is in flight here on the back edge (the iteration ends with vmcnt(0)); saying so
     // also clears loads still pending on loop ENTRY (Q fragments, spill reloads), which the
     // compiler's wait-count insertion would otherwise wait for after this iteration's tile loads
@@ -640,20 +637,22 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
     for (int qb = 0; qb < 2; qb++) r_run[qb] += rsum[qb];
 #if !AE_TOP_PREFETCH
-    if (HN) finish_scores(j1);
+    if (HN) finish_scores(j1, tc1, tnm1);
 #endif
     // tiles for the next iteration must have landed, and everyone must be done with this one's
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);   // vmcnt(0)
     __syncthreads();
     j0 = j1;
     j1 = j2;
+    tc0[0] = tc1[0], tc0[1] = tc1[1], tnm0 = tnm1;
+    tc1[0] = tc2[0], tc1[1] = tc2[1], tnm1 = tnm2;
     n++;
 #if AE_TOP_PREFETCH
     if (HN) {
       // the next iteration's first fragments go out now, and the new tile's maxima are compared with the
       // reference while they travel (an iteration that started with the reads would wait for them)
       prefetch_ring();
-      finish_scores(j0);
+      finish_scores(j0, tc0, tnm0);
     }
 #endif
   };
@@ -689,7 +688,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
     __syncthreads();
     j0 = j1;
     j1 = j2;
-    n++;
+    n++;      // (a wave that only requests tiles no longer looks at their classes)
   };
   if (any_tile) {
     while (true) {

@@ -43,6 +43,10 @@
 // consecutive kv positions per tile
 #define AE_KV_PF_GROUPS (AE_BN / 8)
 #include "ae_functors.h"  // generated: the functor bodies
+#include "ae_tile_table.h"
+#ifndef AE_HEAVY_LAST
+#define AE_HEAVY_LAST 0      // 1: the tile table gives late q tiles more work than early ones
+#endif
 
 // value given to score positions past seqlen_kv before the user functors run: -inf, or 0 for graphs
 // declared with mask_value="0" (no additive -inf mask anywhere, attn_tl.py:124-137 / lower.py:637)
@@ -108,7 +112,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int qt_i = slot % n_qt;
   const int bh = (slot / n_qt) * 8 + xcd;
   if (bh >= n_bh) return;
-#if AE_MASK_MODE == 1
+#if AE_MASK_MODE == 1 || (AE_MASK_MODE == 2 && AE_HEAVY_LAST)     // (long q tiles first)
   const int qt = n_qt - 1 - qt_i;
 #else
   const int qt = qt_i;
@@ -151,25 +155,12 @@ void ae_prefill_kernel(const ae_attn_params p) {
   }
 #endif
 #if AE_MASK_MODE == 2
-  // Tile class from the block table: 0 = skip, 1 = visit with the elementwise mask, 2 = fully
-  // visible.  A q-tile may span several table rows: it is skipped only if every row says so and
-  // fully visible only if every row says so.
-  const int8_t* bm_base = p.block_mask +
-      ((int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : h)) * p.mask_nq * (int64_t)p.mask_nkv;
-  const int bm_r0 = q0 / p.mask_block_m;
-  int bm_r1 = (q0 + AE_BM - 1) / p.mask_block_m;
-  bm_r1 = bm_r1 < p.mask_nq ? bm_r1 : p.mask_nq - 1;
-  auto tile_class = [&](int j) AE_LAMBDA -> int {
-    const int col = (j * AE_BN) / p.mask_block_n;
-    int any = 0, all = 2;
-    for (int r = bm_r0; r <= bm_r1; r++) {
-      int c = bm_base[(int64_t)r * p.mask_nkv + col];
-      any |= c;
-      all = c < all ? c : all;
-    }
-    return any == 0 ? 0 : (all == 2 ? 2 : 1);
-  };
-#define AE_TILE_CLASS(j) tile_class(j)
+  // Tile classes from the block table (ae_tile_table.h): 0 = skip, 1 = visit with the elementwise mask (every
+  // position, where the graph has no mask_mod: a block mask of the user), 2 = fully visible.  A q tile may span
+  // several table rows: a kv tile is skipped only if every row says so, and every lane applies the class of
+  // its own row.
+  ae_tile_table tt;
+  ae_tt_init(tt, p, b, h, q0, AE_BM);
 #endif
 
   const ae_elem* kbase = (const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)hk * p.k_stride_h;
@@ -220,9 +211,17 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // next tile index >= j that has work (block table) or j itself
   auto next_tile = [&](int j) AE_LAMBDA {
 #if AE_MASK_MODE == 2
-    while (j < j_end && AE_TILE_CLASS(j) == 0) j++;
+    j = ae_tt_next(tt, p, j, j_end, AE_BN, n_kvt);
 #endif
     return j;
+  };
+  // class of tile j for this lane's row of row block rb (right after next_tile() found j)
+  auto row_class = [&](int j, int rb) AE_LAMBDA -> int {
+#if AE_MASK_MODE == 2
+    return j < j_end ? ae_tt_class(tt, p, j, qrow[rb]) : 0;
+#else
+    return 2;
+#endif
   };
 
   // ---- state ------------------------------------------------------------------------------
@@ -251,6 +250,9 @@ void ae_prefill_kernel(const ae_attn_params p) {
 
   int j = next_tile(0);
   bool any_tile = j < j_end;
+  int cls[AE_RB];          // class of tile j for this lane's row of each row block
+#pragma unroll
+  for (int rb = 0; rb < AE_RB; rb++) cls[rb] = row_class(j, rb);
   if (any_tile) {
     load_tile(j);
     store_tile(0);
@@ -268,6 +270,9 @@ void ae_prefill_kernel(const ae_attn_params p) {
   int stage = 0;
   while (j < j_end) {
     const int jn = next_tile(j + 1);
+    int cls_n[AE_RB];
+#pragma unroll
+    for (int rb = 0; rb < AE_RB; rb++) cls_n[rb] = row_class(jn, rb);
     if (jn < j_end) load_tile(jn);
 
     ae_lds_byte* ks_ = lds + stage * AE_STAGE_BYTES;
@@ -310,10 +315,19 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
         for (int e = 0; e < AE_NS; e++) s[e] = (qrow[rb] >= kvb + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
       }
-#elif AE_HAS_MASK_MOD
-#if AE_MASK_MODE == 2
-      if (AE_TILE_CLASS(j) != 2)
+#elif AE_MASK_MODE == 2 && !(defined(AE_MASK_VALUE_ZERO) && AE_MASK_VALUE_ZERO)
+      if (__builtin_amdgcn_ballot_w64(cls[rb] != 2) != 0) {   // some row of this block does not see the whole tile
+#pragma unroll
+        for (int e = 0; e < AE_NS; e++) {
+#if AE_HAS_MASK_MOD
+          const bool vis = cls[rb] == 2 || (cls[rb] == 1 && ae_mask_mod(b, h, qrow[rb], kvb + ae_kv_off(e)));
+#else
+          const bool vis = cls[rb] != 0;
 #endif
+          s[e] = vis ? s[e] : AE_NEG_INF;
+        }
+      }
+#elif AE_HAS_MASK_MOD
       {
 #pragma unroll
         for (int e = 0; e < AE_NS; e++)
@@ -385,6 +399,8 @@ void ae_prefill_kernel(const ae_attn_params p) {
     __syncthreads();
     stage ^= 1;
     j = jn;
+#pragma unroll
+    for (int rb = 0; rb < AE_RB; rb++) cls[rb] = cls_n[rb];
   }
 
   // ---- epilogue -------------------------------------------------------------------------------

@@ -114,6 +114,13 @@ def test_softmax_backward_skips_masked_tiles(cuda_device):
         assert eng._op._plan(1, H, S, S, None).mode == 2
 
 
+def test_backward_tile_classes_of_a_long_sequence(cuda_device):
+    """More than 64 streamed items per workgroup (68 q tiles of 64 rows for each of the two q heads of a kv
+    head): the kernels read the tile classes 64 items at a time, so this crosses from one set to the next."""
+    print("case bwd tile classes, 136 items per kv tile", flush=True)
+    _run(1, 2, 1, 4352, 4352, 64, 64, torch.bfloat16, C.make_sliding_window_mask(300), False, seed=13)
+
+
 def test_backward_odd_shapes_against_oracle(cuda_device):
     """Seeded sweep: ragged sequence lengths (also Sq != Skv without a mask), grouped heads, both head
     dims for keys and values, both dtypes, no mask / causal / sliding window / head-dependent masks."""

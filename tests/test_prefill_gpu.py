@@ -265,20 +265,32 @@ def test_mask_is_bit_exact(cuda_device):
         assert torch.equal(out, expect), mask_mod.__name__
 
 
-def test_extern_block_mask(cuda_device):
-    """attn_script/blocksparseattn.py: user-supplied int8 block mask [B,H,S/128,S/128], no
-    mask_mod; reference = masked softmax with the expanded block mask (129-135)."""
-    B, H, S, D = 1, 4, 1024, 128
+@pytest.mark.parametrize("kernel,bm,bn,S", [
+    ("generic", 128, 128, 1024),       # attn_script/blocksparseattn.py: blocks of 128 x 128
+    ("pipelined", 128, 128, 1024),     # two table rows per 256-row q tile
+    ("generic", 64, 64, 640),          # two table rows per 128-row q tile: rows of one tile differ in class
+    ("pipelined", 32, 128, 1024),      # eight table rows per q tile, rows of one WAVE differ in class
+    ("generic", 256, 64, 4096 + 512),  # more than 64 kv tiles: the tile classes are read in two chunks
+    ("pipelined", 128, 128, 4096 + 512),
+])
+def test_extern_block_mask(cuda_device, monkeypatch, kernel, bm, bn, S):
+    """attn_script/blocksparseattn.py: user-supplied int8 block mask [B,H,S/bm,S/bn], no
+    mask_mod; reference = masked softmax with the expanded block mask (129-135).  Tiles whose entry is 0 are
+    skipped, and inside a visited tile every query row follows the entry of its own table row."""
+    print(f"case extern block mask {kernel} {bm}x{bn} S{S}", flush=True)
+    monkeypatch.setenv("AE_PREFILL_KERNEL", kernel)
+    B, H, D = 1, 3, 128
     dtype = torch.float16
     g = torch.Generator().manual_seed(1)
-    nb = S // 128
-    blocks = (torch.rand(B, H, nb, nb, generator=g) < 0.4)
-    blocks |= torch.eye(nb, dtype=torch.bool)      # every row sees something
+    nq, nk = S // bm, S // bn
+    blocks = (torch.rand(B, H, nq, nk, generator=g) < 0.4)
+    blocks[..., 0] = True                           # every row sees something
     q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
     mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), None, C.OnlineSoftmax(),
-                  infer_mask=True, extern_block_mask=True)
+                  infer_mask=True, extern_block_mask=True, infer_mask_block_M=bm, infer_mask_block_N=bn)
+    assert mod.attention.tiles.rows_per_wave == (64 if kernel == "pipelined" else 32)
     out = mod(q.cuda(), k.cuda(), v.cuda(), block_mask=blocks.to(torch.int8).cuda())
-    dense = blocks.repeat_interleave(128, 2).repeat_interleave(128, 3)
+    dense = blocks.repeat_interleave(bm, 2).repeat_interleave(bn, 3)
     ref, lref = R.softmax_attention(q, k, v, mask=dense)
     assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
     assert (mod.final_rowscales["lse"].cpu() - lref).abs().max().item() <= LSE_TOL
