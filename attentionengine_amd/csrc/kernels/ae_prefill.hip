@@ -501,9 +501,11 @@ void ae_prefill_kernel(const ae_attn_params p) {
                     (int64_t)h * p.o_stride_h;
 #pragma unroll
     for (int db = 0; db < AE_NDB; db++) {
+      // (read where it is used: as plain copies the accumulator reads of EVERY block move to the front, which
+      // takes the whole register file and spills; a volatile asm statement stays behind the previous block's stores)
       float o[16];
 #pragma unroll
-      for (int r = 0; r < 16; r++) o[r] = oacc[rb][db][r];
+      for (int r = 0; r < 16; r++) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(o[r]) : "a"(oacc[rb][db][r]));
       if (any_tile) {
         ae_epilogue<16>(o, st[rb], frs, ctx[rb], cust[rb]);
       } else {

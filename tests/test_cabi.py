@@ -237,3 +237,24 @@ def test_prefill_kernels_keep_their_arrays_in_registers(dtype, D, causal):
         for key, (module, _, _) in op._variants.items():
             for kname, k in module.kernel_info().items():
                 assert k[".private_segment_fixed_size"] <= 64, (t, key, kname, k[".private_segment_fixed_size"])
+
+
+@pytest.mark.parametrize("mask", [None, "causal", "window"])
+@pytest.mark.parametrize("S", [128, 100])
+def test_wide_value_heads_do_not_spill(mask, S):
+    """Value head dim 512 (256 accumulator registers per lane): the builds keep everything in registers.  Their
+    epilogue reads the accumulators block by block through volatile asm statements; as plain copies the compiler
+    moved the reads of every block to the front, spilled one block - and in one build (tile table, ragged tiles)
+    lost one of the sixteen registers on the way back."""
+    import attn_cases as C
+    from core import CustomIO, meta_tensor
+    from core.lower.prefill_op import PrefillOp
+    mask_mod = {None: None, "causal": C.causal_mask, "window": C.make_sliding_window_mask(70)}[mask]
+    for D, dtype in ((256, torch.float16), (128, torch.bfloat16)):
+        meta = (meta_tensor(1, 1, S, D, dtype=dtype), meta_tensor(1, 1, S, D, dtype=dtype),
+                meta_tensor(1, 1, S, 512, dtype=dtype))
+        op = PrefillOp(meta, CustomIO({}), C.make_scale_score_mod(D ** -0.5), mask_mod, C.OnlineSoftmax(), "-inf")
+        assert op.DV_launch == 512
+        for key, (module, _, _) in op._variants.items():
+            k = module.kernel_info()["ae_prefill_kernel"]
+            assert k[".vgpr_spill_count"] == 0 and k[".private_segment_fixed_size"] == 0, (D, dtype, mask, S, key)

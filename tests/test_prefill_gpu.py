@@ -450,6 +450,8 @@ def test_small_and_odd_shapes_against_oracle(cuda_device):
     (1, 2, 2, 384, 384, 128, 512, torch.float16, "window", False),     # tile-class table + mask_mod, 32-key tiles
     (1, 2, 1, 200, 200, 64, 256, torch.float16, "causal", False),
     (1, 2, 2, 320, 320, 256, 512, torch.float16, "causal", True),      # the sliced form (two launches of 256 columns)
+    (1, 1, 1, 257, 257, 256, 512, torch.float16, "window", False),     # tile table AND ragged tiles
+    (1, 2, 2, 100, 100, 128, 512, torch.bfloat16, "window", False),
 ])
 def test_wide_head_dims_in_the_direct_to_lds_kernel(cuda_device, monkeypatch, B, H, Hkv, Sq, Skv, D, DV, dtype, mask,
                                                     slice_dv):
