@@ -27,7 +27,7 @@ class PrefillOp:
 
     def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
-                 extern_block_mask=False, split_kv=False, target_workgroups=512,
+                 extern_block_mask=False, split_kv=False, target_workgroups=256,
                  tiles=None, tune=False, tune_file="", tune_bwd=False, tune_file_bwd=""):
         self._ctor = ((qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value),
                       dict(infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
@@ -218,8 +218,10 @@ class PrefillOp:
     COMBINE_THREADS = 128
 
     def plan_splits(self, B, Hq, Sq, Skv):
-        """(number of KV splits, kv positions per split): enough workgroups to fill the chip, whole
-        kv tiles per split, no empty split."""
+        """(number of KV splits, kv positions per split): a workgroup for every CU of the chip (more splits cost
+        more in partial results and their merge than they gain: B1 H32 Sq128 Skv8192, the shape of
+        attn_script/mha_inference.py, 43 us with 8 splits, 44 with 16, 75 with 32), whole kv tiles per split, no
+        empty split."""
         if not self.split_kv:
             return 1, Skv
         bn = self.tiles.block_n

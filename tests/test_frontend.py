@@ -230,9 +230,9 @@ def test_engine_dispatch_and_compile_on_cpu():
     mhad = AttentionEngine(_meta(1, 32, 32, 128, 8192, 128, 128, torch.float16), CustomIO({}), sm, None,
                            C.OnlineSoftmax())
     assert isinstance(mhad._op, PrefillOp) and mhad._op.split_kv
-    assert mhad._op.plan_splits(1, 32, 128, 8192) == (16, 512)
+    assert mhad._op.plan_splits(1, 32, 128, 8192) == (8, 1024)
     assert mhad._op.plan_splits(2, 4, 5, 1000) == (16, 64)       # never an empty split, whole tiles
-    assert "#define AE_NSPLIT 16" in mhad.tl_code and "ae_combine" in mhad.tl_code
+    assert "#define AE_NSPLIT 8" in mhad.tl_code and "ae_combine" in mhad.tl_code
     # tuner / backend arguments of the reference scripts are accepted
     AttentionEngine(_meta(1, 2, 2, 128, 128, 64, 64, torch.float16), CustomIO({}), sm, C.causal_mask,
                     C.OnlineSoftmax(), tune=True, tune_file="x.json", tune_bwd=True, backend="cute")
