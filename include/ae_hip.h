@@ -104,7 +104,11 @@ typedef struct ae_attn_params {
    * block_table[b * block_table_stride + t / page_block_size], and entry b holds
    * min(seqlens_k[b], seqlen_kv) tokens.  Stands where the reference passes block_table,
    * block_table_batch_stride, page_block_size and seqlens_k_ptr
-   * (core/template/cute_template_kvshared/kernels/params.h:33-36, flash_api.cpp:61-72). */
+   * (core/template/cute_template_kvshared/kernels/params.h:33-36, flash_api.cpp:61-72).
+   * The latent part (k) and the rope part (k2) are column ranges of that ONE cache tensor: equal strides,
+   * k2 at most 1 MiB behind k.  A split spans at most 1022 pages (kv_per_split / page_block_size + 2 <= 1024).
+   * In a split launch an entry whose keys all lie in the first split writes `out` itself; splits without
+   * keys write nothing and the merge reads only the splits that hold keys. */
   const int32_t* block_table;                /* int32 [B, block_table_stride]             */
   const int32_t* seqlens_k;                  /* int32 [B]                                 */
   int32_t block_table_stride;                /* entries per batch row of block_table      */
