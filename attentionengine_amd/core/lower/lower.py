@@ -590,7 +590,12 @@ class PrefillTiles:
         return self.rows_per_wave * self.n_waves
 
     def lds_bytes(self, d: int, dv: int) -> int:
-        return 2 * self.block_n * ((2 * d + self.k_pad) + (2 * dv + self.v_pad))
+        stages = 2 * self.block_n * ((2 * d + self.k_pad) + (2 * dv + self.v_pad))
+        if self.template == "ae_prefill_pipe.hip":
+            # behind the tile stages every wave has room for its 64 Q rows (later its 64 O rows), which travel
+            # through LDS as whole rows (AE_QO_BYTES of the kernel)
+            stages += self.n_waves * 64 * 2 * max(d, dv)
+        return stages
 
 
 # Compute units of an MI355X: the pipelined kernel's 256-row tiles are only chosen when there are
@@ -612,14 +617,17 @@ def direct_tile_ok(d: int, dv: int, block_n: int, n_waves: int = 4) -> bool:
 
 
 def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0,
-                         elementwise: bool = False) -> PrefillTiles:
+                         elementwise: bool = False, seqlen_kv: int = 0) -> PrefillTiles:
     """The direct-to-LDS kernels handle head dims 64 and 128 (and, the generic one, 96, 160, 192, 256 and value
     head dims up to 512, with one wave per SIMD where the accumulators need it): the
     software-pipelined one (64 rows per wave, 256-row q tiles, one wave per SIMD) when the graph is
     the online softmax of scaled scores, or elementwise (out = sum f(s) v: the kernel then calls the
     generated functor), and the problem has enough q tiles to occupy the chip
-    (measured on B2 H32 S4096 D128 fp16: 1.0 against 0.86 PFLOP/s non-causal), otherwise the generic
-    one (32 rows per wave, two waves per SIMD, runs any functor).  Other head dims use the
+    (measured on B2 H32 S4096 D128 fp16: 1.0 against 0.86 PFLOP/s non-causal) and its rows are long enough
+    for the pipeline to pay (short sequences are bound by the Q / O traffic and the start-up of a workgroup,
+    which two workgroups per CU hide better: 16k tokens fp16 H32, S256 D128 0.136 against 0.162 ms, S512
+    D64 causal 0.085 against 0.111 ms; from S1024 D128 / S2048 D64 on the pipelined kernel wins), otherwise
+    the generic one (32 rows per wave, two waves per SIMD, runs any functor).  Other head dims use the
     register-staged kernel with padded LDS rows (ae_prefill_simple.hip), with one wave per SIMD and a
     shorter kv tile once the accumulators outgrow 256 registers.  AE_PREFILL_KERNEL=generic|pipelined
     overrides the choice between the first two (tests)."""
@@ -639,6 +647,8 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
         # (elementwise graphs at head dim 64 have too little matrix work per score for the pipelined kernel's
         # one wave per SIMD to pay: relu attention B64 H6 S2048 D64 0.48 ms against 0.45 ms in the generic one)
         fits = softmax is not None or (elementwise and max(d, dv) > 64)
+        if seqlen_kv and seqlen_kv * max(d, dv) < 1024 * 128:
+            fits = False
         if d in (64, 128) and (softmax is not None or elementwise) and force != "generic" and (
                 force == "pipelined" or (fits and n_tiles >= (3 * _MI355X_CUS) // 4)):
             return PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)

@@ -68,7 +68,8 @@ class PrefillOp:
         self.tiles = L.choose_prefill_tiles(self.D, self.DV_launch, _dim(q_meta.shape[2], 0),
                                             self._pipe_softmax,
                                             _dim(q_meta.shape[0], 1) * _dim(q_meta.shape[1], 1),
-                                            elementwise=self._pipe_elementwise)
+                                            elementwise=self._pipe_elementwise,
+                                            seqlen_kv=_dim(k_meta.shape[2], 0))
         # Masks that reach the kernel as a tile table (anything but none / exactly causal) go to the generic
         # kernel: with its 128-row q tiles fewer tiles are partly visible, and its masked path costs less than
         # the pipelined kernel's (B2 H32 S4096 D128, sliding window of 256: 0.13 against 0.31 ms; a random block

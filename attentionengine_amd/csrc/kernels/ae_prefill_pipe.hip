@@ -66,6 +66,7 @@
 #define AE_K_RPI (64 / AE_KCPR)
 #define AE_V_RPI (64 / AE_VCPR)
 #define AE_VPPR (AE_VCPR / 2)
+#define AE_QO_BYTES (AE_WROWS * (AE_KSTR > AE_VSTR ? AE_KSTR : AE_VSTR))   // a wave's Q rows, later its O rows
 #define AE_VPS1 (32 / AE_NKF)      // scores per row handled next to one phase-1 MFMA
 #define AE_VPS2 (32 / AE_NVF)      // scores per row read back next to one phase-2 MFMA
 #ifndef AE_AHEAD
@@ -107,7 +108,7 @@ struct ae_tag_false { static constexpr bool value = false; };
 extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void ae_prefill_kernel(const ae_attn_params p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
-  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // [2][K tile] then [2][V tile]
+  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // [2][K tile], [2][V tile], then AE_QO_BYTES per wave (its Q rows, later its O rows)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -153,20 +154,29 @@ void ae_prefill_kernel(const ae_attn_params p) {
   }
 
   // ---- Q fragments (B operand of S^T = K Q^T), resident ------------------------------------
+  // The wave's 64 rows travel HBM -> LDS as whole rows (16 lanes per 256-byte row: a lane that fetched its own
+  // row's fragments straight into registers asked for 32 rows per instruction, 16 bytes of each, and the
+  // workgroups of a launch, which start and end together, then queue behind each other's requests: 3.5 us
+  // until the first tile could be multiplied), swizzled like a K tile, into a region of the wave's own behind
+  // the tile stages; the fragments are read from there once the first tiles have landed too.
   ae_elem8 qf[2][AE_NKS];
+  ae_lds_byte* qo = lds + 2 * AE_K_BYTES + 2 * AE_V_BYTES + wave * AE_QO_BYTES;
+  {
+    const int q0c = q0w < p.seqlen_q ? q0w : p.seqlen_q - 1;
+    const char* qg = (const char*)((const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)q0c * p.q_stride_s +
+                                   (int64_t)h * p.q_stride_h) - 4096;
 #pragma unroll
-  for (int qb = 0; qb < 2; qb++) {
-    const int qr = q_ok[qb] ? qrow[qb] : p.seqlen_q - 1;
-    const ae_elem* qptr = (const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)qr * p.q_stride_s +
-                          (int64_t)h * p.q_stride_h;
+    for (int g = 0; g < AE_KCPR / 8; g++) {
+      unsigned off[8];
 #pragma unroll
-    for (int ks = 0; ks < AE_NKS; ks++) {
-      ae_elem8 t = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
-#if AE_PRESCALE
-#pragma unroll
-      for (int i = 0; i < 8; i++) t[i] = (ae_elem)((float)t[i] * (AE_SM_SCALE * AE_LOG2E));
-#endif
-      qf[qb][ks] = t;
+      for (int i = 0; i < 8; i++) {
+        const int row = (g * 8 + i) * AE_K_RPI + lane / AE_KCPR;
+        const int c = (lane % AE_KCPR) ^ (row & (AE_KCPR - 1));
+        int ra = q0w + row;                      // rows past the end re-read the last row
+        ra = ra < p.seqlen_q ? ra : p.seqlen_q - 1;
+        off[i] = (unsigned)(((ra - q0c) * (int)p.q_stride_s + c * 8) * 2 + 4096 - (i - 4) * 1024);
+      }
+      ae_load_lds16_burst_base<8>(qg, off, qo + (g * 8 + 4) * 1024);
     }
   }
 
@@ -282,6 +292,23 @@ void ae_prefill_kernel(const ae_attn_params p) {
         g, gp, lds + 2 * AE_K_BYTES + stage * AE_V_BYTES + (wave * AE_V_LOADS + AE_V_LOADS / 2) * 1024);
   };
 
+  // ---- the first tiles are requested before anything else is set up: the zeroing of the accumulators, the
+  // constants and the address arithmetic below (about a thousand instructions of one wave per SIMD) then run
+  // while they and the Q rows travel ----
+  int j0 = next_tile(0);                  // tile whose scores are in sv (exp + PV next)
+  int tc0[2], tc1[2], tc2[2];             // ... and what tiles j0, j1, j2 mean to this wave (tile_info)
+  bool tnm0, tnm1, tnm2 = false;
+  tile_info(j0, tc0, tnm0);
+  tc2[0] = tc2[1] = 2;
+  const bool any_tile = j0 < j_end;
+  int j1 = any_tile ? next_tile(j0 + 1) : j_end;   // tile multiplied by Q next
+  tile_info(j1, tc1, tnm1);
+  if (any_tile) {
+    load_k(j0, 0);
+    load_v(j0, 0);
+    if (j1 < j_end) load_k(j1, 1);
+  }
+
   // ---- state ------------------------------------------------------------------------------
   ae_ctx ctx[2];
   ae_custom cust[2];
@@ -322,6 +349,11 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) oacc[qb][db][r] = 0.f;
   }
+  // (the zeroes are written now, while the first tiles travel: left alone, the compiler writes them after the wait)
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++) asm volatile("" : "+a"(oacc[qb][db]));
 
   // lane-constant pieces of the swizzled LDS fragment addresses (see ae_prefill.hip)
   const int k_row_off = l32 * AE_KSTR;
@@ -511,21 +543,30 @@ void ae_prefill_kernel(const ae_attn_params p) {
   };
 
   // ---- prologue: first tile's scores ------------------------------------------------------------
-  int j0 = next_tile(0);                  // tile whose scores are in sv (exp + PV next)
-  int tc0[2], tc1[2], tc2[2];             // ... and what tiles j0, j1, j2 mean to this wave (tile_info)
-  bool tnm0, tnm1, tnm2 = false;
-  tile_info(j0, tc0, tnm0);
-  tc2[0] = tc2[1] = 2;
-  const bool any_tile = j0 < j_end;
-  int j1 = any_tile ? next_tile(j0 + 1) : j_end;   // tile multiplied by Q next
-  tile_info(j1, tc1, tnm1);
-  if (any_tile) {
-    load_k(j0, 0);
-    load_v(j0, 0);
-    if (j1 < j_end) load_k(j1, 1);
-  }
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
+#pragma unroll
+  for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+    for (int ks = 0; ks < AE_NKS; ks++) {
+      ae_elem8 t = *(const __attribute__((address_space(3))) ae_elem8*)(
+          qo + (qb * 32 + l32) * AE_KSTR + (((2 * ks + hf) ^ k_sw) << 4));
+#if AE_PRESCALE
+      // q * (c log2e), the product in fp32 rounded once to fp16: one mixed-precision fma per value (written as
+      // conversions and a multiplication the compiler issues five instructions per pair)
+      ae_u32x4 tp = __builtin_bit_cast(ae_u32x4, t);
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        unsigned d;
+        asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=&v"(d) : "v"(tp[i]), "s"(AE_SM_SCALE * AE_LOG2E));
+        asm("v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+            : "+&v"(d) : "v"(tp[i]), "s"(AE_SM_SCALE * AE_LOG2E));
+        tp[i] = d;
+      }
+      t = __builtin_bit_cast(ae_elem8, tp);
+#endif
+      qf[qb][ks] = t;
+    }
   if (any_tile) {
 #pragma unroll
     for (int f = 0; f < AE_NKF; f++) {
@@ -749,9 +790,17 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
       for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
     }
-    if (q_ok[qb]) {
-      ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow[qb] * p.o_stride_s +
-                      (int64_t)h * p.o_stride_h;
+    // O leaves through the wave's LDS region (the Q rows are long in registers): a lane holds four adjacent
+    // values of its own row per accumulator group, so stores straight from the registers would touch 32 rows
+    // per instruction, 16 bytes of each
+    {
+      // (the addresses are derived from a copy of the lane id that the compiler cannot trace back: it would
+      // otherwise keep the prologue's Q fragment addresses, which have the same form, in registers across the
+      // whole loop and spill for it)
+      int le = lane;
+      asm volatile("" : "+v"(le));
+      ae_lds_byte* orow = qo + (qb * 32 + (le & 31)) * AE_VSTR + (le >> 5) * 8;
+      const int osw = le & (AE_VCPR - 1);
 #pragma unroll
       for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
@@ -759,13 +808,28 @@ void ae_prefill_kernel(const ae_attn_params p) {
           ae_elem4 w;
 #pragma unroll
           for (int t = 0; t < 4; t++) w[t] = (ae_elem)o[db * 16 + rg * 4 + t];
-          *(ae_elem4*)(optr + db * 32 + rg * 8 + hf * 4) = w;
+          *(__attribute__((address_space(3))) ae_elem4*)(orow + (((db * 4 + rg) ^ osw) << 4)) = w;
         }
-      if (hf == 0) {
+    }
+    if (q_ok[qb] && hf == 0) {
 #pragma unroll
-        for (int i = 0; i < AE_N_ROWSCALES; i++)
-          p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[qb]] = frs[i];
-      }
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+        p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[qb]] = frs[i];
+    }
+  }
+  // (the rows were written by other lanes of this wave: LDS instructions of a wave complete in order)
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  {
+    ae_elem* og = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;
+    int le = lane;
+    asm volatile("" : "+v"(le));
+#pragma unroll
+    for (int i = 0; i < AE_VCPR; i++) {
+      const int row = i * AE_V_RPI + le / AE_VCPR;
+      const int c = le % AE_VCPR;
+      const ae_elem8 w = *(const __attribute__((address_space(3))) ae_elem8*)(
+          qo + row * AE_VSTR + ((c ^ (row & (AE_VCPR - 1))) << 4));
+      if (AE_EVEN_Q || q0w + row < p.seqlen_q) *(ae_elem8*)(og + (int64_t)(q0w + row) * p.o_stride_s + c * 8) = w;
     }
   }
 }
