@@ -113,6 +113,38 @@ AE_DEV int ae_k_swz(int c, int row) {
 #endif
 }
 
+// Q rows on their way in and O rows on their way out pass through LDS as whole rows (16 lanes per 256-byte row).
+// A lane that loads its own row's fragments, or stores its own row's results, touches 32 rows per instruction,
+// 16 bytes of each: the workgroups of a launch start and end together and queue behind each other's requests
+// (measured in the pipelined kernel: 3.5 us until the first tile could be multiplied, 4.4 us to get O out).
+// Q uses stage 1 of the tile ring, which is free until the loop's first prefetch, swizzled like a K tile; O the
+// whole ring after the last tile.  Builds whose rows do not fit there keep the direct accesses.
+#define AE_Q_LOADS ((AE_WROWS * AE_KCPR) / 64)     // direct loads per lane for the wave's Q rows
+#define AE_Q_VIA_LDS (AE_BM * AE_KSTR <= AE_STAGE_BYTES)
+#define AE_O_LOADS ((AE_WROWS * AE_VCPR) / 64)
+#define AE_O_VIA_LDS (AE_NSPLIT == 1 && AE_NO <= 128 && AE_BM * AE_VSTR <= 2 * AE_STAGE_BYTES)
+
+// the wave's Q rows -> qs, in bursts of up to eight loads.  qg: row q0c of this (batch, head), 4 KiB low (see
+// ae_load_lds16_burst_base); row0 = first row of the wave - q0c; rows past `last` (relative to q0c) re-read it.
+template <int G0>
+AE_DEV void ae_q_rows_to_lds(const char* qg, ae_lds_byte* qs, int lane, int row0, int last, int stride_s) {
+  if constexpr (G0 < AE_Q_LOADS) {
+    constexpr int N = AE_Q_LOADS - G0 < 8 ? AE_Q_LOADS - G0 : 8;
+    unsigned off[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int n = (G0 + (i < N ? i : 0)) * 64 + lane;      // chunk of the wave's rows, in LDS order
+      const int row = n / AE_KCPR;
+      const int c = ae_k_swz(n % AE_KCPR, row);
+      int ra = row0 + row;
+      ra = ra < last ? ra : last;
+      off[i] = (unsigned)((ra * stride_s + c * 8) * 2 + 4096 - (i - N / 2) * 1024);
+    }
+    ae_load_lds16_burst_base<N>(qg, off, qs + (G0 + N / 2) * 1024);
+    ae_q_rows_to_lds<G0 + 8>(qg, qs, lane, row0, last, stride_s);
+  }
+}
+
 extern "C" __global__ __launch_bounds__(AE_NT)
 __attribute__((amdgpu_waves_per_eu(AE_WAVES_PER_EU, AE_WAVES_PER_EU)))
 void ae_prefill_kernel(const ae_attn_params p) {
@@ -175,6 +207,15 @@ void ae_prefill_kernel(const ae_attn_params p) {
 
   // ---- Q fragments: B operand of S^T = K Q^T, resident for the whole kernel -------------
   ae_elem8 qf[AE_RB][AE_D / 16];
+#if AE_Q_VIA_LDS
+  ae_lds_byte* qs = lds + AE_STAGE_BYTES + wave * (AE_WROWS * AE_KSTR);
+  {
+    const int q0c = q0w < p.seqlen_q ? q0w : p.seqlen_q - 1;
+    const char* qg = (const char*)((const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)q0c * p.q_stride_s +
+                                   (int64_t)h * p.q_stride_h) - 4096;
+    ae_q_rows_to_lds<0>(qg, qs, lane, q0w - q0c, p.seqlen_q - 1 - q0c, (int)p.q_stride_s);
+  }
+#else
 #pragma unroll
   for (int rb = 0; rb < AE_RB; rb++) {
     const int qr = q_ok[rb] ? qrow[rb] : p.seqlen_q - 1;
@@ -183,6 +224,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #pragma unroll
     for (int ks = 0; ks < AE_D / 16; ks++) qf[rb][ks] = *(const ae_elem8*)(qptr + ks * 16 + hf * 8);
   }
+#endif
 
   // ---- KV tile range ---------------------------------------------------------------------
   const int n_kvt = (p.seqlen_kv + AE_BN - 1) / AE_BN;
@@ -324,6 +366,15 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // iteration wait for that iteration's K/V prefetch, which serialises the pipeline.
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
+#if AE_Q_VIA_LDS
+#pragma unroll
+  for (int rb = 0; rb < AE_RB; rb++)
+#pragma unroll
+    for (int ks = 0; ks < AE_D / 16; ks++)
+      qf[rb][ks] = *(const __attribute__((address_space(3))) ae_elem8*)(
+          qs + (rb * 32 + l32) * AE_KSTR + (ae_k_swz(2 * ks + hf, l32) << 4));
+  __syncthreads();      // every wave has its fragments before the loop's first prefetch refills stage 1
+#endif
 
   int stage = 0;
   while (j < j_end) {
@@ -564,6 +615,29 @@ void ae_prefill_kernel(const ae_attn_params p) {
           p.partial_rs[(int64_t)i * p.batch * p.seqlen_q * p.heads_q * AE_NSPLIT + prow] = frs[i];
       }
     }
+#elif AE_O_VIA_LDS
+    {
+      // (addresses from a copy of the lane id that the compiler cannot trace back to the prologue's, which have
+      // the same form: it would keep those in registers across the loop)
+      int le = lane;
+      asm volatile("" : "+v"(le));
+      ae_lds_byte* orow = lds + wave * (AE_WROWS * AE_VSTR) + (rb * 32 + (le & 31)) * AE_VSTR + (le >> 5) * 8;
+      const int osw = le & (AE_VCPR - 1);
+#pragma unroll
+      for (int db = 0; db < AE_NDB; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int t = 0; t < 4; t++) w[t] = (ae_elem)o[db * 16 + rg * 4 + t];
+          *(__attribute__((address_space(3))) ae_elem4*)(orow + (((db * 4 + rg) ^ osw) << 4)) = w;
+        }
+    }
+    if (q_ok[rb] && hf == 0) {
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+        p.rowscale_out[i][((int64_t)b * p.heads_q + h) * p.seqlen_q + qrow[rb]] = frs[i];
+    }
 #else
     if (q_ok[rb]) {
       ae_elem* optr = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)qrow[rb] * p.o_stride_s +
@@ -585,6 +659,25 @@ void ae_prefill_kernel(const ae_attn_params p) {
     }
 #endif
   }
+#if AE_O_VIA_LDS
+  // (the rows were written by other lanes of this wave: LDS instructions of a wave complete in order)
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  {
+    ae_elem* og = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)h * p.o_stride_h;
+    const ae_lds_byte* os = lds + wave * (AE_WROWS * AE_VSTR);
+    int le = lane;
+    asm volatile("" : "+v"(le));
+#pragma unroll
+    for (int i = 0; i < AE_O_LOADS; i++) {
+      const int n = i * 64 + le;
+      const int row = n / AE_VCPR;
+      const int c = n % AE_VCPR;
+      const ae_elem8 w = *(const __attribute__((address_space(3))) ae_elem8*)(
+          os + row * AE_VSTR + ((c ^ (row & (AE_VCPR - 1))) << 4));
+      if (AE_EVEN_Q || q0w + row < p.seqlen_q) *(ae_elem8*)(og + (int64_t)(q0w + row) * p.o_stride_s + c * 8) = w;
+    }
+  }
+#endif
 #endif  // wide value heads
 }
 
