@@ -119,6 +119,47 @@ AE_DEV int ae_bwd_chunk_pos(int r, int c) {
   return ((((c >> 1) ^ (r & (CPR / 2 - 1))) << 1) | ((c ^ ae_bwd_half_flip<CPR>(r)) & 1));
 }
 
+// Resident rows on their way in and results on their way out pass through LDS as whole rows (16 lanes per
+// 256-byte row), as in the forward kernels: a lane that fetches its own row's fragments, or stores its own row's
+// results, touches 32 rows per instruction, 16 bytes of each, and the workgroups of a launch, which start and end
+// together, queue behind each other's requests.  The resident rows use stages 1 and 2 of the tile ring before the
+// loop starts (the second item is requested once every wave has its fragments), both tensors at once where they
+// fit, else one after the other; the results use the ring after the last item.
+#define AE_R1B (32 * AE_STR1)      // bytes of a wave's resident rows, first tensor
+#define AE_R2B (32 * AE_STR2)
+#define AE_RES_ONEPASS (AE_NWAVES * (AE_R1B + AE_R2B) <= 2 * AE_STAGE_BYTES)
+#define AE_RES_TWOPASS (AE_NWAVES * (AE_R1B > AE_R2B ? AE_R1B : AE_R2B) <= 2 * AE_STAGE_BYTES)
+#define AE_RES_VIA_LDS (AE_NSTAGE == 3 && (AE_RES_ONEPASS || AE_RES_TWOPASS))
+#define AE_OUT_BYTES (AE_R1B + (AE_BWD_ROLE == 1 ? AE_R2B : 0))   // a wave's results
+#define AE_OUT_VIA_LDS (AE_NWAVES * AE_OUT_BYTES <= AE_NSTAGE * AE_STAGE_BYTES)
+
+// 32 rows of CPR 16-byte chunks, HBM -> dst, one burst; LDS chunk c' of row r holds global chunk c' ^ (r mod CPR).
+// g: the wave's first row (clamped into the tensor), 4 KiB low (see ae_load_lds16_burst_base); row0: first row
+// of the wave relative to it; rows past `last` re-read it.
+template <int CPR>
+AE_DEV void ae_bwd_rows_to_lds(const char* g, ae_lds_byte* dst, int lane, int row0, int last, int stride) {
+  constexpr int N = CPR / 2;
+  unsigned off[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int n = (i < N ? i : 0) * 64 + lane;
+    const int row = n / CPR;
+    const int c = (n % CPR) ^ (row & (CPR - 1));
+    int ra = row0 + row;
+    ra = ra < last ? ra : last;
+    off[i] = (unsigned)((ra * stride + c * 8) * 2 + 4096 - (i - N / 2) * 1024);
+  }
+  ae_load_lds16_burst_base<N>(g, off, dst + (N / 2) * 1024);
+}
+// B-operand fragments of row l32 (k = 16*ks + 8*hf + j) from rows laid out by ae_bwd_rows_to_lds
+template <int NKS, int CPR>
+AE_DEV void ae_bwd_frags_from_lds(ae_elem8* rf, const ae_lds_byte* src, int l32, int hf) {
+#pragma unroll
+  for (int ks = 0; ks < NKS; ks++)
+    rf[ks] = *(const __attribute__((address_space(3))) ae_elem8*)(
+        src + l32 * (CPR * 16) + (((2 * ks + hf) ^ (l32 & (CPR - 1))) << 4));
+}
+
 #if AE_BWD_ROLE == 0
 #define AE_BWD_KERNEL ae_bwd_dq_kernel
 #else
@@ -183,10 +224,14 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   ae_bwd_load_custom(cust, p);
 #endif
   ae_elem8 rf1[AE_NKS1], rf2[AE_NKS2];
+#if !AE_RES_VIA_LDS
 #pragma unroll
   for (int ks = 0; ks < AE_NKS1; ks++) rf1[ks] = *(const ae_elem8*)(r1p + ks * 16 + hf * 8);
 #pragma unroll
   for (int ks = 0; ks < AE_NKS2; ks++) rf2[ks] = *(const ae_elem8*)(r2p + ks * 16 + hf * 8);
+#else
+  (void)r1p, (void)r2p;
+#endif
 
 #if AE_BWD_ROLE == 0
   // row scales of the lane's q row: lse in log2 units (+inf for a row without a visible key: p = 0)
@@ -197,7 +242,9 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     lse2_r = p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri];
   }
 #endif
+#if !AE_RES_VIA_LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the resident operands are in registers before any tile request
+#endif
 
   // ---- the streamed items --------------------------------------------------------------------------
   // role 0: kv tiles 0 .. (causal: up to the diagonal); role 1: for every q head of the group, q tiles
@@ -382,12 +429,53 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   // the n-th visited item is multiplied out of stage n % NSTAGE while the next two are on their way
   int cls0, cls1, cls2;                 // ... and the classes of those three items
   int x0 = next_item(0, cls0), x1 = next_item(x0 + 1, cls1), x2 = next_item(x1 + 1, cls2);
+#if AE_RES_VIA_LDS
+  if (x0 < n_items) request_item(x0, 0);
+  {
+    // the wave's 32 resident rows of both tensors travel together with the first item
+    const int rw0 = r0 + wave * 32;
+    const int rw0c = rw0 < n_res ? rw0 : n_res - 1;
+#if AE_BWD_ROLE == 0
+    const char* g1 = (const char*)((const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)rw0c * p.q_stride_s + (int64_t)h * p.q_stride_h);
+    const char* g2 = (const char*)((const ae_elem*)p.dout + (int64_t)b * p.do_stride_b + (int64_t)rw0c * p.do_stride_s + (int64_t)h * p.do_stride_h);
+    const int rs1 = (int)p.q_stride_s, rs2 = (int)p.do_stride_s;
+#else
+    const char* g1 = (const char*)((const ae_elem*)p.k + (int64_t)b * p.k_stride_b + (int64_t)rw0c * p.k_stride_s + (int64_t)h * p.k_stride_h);
+    const char* g2 = (const char*)((const ae_elem*)p.v + (int64_t)b * p.v_stride_b + (int64_t)rw0c * p.v_stride_s + (int64_t)h * p.v_stride_h);
+    const int rs1 = (int)p.k_stride_s, rs2 = (int)p.v_stride_s;
+#endif
+#if AE_RES_ONEPASS
+    ae_lds_byte* rs = lds + AE_STAGE_BYTES + wave * (AE_R1B + AE_R2B);
+    ae_bwd_rows_to_lds<AE_CPR1>(g1 - 4096, rs, lane, rw0 - rw0c, n_res - 1 - rw0c, rs1);
+    ae_bwd_rows_to_lds<AE_CPR2>(g2 - 4096, rs + AE_R1B, lane, rw0 - rw0c, n_res - 1 - rw0c, rs2);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));
+    ae_bwd_frags_from_lds<AE_NKS1, AE_CPR1>(rf1, rs, l32, hf);
+    ae_bwd_frags_from_lds<AE_NKS2, AE_CPR2>(rf2, rs + AE_R1B, l32, hf);
+#else
+    ae_lds_byte* rs = lds + AE_STAGE_BYTES + wave * (AE_R1B > AE_R2B ? AE_R1B : AE_R2B);
+    ae_bwd_rows_to_lds<AE_CPR1>(g1 - 4096, rs, lane, rw0 - rw0c, n_res - 1 - rw0c, rs1);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));
+    ae_bwd_frags_from_lds<AE_NKS1, AE_CPR1>(rf1, rs, l32, hf);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the fragments are out before the rows are replaced
+    ae_bwd_rows_to_lds<AE_CPR2>(g2 - 4096, rs, lane, rw0 - rw0c, n_res - 1 - rw0c, rs2);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));
+    ae_bwd_frags_from_lds<AE_NKS2, AE_CPR2>(rf2, rs, l32, hf);
+#endif
+#if AE_BWD_ROLE == 0
+    // (the row scales were loaded as ordinary loads: used here, their wait falls before the loop and not into it)
+    asm volatile("" :: "v"(lse2_r), "v"(delta_r));
+#endif
+  }
+  __syncthreads();       // every wave has its fragments: stages 1 and 2 go back to the ring
+  if (x0 < n_items) request_item(x1, 1);
+#else
   if (x0 < n_items) {
     request_item(x0, 0);
     if (AE_NSTAGE == 3) request_item(x1, 1);
     __builtin_amdgcn_s_waitcnt(AE_VMCNT((AE_NSTAGE - 2) * AE_NLOADS));   // the first item has landed
   }
   __syncthreads();
+#endif
 
   for (int n = 0; x0 < n_items; n++) {
     const int it = x0;
@@ -555,6 +643,73 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));             // nothing may land in LDS after the workgroup has gone
 
   // ---- results: lane owns its resident row, columns 32*db + 8*(r/4) + 4*hf + r%4 ------------------
+#if AE_OUT_VIA_LDS
+  __syncthreads();       // ... of any wave: the ring becomes the staging area of the results
+  {
+    // (addresses from a copy of the lane id that the compiler cannot trace back to the prologue's)
+    int le = lane;
+    asm volatile("" : "+v"(le));
+    ae_lds_byte* os1 = lds + wave * AE_OUT_BYTES;
+    {
+      ae_lds_byte* orow = os1 + (le & 31) * AE_STR1 + (le >> 5) * 8;
+      const int osw = le & (AE_CPR1 - 1);
+#pragma unroll
+      for (int db = 0; db < AE_NDB1; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int t = 0; t < 4; t++) w[t] = (ae_elem)(acc1[db][rg * 4 + t] * AE_SM_SCALE);
+          *(__attribute__((address_space(3))) ae_elem4*)(orow + (((db * 4 + rg) ^ osw) << 4)) = w;
+        }
+    }
+#if AE_BWD_ROLE == 1
+    {
+      ae_lds_byte* orow = os1 + AE_R1B + (le & 31) * AE_STR2 + (le >> 5) * 8;
+      const int osw = le & (AE_CPR2 - 1);
+#pragma unroll
+      for (int db = 0; db < AE_NDB2; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          ae_elem4 w;
+#pragma unroll
+          for (int t = 0; t < 4; t++) w[t] = (ae_elem)acc2[db][rg * 4 + t];
+          *(__attribute__((address_space(3))) ae_elem4*)(orow + (((db * 4 + rg) ^ osw) << 4)) = w;
+        }
+    }
+#endif
+    // (the rows were written by other lanes of this wave: LDS instructions of a wave complete in order)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int rw0 = r0 + wave * 32;
+#if AE_BWD_ROLE == 0
+    ae_elem* o1 = (ae_elem*)p.dq + (int64_t)b * p.dq_stride_b + (int64_t)h * p.dq_stride_h;
+    const int64_t os1s = p.dq_stride_s;
+#else
+    ae_elem* o1 = (ae_elem*)p.dk + (int64_t)b * p.dk_stride_b + (int64_t)h * p.dk_stride_h;
+    ae_elem* o2 = (ae_elem*)p.dv + (int64_t)b * p.dv_stride_b + (int64_t)h * p.dv_stride_h;
+    const int64_t os1s = p.dk_stride_s, os2s = p.dv_stride_s;
+#endif
+#pragma unroll
+    for (int i = 0; i < AE_CPR1 / 2; i++) {
+      const int n = i * 64 + le;
+      const int row = n / AE_CPR1, c = n % AE_CPR1;
+      const ae_elem8 w = *(const __attribute__((address_space(3))) ae_elem8*)(
+          os1 + row * AE_STR1 + ((c ^ (row & (AE_CPR1 - 1))) << 4));
+      if (rw0 + row < n_res) *(ae_elem8*)(o1 + (int64_t)(rw0 + row) * os1s + c * 8) = w;
+    }
+#if AE_BWD_ROLE == 1
+#pragma unroll
+    for (int i = 0; i < AE_CPR2 / 2; i++) {
+      const int n = i * 64 + le;
+      const int row = n / AE_CPR2, c = n % AE_CPR2;
+      const ae_elem8 w = *(const __attribute__((address_space(3))) ae_elem8*)(
+          os1 + AE_R1B + row * AE_STR2 + ((c ^ (row & (AE_CPR2 - 1))) << 4));
+      if (rw0 + row < n_res) *(ae_elem8*)(o2 + (int64_t)(rw0 + row) * os2s + c * 8) = w;
+    }
+#endif
+  }
+  (void)r_ok;
+#else
   if (r_ok) {
 #if AE_BWD_ROLE == 0
     ae_elem* o1 = (ae_elem*)p.dq + (int64_t)b * p.dq_stride_b + (int64_t)rrow * p.dq_stride_s + (int64_t)h * p.dq_stride_h;
@@ -583,6 +738,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
       }
 #endif
   }
+#endif  // results through LDS
 }
 
 #if AE_BWD_ROLE == 0
