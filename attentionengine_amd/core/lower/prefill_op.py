@@ -312,7 +312,7 @@ class PrefillOp:
             raise ValueError(f"head dims {(D, Dk, v.shape[3])} differ from the compiled {(self.D, self.D, self.DV)}")
         if Bk != B or v.shape[0] != B or v.shape[1] != Skv or v.shape[2] != Hkv or Hq % Hkv:
             raise ValueError("inconsistent q/k/v shapes")
-        q, k, v = (t if t.stride(3) == 1 else t.contiguous() for t in (q, k, v))
+        q, k, v = (rt.rows_for_kernels(t) for t in (q, k, v))
         dev = q.device
 
         if extern_mask is not None and extern_mask is self.block_mask and not self.extern_block_mask:

@@ -367,6 +367,15 @@ class Event:
             pass
 
 
+def rows_for_kernels(t):
+    """``t`` as the kernels can read it: dense in the last dimension, starting on a 16-byte boundary, every
+    other stride a multiple of 8 elements (rows are moved 16 bytes at a time; the C entry points refuse anything
+    else).  Tensors laid out otherwise - a column slice that starts at an odd offset, say - are copied."""
+    if t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(st % 8 == 0 for st in t.stride()[:-1]):
+        return t
+    return t.contiguous()
+
+
 def prefill_fwd(kernel: Kernel, params: AttnParams, cfg: TileCfg, stream: int = 0):
     _check(lib().ae_prefill_fwd(kernel.handle, C.byref(params), C.byref(cfg), _VP(stream)))
 

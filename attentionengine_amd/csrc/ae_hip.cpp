@@ -4,6 +4,7 @@
 // Host-only translation unit (built with g++ or hipcc); links libamdhip64 + libhiprtc.  The library's
 // second translation unit, ae_noalloc.hip, carries its one piece of device data.
 
+#include <cstdint>
 #include "ae_hip.h"
 
 #include <hip/hip_runtime_api.h>
@@ -335,6 +336,20 @@ static int check_common(const char* who, const ae_attn_params* p, const ae_tile_
                   who, p->mask_nq, p->mask_nkv, p->mask_block_m, p->mask_block_n, p->seqlen_q,
                   p->seqlen_kv);
   }
+  // the kernels move 16-byte pieces of rows: every tensor starts on a 16-byte boundary and its batch / position /
+  // head strides are multiples of 8 elements (the last dimension is dense)
+  const void* ptrs[] = {p->q, p->k, p->v, p->out, p->q2, p->k2};
+  for (const void* ptr : ptrs)
+    if (ptr && ((uintptr_t)ptr & 15) != 0)
+      return fail(AE_ERR_INVALID_ARG, "%s: q / k / v / out must start on a 16-byte boundary", who);
+  const int64_t strides[] = {p->q_stride_b, p->q_stride_s, p->q_stride_h, p->k_stride_b, p->k_stride_s, p->k_stride_h,
+                             p->v_stride_b, p->v_stride_s, p->v_stride_h, p->o_stride_b, p->o_stride_s, p->o_stride_h,
+                             p->q2 ? p->q2_stride_b : 0, p->q2 ? p->q2_stride_s : 0, p->q2 ? p->q2_stride_h : 0,
+                             p->k2 ? p->k2_stride_b : 0, p->k2 ? p->k2_stride_s : 0, p->k2 ? p->k2_stride_h : 0};
+  for (int64_t st : strides)
+    if (st % 8 != 0)
+      return fail(AE_ERR_INVALID_ARG, "%s: a stride of %lld elements is not a multiple of 8 (rows are moved 16 bytes at a time)",
+                  who, (long long)st);
   return AE_OK;
 }
 
@@ -542,6 +557,20 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
   if (p->heads_q % p->heads_kv != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: Hq=%d is not a multiple of Hkv=%d", p->heads_q,
                 p->heads_kv);
+  {
+    const void* ptrs[] = {p->q, p->k, p->v, p->out, p->dout, p->dq, p->dk, p->dv};
+    for (const void* ptr : ptrs)
+      if (((uintptr_t)ptr & 15) != 0)
+        return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: the tensors must start on a 16-byte boundary");
+    const int64_t strides[] = {p->q_stride_b, p->q_stride_s, p->q_stride_h, p->k_stride_b, p->k_stride_s, p->k_stride_h,
+                               p->v_stride_b, p->v_stride_s, p->v_stride_h, p->o_stride_b, p->o_stride_s, p->o_stride_h,
+                               p->do_stride_b, p->do_stride_s, p->do_stride_h, p->dq_stride_b, p->dq_stride_s, p->dq_stride_h,
+                               p->dk_stride_b, p->dk_stride_s, p->dk_stride_h, p->dv_stride_b, p->dv_stride_s, p->dv_stride_h};
+    for (int64_t st : strides)
+      if (st % 8 != 0)
+        return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: a stride of %lld elements is not a multiple of 8 (rows are moved 16 bytes at a time)",
+                    (long long)st);
+  }
   // block_m / threads describe the dq launch (4 or 8 waves of 32 resident rows); dk/dv always runs 4 waves
   if ((cfg->block_m != 128 && cfg->block_m != 256) || cfg->block_n != 64 || cfg->threads != 2 * cfg->block_m || cfg->lds_bytes <= 0 ||
       cfg->lds_bytes > 160 * 1024 || cfg->head_dim_v <= 0 || cfg->head_dim_v % 8 != 0)

@@ -21,6 +21,9 @@
  *     buffers before a launch; device pointers are passed inside ae_attn_params
  *     together with their strides in ELEMENTS (the layout of Flash_fwd_params,
  *     core/template/cute_template/flash.h:14-60, reduced to what the forward needs).
+ *     The kernels move rows 16 bytes at a time: the last dimension is dense, every
+ *     tensor starts on a 16-byte boundary and every stride is a multiple of 8
+ *     elements; the launch functions refuse anything else (AE_ERR_INVALID_ARG).
  *   - launches are asynchronous on the caller's HIP stream (`void* stream` is a
  *     hipStream_t; NULL is the default stream). The library never synchronises the
  *     device except inside ae_event_elapsed_ms().

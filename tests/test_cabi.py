@@ -164,6 +164,43 @@ def test_paged_cache_arguments_are_checked_before_any_launch():
     assert "reads a dense cache" in lib.ae_last_error().decode()
 
 
+def test_misaligned_tensors_are_refused_before_any_launch():
+    """The kernels move rows 16 bytes at a time: a tensor that does not start on a 16-byte boundary, or whose
+    strides are not multiples of 8 elements, is refused by the argument checks (the Python operators copy such
+    views first, core/runtime/hip_rt.py::rows_for_kernels)."""
+    lib = rt.lib()
+    fake = ctypes.c_void_p(8)
+    buf = ctypes.create_string_buffer(256)
+    addr = (ctypes.addressof(buf) + 15) & ~15
+
+    def params(**kw):
+        p = rt.AttnParams()
+        p.q = p.k = p.v = p.out = addr
+        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = 1, 2, 2, 64, 64
+        p.q_stride_b = p.k_stride_b = p.v_stride_b = p.o_stride_b = 64 * 2 * 64
+        p.q_stride_s = p.k_stride_s = p.v_stride_s = p.o_stride_s = 2 * 64
+        p.q_stride_h = p.k_stride_h = p.v_stride_h = p.o_stride_h = 64
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
+
+    cfg = rt.TileCfg(block_m=128, block_n=64, threads=256, lds_bytes=1024, head_dim=64, head_dim_v=64,
+                     elem_bytes=2, n_rowscales=0, mask_mode=0)
+    for bad in (dict(q=addr + 8), dict(out=addr + 2), dict(k_stride_s=2 * 64 + 4), dict(v_stride_h=60)):
+        assert lib.ae_prefill_fwd(fake, ctypes.byref(params(**bad)), ctypes.byref(cfg), None) == 1, bad
+        msg = lib.ae_last_error().decode()
+        assert "16-byte boundary" in msg or "not a multiple of 8" in msg, msg
+    bp = rt.AttnBwdParams()
+    for name in ("q", "k", "v", "out", "dout", "delta", "dq", "dk", "dv"):
+        setattr(bp, name, addr)
+    bp.batch, bp.heads_q, bp.heads_kv, bp.seqlen_q, bp.seqlen_kv = 1, 2, 2, 64, 64
+    bp.dq = addr + 4
+    bcfg = rt.TileCfg(block_m=128, block_n=64, threads=256, lds_bytes=1024, head_dim=64, head_dim_v=64,
+                      elem_bytes=2, n_rowscales=0, mask_mode=0)
+    assert lib.ae_prefill_bwd(fake, fake, fake, ctypes.byref(bp), ctypes.byref(bcfg), None) == 1
+    assert "16-byte boundary" in lib.ae_last_error().decode()
+
+
 @pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")
 def test_no_gpu_is_reported_not_hidden():
     lib = rt.lib()

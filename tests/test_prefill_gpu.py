@@ -325,6 +325,33 @@ def test_gqa_prefill(cuda_device):
     assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
+def test_views_of_a_packed_projection(cuda_device):
+    """q, k and v as column slices of one packed [B, S, H, 3D + 4] tensor: the slices that start on a 16-byte
+    boundary are read in place (strided rows), the ones shifted by 4 elements are copied first; forward and
+    backward agree with the oracle either way."""
+    B, H, S, D = 1, 4, 300, 64
+    dtype = torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    ref, lse = R.softmax_attention(q, k, v, causal=True)
+    dq_ref, dk_ref, dv_ref = R.softmax_attention_grads(q, k, v, torch.ones_like(ref), causal=True)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask, C.OnlineSoftmax())
+    for shift in (0, 4):
+        packed = torch.zeros(B, S, H, 3 * D + 4, dtype=dtype, device="cuda")
+        views = [packed[..., shift + i * D: shift + (i + 1) * D] for i in range(3)]
+        for dst, src in zip(views, (q, k, v)):
+            dst.copy_(src)
+        assert all(t.data_ptr() % 16 == (2 * shift) % 16 for t in views)
+        packed.requires_grad_()
+        qv, kv, vv = (packed[..., shift + i * D: shift + (i + 1) * D] for i in range(3))
+        out = mod(qv, kv, vv)
+        assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL, shift
+        assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL, shift
+        out.backward(torch.ones_like(out))
+        g = packed.grad.float().cpu()
+        for i, gr in enumerate((dq_ref, dk_ref, dv_ref)):
+            assert (g[..., shift + i * D: shift + (i + 1) * D] - gr).abs().max().item() <= 2e-2, (shift, i)
+
+
 def test_abs_norm_online_func(cuda_device):
     """An OnlineFunc other than softmax: running abs-sum normalisation with a clamp."""
     from oracle.online_interp import online_attention
