@@ -411,4 +411,5 @@ def mla_decode_fwd(split: Kernel, combine: Kernel, params: AttnParams, cfg: Tile
 
 
 def prefill_bwd(delta: Kernel, dkv: Kernel, dq: Kernel, params: AttnBwdParams, cfg: TileCfg, stream: int = 0):
-    _check(lib().ae_prefill_bwd(delta.handle, dkv.handle, dq.handle, C.byref(params), C.byref(cfg), _VP(stream)))
+    _check(lib().ae_prefill_bwd(delta.handle if delta is not None else None, dkv.handle, dq.handle, C.byref(params),
+                                C.byref(cfg), _VP(stream)))

@@ -547,7 +547,8 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
 
 int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
                    const ae_tile_cfg* cfg, void* stream) {
-  if (!delta || !dkv || !dq) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: kernel is NULL");
+  // delta == NULL: kernels built with AE_BWD_FUSE_DELTA 1 - the dq launch fills the work buffer and goes first
+  if (!dkv || !dq) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: kernel is NULL");
   if (!p || !cfg) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: params/cfg is NULL");
   if (!p->q || !p->k || !p->v || !p->out || !p->dout || !p->delta || !p->dq || !p->dk || !p->dv)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: a tensor pointer is NULL");
@@ -593,7 +594,18 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: grid too large");
   uint32_t block[3] = {256, 1, 1};
   uint32_t grid[3] = {(uint32_t)g_delta, 1, 1};
-  int rc = ae_launch(delta, p, sizeof *p, grid, block, 0, stream);
+  int rc;
+  if (!delta) {
+    if (!p->lse) return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: the dq launch forms the row scales from lse, which is NULL");
+    grid[0] = (uint32_t)g_dq;
+    block[0] = (uint32_t)cfg->threads;
+    rc = ae_launch(dq, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+    if (rc) return rc;
+    grid[0] = (uint32_t)g_dkv;
+    block[0] = 256;
+    return ae_launch(dkv, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
+  }
+  rc = ae_launch(delta, p, sizeof *p, grid, block, 0, stream);
   if (rc) return rc;
   grid[0] = (uint32_t)g_dkv;
   rc = ae_launch(dkv, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);

@@ -132,6 +132,14 @@ AE_DEV int ae_bwd_chunk_pos(int r, int c) {
 #define AE_RES_VIA_LDS (AE_NSTAGE == 3 && (AE_RES_ONEPASS || AE_RES_TWOPASS))
 #define AE_OUT_BYTES (AE_R1B + (AE_BWD_ROLE == 1 ? AE_R2B : 0))   // a wave's results
 #define AE_OUT_VIA_LDS (AE_NWAVES * AE_OUT_BYTES <= AE_NSTAGE * AE_STAGE_BYTES)
+// 1 (softmax attention, set by the host with both launches): there is no ae_bwd_delta_kernel launch.  The dq
+// launch, which holds the dO rows anyway, fetches its O rows behind them, forms rowsum(dO * O) and writes both
+// planes of the work buffer; the dk/dv launch runs after it.  (The separate launch read O and dO once more:
+// 28 us and 138 MB of the C2 causal backward.)
+#ifndef AE_BWD_FUSE_DELTA
+#define AE_BWD_FUSE_DELTA 0
+#endif
+static_assert(!AE_BWD_FUSE_DELTA || (AE_RES_VIA_LDS && AE_BWD_KIND == 0), "the fused row sums need the staged resident rows");
 
 // 32 rows of CPR 16-byte chunks, HBM -> dst, one burst; LDS chunk c' of row r holds global chunk c' ^ (r mod CPR).
 // g: the wave's first row (clamped into the tensor), 4 KiB low (see ae_load_lds16_burst_base); row0: first row
@@ -238,8 +246,14 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
   float lse2_r, delta_r;
   {
     const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + rrow_c;
+#if AE_BWD_FUSE_DELTA
+    const float l = p.lse[ri];
+    lse2_r = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;     // +inf: a row without a visible key, p = 0
+    delta_r = 0.f;                                                    // formed below, once dO and O are here
+#else
     delta_r = p.delta[ri];
     lse2_r = p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri];
+#endif
   }
 #endif
 #if !AE_RES_VIA_LDS
@@ -460,6 +474,29 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     ae_bwd_rows_to_lds<AE_CPR2>(g2 - 4096, rs, lane, rw0 - rw0c, n_res - 1 - rw0c, rs2);
     __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));
     ae_bwd_frags_from_lds<AE_NKS2, AE_CPR2>(rf2, rs, l32, hf);
+#endif
+#if AE_BWD_ROLE == 0 && AE_BWD_FUSE_DELTA
+    {
+      // rowsum(dO * O) of the lane's row: the O rows follow the dO rows through the staging region, are read in
+      // the same fragment layout, and the two lanes that share a row add their halves
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      const char* g3 = (const char*)((const ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)rw0c * p.o_stride_s + (int64_t)h * p.o_stride_h);
+      ae_bwd_rows_to_lds<AE_CPR2>(g3 - 4096, rs, lane, rw0 - rw0c, n_res - 1 - rw0c, (int)p.o_stride_s);
+      __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));
+      ae_elem8 of[AE_NKS2];
+      ae_bwd_frags_from_lds<AE_NKS2, AE_CPR2>(of, rs, l32, hf);
+      float acc = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < AE_NKS2; ks++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc += (float)of[ks][j] * (float)rf2[ks][j];
+      delta_r = acc + __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, acc)));
+      if (r_ok && hf == 0) {
+        const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + rrow;
+        p.delta[ri] = delta_r;
+        p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = lse2_r;
+      }
+    }
 #endif
 #if AE_BWD_ROLE == 0
     // (the row scales were loaded as ordinary loads: used here, their wait falls before the loop and not into it)

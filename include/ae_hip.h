@@ -279,6 +279,8 @@ int ae_mla_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params
  *   element, 2 fully visible); head dims as compiled. All gradients are written in full (no accumulation).
  *   The same three launches serve the graphs whose online function does nothing (sigmoid, relu attention:
  *   kernels compiled with AE_BWD_KIND 1 and the generated derivative of score_mod; lse is NULL then).
+ *   `delta` may be NULL for softmax kernels compiled with AE_BWD_FUSE_DELTA 1: the dq launch then forms
+ *   rowsum(dout*out) for its own rows, fills the work buffer and runs first, dkv second (two launches).
  */
 int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_attn_bwd_params* p,
                    const ae_tile_cfg* cfg, void* stream);
