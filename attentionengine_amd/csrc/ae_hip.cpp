@@ -395,12 +395,18 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
   if (p->kv_per_split % cfg->block_n != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: kv_per_split=%d is not a multiple of block_n=%d",
                 p->kv_per_split, cfg->block_n);
-  if (!p->partial_o || !p->partial_rs)
-    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
-  if (!combine || !combine_cfg)
-    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel is NULL");
   // one partial per wave: a workgroup of W waves produces W consecutive partials
   int waves = cfg->threads / 64;
+  // combine == NULL: a split kernel built with AE_MERGE_IN_WG 1, whose one workgroup per (batch, kv head, head
+  // tile) merges its waves' partial results itself and writes out; no work buffers
+  const bool merged = (combine == nullptr);
+  if (merged && p->num_splits != waves)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: without a combine kernel the %d splits must be the %d waves of one workgroup",
+                p->num_splits, waves);
+  if (!merged && (!p->partial_o || !p->partial_rs))
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
+  if (!merged && !combine_cfg)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel is NULL");
   if (p->num_splits % waves != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: num_splits=%d is not a multiple of %d waves",
                 p->num_splits, waves);
@@ -413,7 +419,7 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                       (uint32_t)p->batch};
   uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
   rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
-  if (rc) return rc;
+  if (rc || merged) return rc;
   if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: bad combine workgroup size %d",
                 combine_cfg->threads);

@@ -237,7 +237,9 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
  *   (attn_gqa_decode_tl.py:150-151, 224-266). Every WAVE of the split kernel produces one partial,
  *   so its grid is (num_splits / (threads/64), ceil(Hq/Hkv / block_m)*Hkv, B); kv_per_split is the
  *   share of one partial and must be a multiple of block_n; combine_cfg->block_n is the number of
- *   splits the combine kernel was compiled for and must equal num_splits.
+ *   splits the combine kernel was compiled for and must equal num_splits.  `combine` may be NULL for a
+ *   split kernel compiled with AE_MERGE_IN_WG 1 when num_splits equals the waves of one workgroup: that
+ *   workgroup merges its waves' partial results itself and writes out (one launch, no work buffers).
  */
 int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream);
 int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
