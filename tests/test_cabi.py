@@ -162,6 +162,10 @@ def test_paged_cache_arguments_are_checked_before_any_launch():
     cc = rt.TileCfg(block_m=1, block_n=1, threads=128)
     assert lib.ae_decode_fwd(fake, fake, ctypes.byref(p), ctypes.byref(cfg()), ctypes.byref(cc), None) == 1
     assert "reads a dense cache" in lib.ae_last_error().decode()
+    # without a merge kernel the splits must be the waves of one workgroup
+    p = params(num_splits=16, kv_per_split=32)
+    assert lib.ae_decode_fwd(fake, None, ctypes.byref(p), ctypes.byref(cfg(threads=256)), None, None) == 1
+    assert "must be the 4 waves of one workgroup" in lib.ae_last_error().decode()
 
 
 def test_misaligned_tensors_are_refused_before_any_launch():

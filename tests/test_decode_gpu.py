@@ -40,6 +40,33 @@ def test_gqa_decode(cuda_device, B, Hq, Hkv, Skv, D, dtype):
     assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Skv,D,dtype", [
+    (64, 16, 4, 500, 64, torch.float16),       # ragged kv, fewer keys in the last waves' tiles
+    (64, 40, 2, 160, 128, torch.bfloat16),     # 20 heads per group: a full and a partly filled head tile
+    (256, 8, 1, 40, 128, torch.float16),       # two tiles for four waves: two partial results are empty
+])
+def test_gqa_decode_merged_in_the_workgroup(cuda_device, monkeypatch, B, Hq, Hkv, Skv, D, dtype):
+    """Launches with one workgroup per (batch, kv head, head tile) merge their waves' partial results in LDS and
+    write out themselves (one launch, no work buffers): against the oracle, and bit for bit against the same
+    launch followed by the merge kernel (attn_gqa_decode_tl.py:224-266)."""
+    print(f"case merged gqa decode B{B} Hq{Hq} Hkv{Hkv} Skv{Skv} D{D} {dtype}", flush=True)
+    q, k, v = C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, dtype)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    res = {}
+    for merge in ("1", "0"):
+        monkeypatch.setenv("AE_DECODE_MERGE_IN_WG", merge)
+        mod = _decode_engine(B, Hq, Hkv, Skv, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.OnlineSoftmax())
+        op = mod.attention
+        n_split, _ = op.plan_splits(B, Hq, Hkv, Skv)
+        assert n_split == op.N_WAVES and op.merges_in_workgroup(n_split) == (merge == "1")
+        res[merge] = (mod(qc, kc, vc).clone(), mod.final_rowscales["lse"].clone())
+    assert torch.equal(res["1"][0], res["0"][0]) and torch.equal(res["1"][1], res["0"][1])
+    for b in (0, B - 1):
+        ref, lse = R.softmax_attention(q[b:b + 1], k[b:b + 1], v[b:b + 1], causal=False)
+        assert (res["1"][0][b:b + 1].float().cpu() - ref).abs().max().item() <= OUT_TOL
+        assert (res["1"][1][b:b + 1].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
 def test_gqa_decode_full_size_properties(cuda_device):
     """BASELINE config 4 at full size (B64 Hq32 Hkv8 Skv8192 D128 fp16).  Checked against the oracle
     on two batch entries, and everywhere through linearity in V: decode(q, k, a*v1 + v2) ==
