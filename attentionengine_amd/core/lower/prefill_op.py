@@ -241,6 +241,12 @@ class PrefillOp:
             return 0
         return self.tiles.n_waves * (self.tiles.rows_per_wave // 32) * 2560
 
+    def _clock_stamps(self):
+        """AE_CLOCK_STAMPS=1 (a measurement switch, read by ``bench.py --mfma-probe``): the pipelined kernel is
+        built so that every workgroup reports the shader-clock cycles and the 100 MHz ticks it ran for; the
+        pairs of the last launch are kept on ``self.clock_stamps`` (int64 [workgroups, 2])."""
+        return os.environ.get("AE_CLOCK_STAMPS", "") == "1" and self.tiles.template == "ae_prefill_pipe.hip"
+
     def _table_rows(self, mask_block_m):
         """Block-table rows a q tile spans (1, 2, 4 or 8): the kernels keep that many pairs of 64-bit masks."""
         if not mask_block_m:
@@ -265,13 +271,15 @@ class PrefillOp:
                 cfg_src += f"#define AE_TT_ROWS {table_rows}\n#define AE_HEAVY_LAST {1 if heavy_last else 0}\n"
             if n_split > 1:
                 cfg_src += f"#define AE_NSPLIT {n_split}\n#define AE_COMBINE_THREADS {self.COMBINE_THREADS}\n"
+            if self._clock_stamps():
+                cfg_src += "#define AE_CLOCK_STAMPS 1\n"
             module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,
                                                           "ae_functors.h": self.functor_src})
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
                              threads=64 * self.tiles.n_waves,
                              lds_bytes=self.tiles.lds_bytes(self.D, self.DV_launch) + self._kv_custom_scratch(), head_dim=self.D,
                              head_dim_v=self.DV_launch, elem_bytes=2, n_rowscales=self.n_rowscales,
-                             mask_mode=mask_mode)
+                             mask_mode=mask_mode, table_rows=table_rows if mask_mode == 2 else 0)
             v = self._variants[key] = (module, cfg, cfg_src)
         return v
 
@@ -379,6 +387,10 @@ class PrefillOp:
             rt.prefill_split_fwd(kern, module.kernel("ae_decode_combine_kernel"), p, cfg, ccfg, stream)
             rowscales = [r.transpose(1, 2).contiguous() for r in rowscales]
         else:
+            if self._clock_stamps():
+                n_wg = -(-Sq // self.tiles.block_m) * (-(-(B * Hq) // 8) * 8)
+                self.clock_stamps = torch.zeros((n_wg, 2), dtype=torch.int64, device=dev)
+                p.partial_o = self.clock_stamps.data_ptr()
             # one launch per slice of DV_launch value columns (a single one unless DV > 256)
             esz = v.element_size()
             for c0 in range(0, self.DV, self.DV_launch):

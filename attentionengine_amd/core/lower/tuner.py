@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import json
 import os
+import tempfile
 
 import torch
 
@@ -33,14 +34,36 @@ def problem_keys(q_shape, dim, dimv):
             "seq_len": ext(q_shape[2], "seq_len"), "dim": int(dim), "dimv": int(dimv)}
 
 
+def _salvage(text):
+    """The complete records of a damaged file (a write that was cut short, two writers): every json object
+    that still parses and carries a ``tuned_config``."""
+    dec, recs, pos = json.JSONDecoder(), [], 0
+    while True:
+        pos = text.find("{", pos)
+        if pos < 0:
+            return recs
+        try:
+            obj, end = dec.raw_decode(text, pos)
+        except ValueError:
+            pos += 1
+            continue
+        if isinstance(obj, dict) and "tuned_config" in obj:
+            recs.append(obj)
+        pos = end
+
+
 def _records(tune_file):
     if not tune_file or not os.path.exists(tune_file):
         return []
     try:
         with open(tune_file) as f:
-            recs = json.load(f)
-    except (OSError, ValueError):
+            text = f.read()
+    except OSError:
         return []
+    try:
+        recs = json.loads(text)
+    except ValueError:
+        return _salvage(text)
     return recs if isinstance(recs, list) else []
 
 
@@ -53,12 +76,24 @@ def lookup(tune_file, pk):
 
 
 def store(tune_file, pk, tuned_config):
-    """Adds (or replaces) the record of this problem; the other records of the file are kept."""
+    """Adds (or replaces) the record of this problem; the other records of the file are kept.  The new contents
+    go to a temporary file of this process in the same directory, which then replaces ``tune_file`` in one step:
+    a reader never sees half a file, and a crash in the middle leaves the old one."""
     recs = [r for r in _records(tune_file)
             if not (isinstance(r, dict) and all(r.get(k) == v for k, v in pk.items()))]
     recs.append({**pk, "tuned_config": list(tuned_config)})
-    with open(tune_file, "w") as f:
-        json.dump(recs, f, indent=4)
+    d = os.path.dirname(os.path.abspath(tune_file))
+    fd, tmp = tempfile.mkstemp(prefix=os.path.basename(tune_file) + ".", suffix=".tmp", dir=d)
+    try:
+        with os.fdopen(fd, "w") as f:
+            json.dump(recs, f, indent=4)
+        os.replace(tmp, tune_file)
+    except BaseException:
+        try:
+            os.unlink(tmp)
+        except OSError:
+            pass
+        raise
 
 
 def prefill_candidates(d, dv, softmax, elementwise):

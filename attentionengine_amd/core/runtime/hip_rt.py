@@ -87,7 +87,7 @@ class TileCfg(C.Structure):
         ("block_m", C.c_int32), ("block_n", C.c_int32), ("threads", C.c_int32),
         ("lds_bytes", C.c_int32), ("head_dim", C.c_int32), ("head_dim_v", C.c_int32),
         ("elem_bytes", C.c_int32), ("n_rowscales", C.c_int32), ("mask_mode", C.c_int32),
-        ("paged", C.c_int32), ("reserved", C.c_int32 * 2),
+        ("paged", C.c_int32), ("merge_in_wg", C.c_int32), ("table_rows", C.c_int32),
     ]
 
 

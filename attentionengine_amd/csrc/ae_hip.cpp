@@ -353,6 +353,30 @@ static int check_common(const char* who, const ae_attn_params* p, const ae_tile_
   return AE_OK;
 }
 
+// mask_mode 2: the block table's geometry against the kernel's tiles (shared by ae_prefill_fwd and
+// ae_prefill_split_fwd)
+static int check_block_table_geometry(const char* who, const ae_attn_params* p, const ae_tile_cfg* cfg) {
+  if (cfg->mask_mode != 2) return AE_OK;
+  if (cfg->block_m % p->mask_block_m != 0 && p->mask_block_m % cfg->block_m != 0)
+    return fail(AE_ERR_INVALID_ARG, "%s: mask block rows %d incompatible with tile %d", who,
+                p->mask_block_m, cfg->block_m);
+  // a kv tile must lie inside ONE column of the table: the kernels classify a tile by the column of its
+  // first key
+  if (p->mask_block_n % cfg->block_n != 0)
+    return fail(AE_ERR_INVALID_ARG, "%s: block-mask columns of %d keys are not a multiple of the %d-key kv tile",
+                who, p->mask_block_n, cfg->block_n);
+  // a q tile spans ceil(block_m / mask_block_m) table rows; the kernel keeps masks for the AE_TT_ROWS it was
+  // compiled with and would apply the last of them to every further row
+  if (cfg->table_rows < 0)
+    return fail(AE_ERR_INVALID_ARG, "%s: table_rows=%d", who, cfg->table_rows);
+  const int compiled_rows = cfg->table_rows ? cfg->table_rows : 8;
+  const int spanned = (cfg->block_m + p->mask_block_m - 1) / p->mask_block_m;
+  if (spanned > compiled_rows)
+    return fail(AE_ERR_INVALID_ARG, "%s: a %d-row q tile spans %d rows of a table with %d-row blocks, the kernel was "
+                "compiled for %d", who, cfg->block_m, spanned, p->mask_block_m, compiled_rows);
+  return AE_OK;
+}
+
 int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream) {
   if (!k) return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: kernel is NULL");
   int rc = check_common("ae_prefill_fwd", p, cfg);
@@ -360,14 +384,8 @@ int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg
   for (int i = 0; i < cfg->n_rowscales; i++)
     if (!p->rowscale_out[i])
       return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: rowscale_out[%d] is NULL", i);
-  if (cfg->mask_mode == 2 && (cfg->block_m % p->mask_block_m != 0 && p->mask_block_m % cfg->block_m != 0))
-    return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: mask block rows %d incompatible with tile %d",
-                p->mask_block_m, cfg->block_m);
-  // a kv tile must lie inside ONE column of the table: the kernels classify a tile by the column of its
-  // first key
-  if (cfg->mask_mode == 2 && p->mask_block_n % cfg->block_n != 0)
-    return fail(AE_ERR_INVALID_ARG, "ae_prefill_fwd: block-mask columns of %d keys are not a multiple of the %d-key kv tile",
-                p->mask_block_n, cfg->block_n);
+  rc = check_block_table_geometry("ae_prefill_fwd", p, cfg);
+  if (rc) return rc;
   // ids are 8*slot + xcd with slot = (batch*head / 8)*q_tiles + q_tile, see ae_prefill.hip
   uint64_t q_tiles = ((uint64_t)p->seqlen_q + cfg->block_m - 1) / cfg->block_m;
   uint64_t bh = (uint64_t)p->heads_q * (uint64_t)p->batch;
@@ -380,8 +398,9 @@ int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg
   return ae_launch(k, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
 }
 
-int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
-                  const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
+// launch == false: only the argument checks (ae_decode_fwd_noalloc runs them before it touches the device)
+static int decode_fwd_impl(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                           const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream, bool launch) {
   if (!split) return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split kernel is NULL");
   int rc = check_common("ae_decode_fwd", p, cfg);
   if (rc) return rc;
@@ -397,16 +416,29 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                 p->kv_per_split, cfg->block_n);
   // one partial per wave: a workgroup of W waves produces W consecutive partials
   int waves = cfg->threads / 64;
-  // combine == NULL: a split kernel built with AE_MERGE_IN_WG 1, whose one workgroup per (batch, kv head, head
-  // tile) merges its waves' partial results itself and writes out; no work buffers
-  const bool merged = (combine == nullptr);
+  // cfg->merge_in_wg: the split kernel was built with AE_MERGE_IN_WG 1 - its one workgroup per (batch, kv head,
+  // head tile) merges its waves' partial results itself and writes out; no combine kernel, no work buffers.
+  // The host cannot see how a kernel was compiled, so the flag travels with the tile configuration: a kernel
+  // built WITHOUT the merge stores its partials through p->partial_o and must never run with NULL buffers.
+  if (cfg->merge_in_wg != 0 && cfg->merge_in_wg != 1)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: merge_in_wg=%d", cfg->merge_in_wg);
+  const bool merged = cfg->merge_in_wg == 1;
+  if (merged && combine)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel that merges in the workgroup takes no combine kernel");
   if (merged && p->num_splits != waves)
-    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: without a combine kernel the %d splits must be the %d waves of one workgroup",
-                p->num_splits, waves);
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel that merges in the workgroup needs the %d splits to be "
+                "the %d waves of one workgroup", p->num_splits, waves);
+  if (!merged && !combine)
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel is NULL and the split kernel does not merge in the "
+                "workgroup (cfg->merge_in_wg is 0)");
   if (!merged && (!p->partial_o || !p->partial_rs))
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
   if (!merged && !combine_cfg)
-    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine kernel is NULL");
+    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: combine configuration is NULL");
+  if (merged)     // the split kernel itself writes the merged row scales
+    for (int i = 0; i < cfg->n_rowscales; i++)
+      if (!p->rowscale_out[i])
+        return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: rowscale_out[%d] is NULL", i);
   if (p->num_splits % waves != 0)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: num_splits=%d is not a multiple of %d waves",
                 p->num_splits, waves);
@@ -418,17 +450,32 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
   uint32_t grid[3] = {(uint32_t)(p->num_splits / waves), (uint32_t)(head_tiles * p->heads_kv),
                       (uint32_t)p->batch};
   uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
+  if (!merged) {
+    if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
+      return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: bad combine workgroup size %d",
+                  combine_cfg->threads);
+    for (int i = 0; i < combine_cfg->n_rowscales; i++)
+      if (!p->rowscale_out[i])
+        return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: rowscale_out[%d] is NULL", i);
+  }
+  if (!launch) return AE_OK;
   rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
   if (rc || merged) return rc;
-  if (combine_cfg->threads <= 0 || combine_cfg->threads % 64 != 0 || combine_cfg->threads > 1024)
-    return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: bad combine workgroup size %d",
-                combine_cfg->threads);
-  for (int i = 0; i < combine_cfg->n_rowscales; i++)
-    if (!p->rowscale_out[i])
-      return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: rowscale_out[%d] is NULL", i);
   uint32_t cgrid[3] = {(uint32_t)p->heads_q, (uint32_t)p->batch, 1};
   uint32_t cblock[3] = {(uint32_t)combine_cfg->threads, 1, 1};
   return ae_launch(combine, p, sizeof *p, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);
+}
+
+int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
+                  const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream) {
+  return decode_fwd_impl(split, combine, p, cfg, combine_cfg, stream, true);
+}
+
+// for ae_noalloc.hip: the checks of ae_decode_fwd without the launches
+extern "C" __attribute__((visibility("hidden"))) int ae_internal_decode_check(
+    ae_kernel* split, ae_kernel* combine, const ae_attn_params* p, const ae_tile_cfg* cfg,
+    const ae_tile_cfg* combine_cfg) {
+  return decode_fwd_impl(split, combine, p, cfg, combine_cfg, nullptr, false);
 }
 
 int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
@@ -436,6 +483,8 @@ int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_par
   if (!split || !combine || !combine_cfg)
     return fail(AE_ERR_INVALID_ARG, "ae_prefill_split_fwd: kernel/cfg is NULL");
   int rc = check_common("ae_prefill_split_fwd", p, cfg);
+  if (rc) return rc;
+  rc = check_block_table_geometry("ae_prefill_split_fwd", p, cfg);
   if (rc) return rc;
   if (p->num_splits <= 1 || p->kv_per_split <= 0 ||
       (int64_t)p->num_splits * p->kv_per_split < p->seqlen_kv)

@@ -25,6 +25,10 @@ static __device__ __align__(256) unsigned char scratch[AE_NOALLOC_SCRATCH_BYTES]
 
 // defined in ae_hip.cpp: sets the calling thread's ae_last_error text and returns `code`
 extern "C" __attribute__((visibility("hidden"))) int ae_internal_fail(int code, const char* fmt, ...);
+// defined in ae_hip.cpp: every argument check of ae_decode_fwd, no launch
+extern "C" __attribute__((visibility("hidden"))) int ae_internal_decode_check(
+    ae_kernel* split, ae_kernel* combine, const ae_attn_params* p, const ae_tile_cfg* cfg,
+    const ae_tile_cfg* combine_cfg);
 
 namespace {
 
@@ -74,10 +78,16 @@ extern "C" int ae_decode_fwd_noalloc(ae_kernel* split, ae_kernel* combine, const
                             "the built-in buffer holds %llu (use ae_decode_fwd with caller-allocated buffers)",
                             p->batch, p->heads_q, p->num_splits, cfg->head_dim_v,
                             (unsigned long long)(o_bytes + rs_bytes), (unsigned long long)AE_NOALLOC_SCRATCH_BYTES);
-  unsigned char* base = nullptr;
-  int rc = scratch_address(&base);
-  if (rc) return rc;
+  // every check of ae_decode_fwd runs before the device is touched (the work buffers stand in as non-NULL
+  // placeholders: a split kernel that merges in its workgroup ignores them, any other needs them)
   ae_attn_params q = *p;
+  q.partial_o = (float*)(uintptr_t)256;
+  q.partial_rs = (float*)(uintptr_t)256;
+  int rc = ae_internal_decode_check(split, combine, &q, cfg, combine_cfg);
+  if (rc) return rc;
+  unsigned char* base = nullptr;
+  rc = scratch_address(&base);
+  if (rc) return rc;
   q.partial_o = (float*)base;
   q.partial_rs = (float*)(base + o_bytes);
   // Nothing has to start at zero: every wave of the split kernel writes its partial and its row scales in

@@ -83,6 +83,13 @@ static_assert(AE_NSTAGE >= 3, "a tile is multiplied by K one trip before it is m
 #ifndef AE_PAGED
 #define AE_PAGED 0
 #endif
+// 1 (single-split builds only, a measurement switch): every workgroup reports the shader-clock cycles (s_memtime)
+// and the constant-rate 100 MHz ticks (s_memrealtime) between its entry and its last store, as two 64-bit values
+// at ((unsigned long long*)p.partial_o)[2 * blockIdx.x] - a buffer a single-split launch does not otherwise use.
+#ifndef AE_CLOCK_STAMPS
+#define AE_CLOCK_STAMPS 0
+#endif
+static_assert(!AE_CLOCK_STAMPS || AE_NSPLIT == 1, "the clock stamps go where a split launch keeps its partial results");
 #if AE_PAGED
 #include "ae_mla_paged.h"
 #endif
@@ -107,6 +114,10 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const bool score_wave = wave < 2;
+#if AE_CLOCK_STAMPS
+  const unsigned long long ae_t0 = __builtin_amdgcn_s_memtime();
+  const unsigned long long ae_w0 = __builtin_amdgcn_s_memrealtime();
+#endif
 
   // ---- which (head tile, split, kv head, batch): 1-D grid, ids 8 apart share their KV range ---------
   const int group = p.heads_q / p.heads_kv;
@@ -631,6 +642,18 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
         p.partial_rs[(int64_t)i * p.batch * p.heads_q * p.num_splits + row] = frs[i];
     }
   }
+#if AE_CLOCK_STAMPS
+  __builtin_amdgcn_s_waitcnt(0);          // the stores have been acknowledged
+  if (wave == 2) {
+    const unsigned long long t1 = __builtin_amdgcn_s_memtime();
+    const unsigned long long w1 = __builtin_amdgcn_s_memrealtime();
+    if (lane == 0) {
+      unsigned long long* st = (unsigned long long*)p.partial_o + 2 * (unsigned long long)blockIdx.x;
+      st[0] = t1 - ae_t0;
+      st[1] = w1 - ae_w0;
+    }
+  }
+#endif
 }
 
 #include "ae_combine.h"

@@ -94,6 +94,14 @@
 #ifndef AE_PIPE_KIND
 #define AE_PIPE_KIND 0
 #endif
+// 1: every workgroup reports the shader-clock cycles (s_memtime) and the constant-rate 100 MHz ticks
+// (s_memrealtime) between its entry and its last store, as two 64-bit values at
+// ((unsigned long long*)p.partial_o)[2 * blockIdx.x] - a buffer the prefill launch does not otherwise use.
+// Their ratio is the shader clock the chip granted while the workgroup ran (a measurement build: bench.py
+// --mfma-probe).
+#ifndef AE_CLOCK_STAMPS
+#define AE_CLOCK_STAMPS 0
+#endif
 // 1: Q carries c*log2e and the reference is the C operand of the first k-step (see above)
 #ifndef AE_PRESCALE
 #define AE_PRESCALE (!AE_DTYPE_BF16 && AE_PIPE_KIND == 0)
@@ -115,6 +123,10 @@ void ae_prefill_kernel(const ae_attn_params p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31;
   const int hf = lane >> 5;
+#if AE_CLOCK_STAMPS
+  const unsigned long long ae_t0 = __builtin_amdgcn_s_memtime();
+  const unsigned long long ae_w0 = __builtin_amdgcn_s_memrealtime();
+#endif
 
   // ---- which (q-tile, head, batch): ids dealt so that the heads sharing K/V meet in one XCD's L2,
   // heavy causal q-tiles first (see ae_prefill.hip) -------------------------------------------
@@ -832,4 +844,16 @@ void ae_prefill_kernel(const ae_attn_params p) {
       if (AE_EVEN_Q || q0w + row < p.seqlen_q) *(ae_elem8*)(og + (int64_t)(q0w + row) * p.o_stride_s + c * 8) = w;
     }
   }
+#if AE_CLOCK_STAMPS
+  __builtin_amdgcn_s_waitcnt(0);          // the stores have been acknowledged
+  {
+    const unsigned long long t1 = __builtin_amdgcn_s_memtime();
+    const unsigned long long w1 = __builtin_amdgcn_s_memrealtime();
+    if (tid == 0) {
+      unsigned long long* st = (unsigned long long*)p.partial_o + 2 * (unsigned long long)blockIdx.x;
+      st[0] = t1 - ae_t0;
+      st[1] = w1 - ae_w0;
+    }
+  }
+#endif
 }

@@ -143,6 +143,9 @@ def measure(name, steps, warmup):
            "checked": checked, **info}
     res["tflops"] = info["flops"] / (wall_ms * 1e-3) / 1e12
     res["gbs"] = info["bytes"] / (wall_ms * 1e-3) / 1e9
+    stamps = getattr(getattr(mod, "_op", None), "clock_stamps", None)     # builds with AE_CLOCK_STAMPS=1 only
+    if stamps is not None:
+        res["clock_mhz"] = _clock_mhz(stamps)
     if kind in ("prefill", "prefill_bwd"):
         ach = info["flops"] / (ev_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
@@ -245,6 +248,95 @@ def copy_probe():
     assert torch.equal(src, dst)
 
 
+MFMA_FLOP_PER_CLK = 256 * 4 * 1024.0     # 256 CUs x 4 SIMDs x (32*32*16*2 flop per 32-cycle MFMA)
+
+
+def _clock_mhz(stamps):
+    """Shader clock from per-workgroup (s_memtime cycles, s_memrealtime 100 MHz ticks) pairs."""
+    st = stamps.cpu().double()
+    st = st[st[:, 1] > 0]
+    return float(st[:, 0].sum() / st[:, 1].sum() * 100.0) if len(st) else float("nan")
+
+
+def mfma_probe(waves_per_simd=1, extra_valu=0, launches=20, iters=250):
+    """The matrix-pipe ceiling of this chip, measured: ae_mfma_probe_kernel (nothing but fp16 32x32x16 MFMAs,
+    one or two waves per SIMD) on all-zero and on N(0,1) operands -- the same code object, so the difference
+    is the chip's power management reacting to the operand data.  Returns {operands: {tflops, clock_mhz,
+    cycles_per_mfma}}; clock from the kernel's own s_memtime / s_memrealtime stamps."""
+    import ctypes
+    import torch
+    from core.runtime import hip_rt as rt
+
+    class ProbeParams(ctypes.Structure):
+        _fields_ = [("src", ctypes.c_void_p), ("sink", ctypes.c_void_p), ("stamps", ctypes.c_void_p),
+                    ("n_src", ctypes.c_uint32), ("iters", ctypes.c_int32)]
+    cfg = f"#define AE_PROBE_WAVES_PER_SIMD {waves_per_simd}\n#define AE_PROBE_EXTRA_VALU {extra_valu}\n"
+    kern = rt.compile_module("ae_mfma_probe.hip", {"ae_config.h": cfg}).kernel("ae_mfma_probe_kernel")
+    dev = torch.device("cuda:0")
+    n_src = 1 << 20
+    grid = 256 * 8
+    g = torch.Generator().manual_seed(0)
+    pools = {"zeros": torch.zeros(n_src, dtype=torch.float16, device=dev),
+             "randn": torch.randn(n_src, generator=g, dtype=torch.float32).half().to(dev)}
+    sink = torch.zeros(1024, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    out = {}
+    for name, pool in pools.items():
+        stamps = torch.zeros((grid, 2), dtype=torch.int64, device=dev)
+        prm = ProbeParams(pool.data_ptr(), sink.data_ptr(), stamps.data_ptr(), n_src, iters)
+        threads = 256 * waves_per_simd
+
+        def launch():
+            kern.launch(prm, (grid, 1, 1), (threads, 1, 1), 0, stream)
+        t_w = time.perf_counter()
+        while (time.perf_counter() - t_w) * 1e3 < 2 * CLOCK_RAMP_MS:      # to the working clock first
+            for _ in range(4):
+                launch()
+            torch.cuda.synchronize()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record(stream)
+        for _ in range(launches):
+            launch()
+        e1.record(stream)
+        ms = e0.elapsed_ms(e1) / launches
+        flop = grid * 4.0 * waves_per_simd * iters * 32 * 32768.0
+        st = stamps.cpu().double()
+        out[name] = {"tflops": flop / (ms * 1e-3) / 1e12, "ms": ms, "clock_mhz": _clock_mhz(stamps),
+                     "cycles_per_mfma": float(st[:, 0].mean() / (iters * 32.0 * waves_per_simd))}
+    return out
+
+
+def mfma_probe_report(steps, warmup):
+    """`--mfma-probe`: the measured matrix ceiling (zeros / N(0,1) operands, one and two waves per SIMD, with
+    and without other arithmetic between the MFMAs) and, beside it, the prefill and MLA kernels of the
+    benchmark built with clock stamps: their TFLOP/s, the shader clock they ran at, and what the matrix pipes
+    could deliver at that clock."""
+    lines = ["# matrix-pipe ceiling probe (ae_mfma_probe_kernel: fp16 32x32x16 MFMAs only) and the clock the attention kernels run at",
+             "# columns: case, operands, TFLOP/s, shader clock MHz (s_memtime / s_memrealtime inside the kernel), "
+             "cycles per MFMA and wave, share of 2500 TFLOP/s"]
+    rec = {}
+    for wps, extra in ((1, 0), (2, 0), (1, 4)):
+        r = mfma_probe(wps, extra)
+        tag = f"probe {wps} wave(s)/SIMD" + (f" + {extra} v_fma per MFMA" if extra else "")
+        rec[tag] = r
+        for ops, v in r.items():
+            lines.append(f"{tag}, {ops}, {v['tflops']:.0f}, {v['clock_mhz']:.0f}, {v['cycles_per_mfma']:.1f}, "
+                         f"{v['tflops'] / PEAK_MFMA_TFLOPS:.3f}")
+    os.environ["AE_CLOCK_STAMPS"] = "1"
+    lines.append("# columns: workload, TFLOP/s (HIP events), ms per launch, shader clock MHz over the launch's workgroups, "
+                 "matrix-pipe rate at that clock TFLOP/s, kernel's share of it, share of 2500 TFLOP/s")
+    for name in ("c2_causal", "c2_full", "c3_sigmoid", "c5_mla_decode"):
+        r = measure(name, steps, warmup)
+        clk = r.get("clock_mhz", float("nan"))
+        tf = r["flops"] / (r["kernel_ms"] * 1e-3) / 1e12
+        at_clock = MFMA_FLOP_PER_CLK * clk * 1e6 / 1e12
+        rec[name] = {"tflops": tf, "ms": r["kernel_ms"], "clock_mhz": clk}
+        lines.append(f"{name}, {tf:.0f}, {r['kernel_ms']:.4f}, {clk:.0f}, {at_clock:.0f}, {tf / at_clock:.3f}, "
+                     f"{tf / PEAK_MFMA_TFLOPS:.3f}")
+    print("\n".join(lines))
+    print(json.dumps({"mfma_probe": rec}), flush=True)
+
+
 def cpu_baseline(name):
     """The CPU oracle on a bounded sample of the workload (one batch entry; heads in chunks so the
     [heads, S, S] fp32 score tensor stays below ~1 GiB), fp32 compute on the rounded inputs."""
@@ -323,6 +415,9 @@ def main():
     ap.add_argument("--workload", default="c2_causal", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extra", action="store_true", help="measure only --workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of the benchmark line: measure the matrix-pipe ceiling (a pure MFMA loop on zero and "
+                         "on N(0,1) operands) and the shader clock the prefill / MLA kernels run at")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain 256 MiB copy kernel (ae_copy_probe_kernel) so that a "
                          "hardware-counter run can scale FETCH_SIZE / WRITE_SIZE by a known transfer")
@@ -338,6 +433,9 @@ def main():
         sys.exit(3)
     from core.runtime import hip_rt as rt
     info = rt.device_info(0)
+    if a.mfma_probe:
+        mfma_probe_report(a.steps, a.warmup)
+        return
 
     head = measure(a.workload, a.steps, a.warmup)
     if a.copy_probe:
@@ -357,6 +455,11 @@ def main():
     }
     if "mfma_frac" in head:
         line["mfma_frac"] = head["mfma_frac"]
+    if head["roofline"]["bound"] == "mfma":
+        # beside (never instead of) the fraction of the published peak: what a pure MFMA loop reaches on this
+        # chip on the same kind of operand data, and on zeros
+        pr = mfma_probe(launches=10)
+        line["mfma_ceiling_measured"] = {k: {"tflops": v["tflops"], "clock_mhz": v["clock_mhz"]} for k, v in pr.items()}
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.workload)
     if not a.no_extra:

@@ -52,7 +52,7 @@ using __hip_internal::uint64_t;
 extern "C" {
 #endif
 
-#define AE_ABI_VERSION 4
+#define AE_ABI_VERSION 5
 
 typedef enum ae_status {
   AE_OK = 0,
@@ -132,7 +132,11 @@ typedef struct ae_tile_cfg {
   int32_t n_rowscales; /* number of final rowscales the kernel writes                     */
   int32_t mask_mode;   /* 0 none, 1 analytic causal, 2 block table                        */
   int32_t paged;       /* MLA decode: 1 when the kernel reads KV through block_table / seqlens_k */
-  int32_t reserved[2];
+  int32_t merge_in_wg; /* GQA decode: 1 when the split kernel was compiled with AE_MERGE_IN_WG 1 (its one
+                          workgroup per (batch, kv head, head tile) merges its waves' partial results and
+                          writes out itself: no combine kernel, no work buffers), else 0                   */
+  int32_t table_rows;  /* mask_mode 2: block-mask rows one q tile may span, the AE_TT_ROWS the kernel was
+                          compiled with (1, 2, 4 or 8); 0 stands for the kernels' default of 8             */
 } ae_tile_cfg;
 
 /*
@@ -237,9 +241,11 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
  *   (attn_gqa_decode_tl.py:150-151, 224-266). Every WAVE of the split kernel produces one partial,
  *   so its grid is (num_splits / (threads/64), ceil(Hq/Hkv / block_m)*Hkv, B); kv_per_split is the
  *   share of one partial and must be a multiple of block_n; combine_cfg->block_n is the number of
- *   splits the combine kernel was compiled for and must equal num_splits.  `combine` may be NULL for a
- *   split kernel compiled with AE_MERGE_IN_WG 1 when num_splits equals the waves of one workgroup: that
- *   workgroup merges its waves' partial results itself and writes out (one launch, no work buffers).
+ *   splits the combine kernel was compiled for and must equal num_splits.  A split kernel compiled with
+ *   AE_MERGE_IN_WG 1 is announced by cfg->merge_in_wg = 1: num_splits must then equal the waves of one
+ *   workgroup, `combine` must be NULL (that workgroup merges its waves' partial results itself and writes
+ *   out: one launch, no work buffers).  With cfg->merge_in_wg = 0 the combine kernel, its configuration and
+ *   both work buffers are required; a launch that lacks any of them is refused, nothing runs.
  */
 int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream);
 int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,

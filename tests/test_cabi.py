@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in ae_hip.h but not exported"
     assert sorted(rt.EXPORTED_SYMBOLS) == names
-    assert rt.lib().ae_abi_version() == 4
+    assert rt.lib().ae_abi_version() == 5
 
 
 def test_struct_layout_matches_the_header():
@@ -162,10 +162,110 @@ def test_paged_cache_arguments_are_checked_before_any_launch():
     cc = rt.TileCfg(block_m=1, block_n=1, threads=128)
     assert lib.ae_decode_fwd(fake, fake, ctypes.byref(p), ctypes.byref(cfg()), ctypes.byref(cc), None) == 1
     assert "reads a dense cache" in lib.ae_last_error().decode()
-    # without a merge kernel the splits must be the waves of one workgroup
-    p = params(num_splits=16, kv_per_split=32)
-    assert lib.ae_decode_fwd(fake, None, ctypes.byref(p), ctypes.byref(cfg(threads=256)), None, None) == 1
-    assert "must be the 4 waves of one workgroup" in lib.ae_last_error().decode()
+
+
+def test_decode_merge_form_is_checked_before_any_launch():
+    """Whether a GQA split kernel merges its waves' partial results itself (AE_MERGE_IN_WG) travels in
+    ae_tile_cfg.merge_in_wg, and ae_decode_fwd holds every launch to it: a kernel that does not merge never
+    runs without a combine kernel and both work buffers (it would store through NULL), a kernel that merges
+    takes no combine kernel and needs its splits to be the waves of one workgroup.  All refusals happen in the
+    argument checks, so the kernel handles are dummies."""
+    lib = rt.lib()
+    fake = ctypes.c_void_p(8)
+    buf = ctypes.create_string_buffer(64)
+    addr = ctypes.addressof(buf)
+
+    def params(**kw):
+        p = rt.AttnParams()
+        p.q = p.k = p.v = p.out = addr
+        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = 2, 32, 8, 1, 256
+        p.num_splits, p.kv_per_split = 4, 64
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
+
+    def cfg(**kw):
+        c = rt.TileCfg(block_m=16, block_n=32, threads=256, lds_bytes=1024, head_dim=128, head_dim_v=128,
+                       elem_bytes=2, n_rowscales=0, mask_mode=0)
+        for k, v in kw.items():
+            setattr(c, k, v)
+        return c
+
+    def run(entry, p, c, combine, ccfg=True):
+        cc = rt.TileCfg(block_m=1, block_n=p.num_splits, threads=64)
+        rc = entry(fake, combine, ctypes.byref(p), ctypes.byref(c), ctypes.byref(cc) if ccfg else None, None)
+        return rc, lib.ae_last_error().decode()
+
+    for entry in (lib.ae_decode_fwd, lib.ae_decode_fwd_noalloc):
+        # a kernel that does not merge, launched without a combine kernel (what a stale kernel cache once did)
+        rc, msg = run(entry, params(), cfg(merge_in_wg=0), None)
+        assert rc == 1 and "does not merge in the workgroup" in msg, msg
+        # a merging kernel takes no combine kernel, and only the waves of one workgroup as its splits
+        rc, msg = run(entry, params(), cfg(merge_in_wg=1), fake)
+        assert rc == 1 and "takes no combine kernel" in msg, msg
+        rc, msg = run(entry, params(num_splits=16, kv_per_split=32), cfg(merge_in_wg=1), None)
+        assert rc == 1 and "the 4 waves of one workgroup" in msg, msg
+        rc, msg = run(entry, params(), cfg(merge_in_wg=7), None)
+        assert rc == 1 and "merge_in_wg=7" in msg, msg
+        rc, msg = run(entry, params(), cfg(merge_in_wg=1, n_rowscales=1), None)
+        assert rc == 1 and "rowscale_out[0] is NULL" in msg, msg
+    # without the merge: both work buffers and the combine configuration are required
+    rc, msg = run(lib.ae_decode_fwd, params(), cfg(), fake)
+    assert rc == 1 and "work buffers are NULL" in msg, msg
+    rc, msg = run(lib.ae_decode_fwd, params(partial_o=addr, partial_rs=addr), cfg(), fake, ccfg=False)
+    assert rc == 1 and "combine configuration is NULL" in msg, msg
+
+
+def test_block_table_geometry_is_checked_before_any_launch():
+    """mask_mode 2: both prefill launches refuse a table whose blocks do not fit the kernel's tiles - rows that
+    neither divide nor are divided by the q tile, columns that are not whole kv tiles, and more table rows per q
+    tile than the kernel keeps masks for (ae_tile_cfg.table_rows, the AE_TT_ROWS it was compiled with): such a
+    kernel would apply the classes of its last table row to every further row of the q tile."""
+    lib = rt.lib()
+    fake = ctypes.c_void_p(8)
+    buf = ctypes.create_string_buffer(64)
+    addr = ctypes.addressof(buf)
+
+    def params(**kw):
+        p = rt.AttnParams()
+        p.q = p.k = p.v = p.out = p.block_mask = p.partial_o = p.partial_rs = addr
+        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = 1, 8, 8, 256, 1024
+        p.mask_b, p.mask_h, p.mask_nq, p.mask_nkv, p.mask_block_m, p.mask_block_n = 1, 1, 8, 16, 32, 64
+        p.num_splits, p.kv_per_split = 2, 512
+        p.o_stride_h, p.o_stride_s, p.o_stride_b = 64, 8 * 64, 256 * 8 * 64
+        for k, v in kw.items():
+            setattr(p, k, v)
+        return p
+
+    def cfg(**kw):
+        c = rt.TileCfg(block_m=128, block_n=64, threads=256, lds_bytes=1024, head_dim=64, head_dim_v=64,
+                       elem_bytes=2, n_rowscales=0, mask_mode=2, table_rows=4)
+        for k, v in kw.items():
+            setattr(c, k, v)
+        return c
+
+    def fwd(p, c):
+        rc = lib.ae_prefill_fwd(fake, ctypes.byref(p), ctypes.byref(c), None)
+        return rc, lib.ae_last_error().decode()
+
+    def split(p, c):
+        cc = rt.TileCfg(block_m=1, block_n=p.num_splits, threads=128)
+        rc = lib.ae_prefill_split_fwd(fake, fake, ctypes.byref(p), ctypes.byref(c), ctypes.byref(cc), None)
+        return rc, lib.ae_last_error().decode()
+
+    for launch in (fwd, split):
+        rc, msg = launch(params(), cfg(table_rows=1))            # 128-row tile over 32-row blocks: 4 rows
+        assert rc == 1 and "spans 4 rows" in msg and "compiled for 1" in msg, msg
+        rc, msg = launch(params(), cfg(table_rows=2))
+        assert rc == 1 and "compiled for 2" in msg, msg
+        rc, msg = launch(params(mask_block_m=8, mask_nq=32), cfg(table_rows=0))     # 16 rows > the default of 8
+        assert rc == 1 and "spans 16 rows" in msg and "compiled for 8" in msg, msg
+        rc, msg = launch(params(mask_block_m=48, mask_nq=6), cfg())
+        assert rc == 1 and "incompatible with tile" in msg, msg
+        rc, msg = launch(params(mask_block_n=96, mask_nkv=11), cfg())
+        assert rc == 1 and "not a multiple of the 64-key kv tile" in msg, msg
+        rc, msg = launch(params(), cfg(table_rows=-1))
+        assert rc == 1 and "table_rows=-1" in msg, msg
 
 
 def test_misaligned_tensors_are_refused_before_any_launch():

@@ -534,3 +534,63 @@ def test_tuner_cache_records(tmp_path):
     tuner.store(f, pk, tuner.encode_tiles(cands[1]))                  # replaces the record of that problem
     assert len(json.load(open(f))) == 2 and tuner.decode_tiles(tuner.lookup(f, pk), cands) == cands[1]
     assert json.load(open(f)) == recs[1:] + [{**pk, "tuned_config": tuner.encode_tiles(cands[1])}]
+
+
+def test_tuner_store_survives_a_damaged_file(tmp_path):
+    """A tune_file that was cut short in the middle of a write (or written by two processes at once) still gives
+    up its complete records, and the next store keeps them; the store itself replaces the file in one step and
+    leaves no temporary file behind."""
+    import json
+    import os
+    from core.lower import tuner
+    f = str(tmp_path / "tuned.json")
+    pk = {"batch": 2, "heads": 32, "seq_len": 1024, "dim": 128, "dimv": 128}
+    for b in (1, 2, 3):
+        tuner.store(f, {**pk, "batch": b}, [128, 64, 2, 256, 2, "ae_prefill.hip"])
+    text = open(f).read()
+    third = text.rindex("{")
+    open(f, "w").write(text[:third + 40])             # the third record is torn, the closing bracket is gone
+    with pytest.raises(ValueError):
+        json.load(open(f))
+    assert tuner.lookup(f, {**pk, "batch": 1}) == [128, 64, 2, 256, 2, "ae_prefill.hip"]
+    assert tuner.lookup(f, {**pk, "batch": 3}) is None
+    tuner.store(f, {**pk, "batch": 4}, [256, 64, 2, 256, 1, "ae_prefill_pipe.hip"])
+    recs = json.load(open(f))                          # whole again
+    assert [r["batch"] for r in recs] == [1, 2, 4]
+    assert os.listdir(tmp_path) == ["tuned.json"]
+    open(f, "w").write("not json at all")
+    assert tuner.lookup(f, pk) is None
+    tuner.store(f, pk, [1])
+    assert json.load(open(f)) == [{**pk, "tuned_config": [1]}]
+
+
+def test_decode_kernel_cache_is_keyed_by_the_merge_form(monkeypatch):
+    """GQADecodeOp keeps one compiled kernel pair per (splits, even kv, merge form).  Whether the split kernel
+    merges its waves' partial results itself (AE_MERGE_IN_WG) depends on ``static_workspace`` and on an
+    environment variable, both of which may change between two calls of one engine; a kernel compiled for one
+    form must never be handed to the launch of the other (the merging kernel leaves the work buffers unwritten,
+    the other one stores through them).  hipRTC runs on the CPU, so the variants are really compiled here."""
+    from core.lower.lower_decode import GQADecodeOp
+    dt = torch.float16
+    B, Hq, Hkv, Skv, D = 128, 32, 8, 777, 128          # plans 4 splits: the waves of one workgroup
+    meta = (meta_tensor(B, Hq, 1, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt))
+    op = GQADecodeOp(meta, CustomIO({}), C.make_scale_score_mod(D ** -0.5), None, C.OnlineSoftmax(), "-inf")
+    n_split, _ = op.plan_splits(B, Hq, Hkv, Skv)
+    assert n_split == op.N_WAVES
+    monkeypatch.delenv("AE_DECODE_MERGE_IN_WG", raising=False)
+    # the constructor compiled the merging form
+    assert set(op._variants) == {(4, False, True)}
+    merged = op._variant(n_split, False, op.merges_in_workgroup(n_split))
+    assert "#define AE_MERGE_IN_WG 1" in merged[3] and merged[1].merge_in_wg == 1
+    # the documented toggle: the launch without allocations keeps the merge kernel
+    op.static_workspace = True
+    assert not op.merges_in_workgroup(n_split)
+    plain = op._variant(n_split, False, op.merges_in_workgroup(n_split))
+    assert plain is not merged and plain[0] is not merged[0]
+    assert "#define AE_MERGE_IN_WG 0" in plain[3] and plain[1].merge_in_wg == 0
+    op.static_workspace = False
+    assert op._variant(n_split, False, op.merges_in_workgroup(n_split)) is merged
+    # ... and the environment variable that keeps the two launches
+    monkeypatch.setenv("AE_DECODE_MERGE_IN_WG", "0")
+    assert op._variant(n_split, False, op.merges_in_workgroup(n_split)) is plain
+    assert set(op._variants) == {(4, False, True), (4, False, False)}

@@ -38,7 +38,11 @@ def test_decode_on_the_built_in_work_buffer(cuda_device):
     dtype = torch.float16
     cases = [(8, 32, 8, 4096, 128),      # 32 partials per head: 4.2 MB of the 16 MiB buffer
              (2, 32, 8, 1000, 128),      # smaller, ragged KV: the buffer still holds the first call's partials
-             (3, 8, 2, 333, 64)]
+             (3, 8, 2, 333, 64),
+             # 4 splits = the waves of one workgroup: the allocating path merges inside the workgroup (one launch,
+             # no partial buffers), this entry point keeps the merge kernel -- two differently compiled split
+             # kernels of one engine, which its kernel cache must keep apart
+             (128, 32, 8, 777, 128)]
     for n, (B, Hq, Hkv, Skv, D) in enumerate(cases):
         print(f"case no-alloc decode B{B} Hq{Hq} Hkv{Hkv} Skv{Skv} D{D}", flush=True)
         q, k, v = (t.cuda() for t in C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, dtype, seed=40 + n))
@@ -49,6 +53,8 @@ def test_decode_on_the_built_in_work_buffer(cuda_device):
         out_a, lse_a, out_b, lse_b = _both(mod, q, k, v)
         assert torch.isfinite(out_a).all() and torch.isfinite(lse_a).all()
         assert torch.equal(out_a, out_b) and torch.equal(lse_a, lse_b), (B, Hq, Hkv, Skv, D)
+        if n_split == mod.attention.N_WAVES:
+            assert {k[2] for k in mod.attention._variants} == {True, False}, mod.attention._variants.keys()
 
 
 def test_decode_too_large_for_the_built_in_work_buffer_is_refused(cuda_device):
