@@ -9,8 +9,11 @@ Behind the API everything is new: the traced functions are lowered to HIP functo
 the hand-written gfx950 kernel templates under csrc/kernels, compiled with hipRTC through
 libae_hip.so and launched on torch's current stream.  There is a single backend; ``backend="tl"``
 and ``backend="cute"`` are both accepted and select the call convention only (for MLA the CuTe
-form ``mod(q, kv_cache) -> (out, lse)``, attn_engine.py:193-214).  Tuner arguments are accepted
-and ignored: tile shapes are fixed per head dimension.
+form ``mod(q, kv_cache) -> (out, lse)``, attn_engine.py:193-214).  ``tune=True`` with a ``tune_file``
+(``tune_bwd`` / ``tune_file_bwd`` for the backward) takes the tile configuration -- for decode engines the
+split count -- from that file's record of the problem, or measures the candidates at the first call on a
+GPU and records the winner there (core/lower/tuner.py; the reference: attn_tl.py:465-521); without it the
+choice is fixed per head dimension and problem size.
 """
 from __future__ import annotations
 
@@ -71,7 +74,22 @@ class AttentionEngine:
                  mask_value="-inf", device=None, backend="tl",
                  tune=False, tune_file="", tune_bwd=False, tune_file_bwd="",
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
-                 extern_block_mask=False, kv_shared=False):
+                 extern_block_mask=False, kv_shared=False, exact_scale=None, defer_norm=None):
+        """The reference's constructor (attn_engine.py:109-115) plus two numerics switches of this build, both
+        None by default (= the faster form) and both only meaningful for prefill engines:
+
+        ``exact_scale=True``: the software-pipelined fp16 softmax kernel multiplies every score by the constant
+        of ``score_mod`` in fp32.  By default it folds that constant (times log2 e) into its resident fp16 Q
+        fragments, one rounding of the product to fp16, which moves a score by up to 2^-12 of sum|q_d k_d|*c:
+        lse then stays within 1e-3 of the fp32 reference while the scaled scores stay below a few tens
+        (3e-4 on N(0,1) inputs at head dim 128) and within 2^-11 * max sum|q_d||k_d| * c in general.  bf16
+        engines and the other kernels never pre-scale.
+
+        ``defer_norm=False``: online functions of the form ``scores / r_new`` with ``o_scale = r_old / r_new``
+        (retention) keep that per-tile form.  By default the lowering accumulates the unnormalised scores and
+        divides once in the epilogue (the factors telescope); P, the fp16 operand of the second product, then
+        holds |X| instead of |X / r| <= 1, so scores of 65504 and more overflow where the script's form stays
+        finite (bf16 has the range of fp32)."""
         if backend not in ("tl", "cute", "hip"):
             raise ValueError(f"unknown backend {backend!r}")
         if mask_value not in ("-inf", "0"):
@@ -89,7 +107,8 @@ class AttentionEngine:
             infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
             infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
             kv_shared=kv_shared,
-            tune=dict(tune=bool(tune), tune_file=tune_file, tune_bwd=bool(tune_bwd), tune_file_bwd=tune_file_bwd))
+            tune=dict(tune=bool(tune), tune_file=tune_file, tune_bwd=bool(tune_bwd), tune_file_bwd=tune_file_bwd),
+            numerics=dict(exact_scale=exact_scale, defer_norm=defer_norm))
         # generated device source, under the attribute name scripts read
         # (attn_script/reluattn.py:75-76)
         self.tl_code = self._op.source
@@ -100,7 +119,7 @@ class AttentionEngine:
     # same dispatch order as attn_engine.py:218-332
     def _select_lower_template(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
                                mask_value, infer_mask, infer_mask_block_M, infer_mask_block_N,
-                               extern_block_mask, kv_shared, tune=None):
+                               extern_block_mask, kv_shared, tune=None, numerics=None):
         dtype_map = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
         q_meta, k_meta, v_meta = qkv_meta
         dtype_map[q_meta.dtype]  # KeyError for unsupported dtypes, as in the reference (225-228, 304)
@@ -132,7 +151,7 @@ class AttentionEngine:
         return PrefillOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                          infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
                          infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
-                         split_kv=split_kv, **(tune or {}))
+                         split_kv=split_kv, **(tune or {}), **(numerics or {}))
 
     def __call__(self, *args, **kargs):
         if kargs.get("block_mask") is not None:

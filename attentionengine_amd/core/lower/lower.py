@@ -354,7 +354,8 @@ def find_deferred_norm(rowscales, new_scores, new_rowscales, o_scale):
     so the kernels may accumulate X v unscaled - no rescale of the whole accumulator per tile - and divide
     once in the epilogue.  What changes is the range of P, the operand of the second product: |X / r| <= 1 in
     the script's form, |X| itself here, so scores of size 65504 and more overflow an fp16 P (bf16 has the
-    range of fp32); AE_DEFER_NORM=0 in the environment keeps the script's form.  Returns (name of r, X) or None."""
+    range of fp32); ``AttentionEngine(..., defer_norm=False)`` (or AE_DEFER_NORM=0 in the environment) keeps the
+    script's form.  Returns (name of r, X) or None."""
     if not (isinstance(new_scores, SymbolScalar) and isinstance(o_scale, SymbolScalar)):
         return None
     if new_scores.code.type != "Div" or o_scale.code.type != "Div":
@@ -372,8 +373,9 @@ def find_deferred_norm(rowscales, new_scores, new_rowscales, o_scale):
 
 
 def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO, in_dtype,
-                   mask_value: str = "-inf") -> LoweredFunctors:
-    """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies."""
+                   mask_value: str = "-inf", defer_norm=None) -> LoweredFunctors:
+    """Trace score_mod / online_fwd / online_fwd_epilogue on symbols and emit their bodies.  ``defer_norm``
+    (None: on, unless AE_DEFER_NORM=0 is in the environment): see find_deferred_norm."""
     custom_fwd_inputs = custom_fwd_inputs if custom_fwd_inputs is not None else CustomIO()
     cust_leaves, customs, cust_loads, cust_fields, cust_preambles = _custom_leaves(custom_fwd_inputs, in_dtype)
     cust_prefetch = cust_preambles.pop("prefetch")
@@ -410,7 +412,9 @@ def trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs: CustomIO
         inits.append(init_literal(v.code.name))
     new_scores, new_rowscales, o_scale = online_func.online_fwd(scores_mod, rowscales, b, h, q_idx)
     deferred = find_deferred_norm(rowscales, new_scores, new_rowscales, o_scale)
-    if deferred is not None and os.environ.get("AE_DEFER_NORM", "1") != "0":
+    if defer_norm is None:
+        defer_norm = os.environ.get("AE_DEFER_NORM", "1") != "0"
+    if deferred is not None and defer_norm:
         # accumulate unscaled, divide by the final row scale in the epilogue (see find_deferred_norm)
         new_scores, o_scale = deferred[1], 1.0
     else:
@@ -674,9 +678,11 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
 
 def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, has_mask_mod: bool,
                   n_rowscales: int, o_scale_one: bool, even_q: bool, even_kv: bool, softmax=None,
-                  elementwise: bool = False) -> str:
+                  elementwise: bool = False, exact_scale=None) -> str:
     """Text of ae_config.h.  ``softmax`` / ``elementwise`` say what the software-pipelined kernel does with a
-    score (AE_PIPE_KIND 0: its built-in online softmax; 1: the generated functor); other kernels ignore them."""
+    score (AE_PIPE_KIND 0: its built-in online softmax; 1: the generated functor); other kernels ignore them.
+    ``exact_scale`` (None: the kernel's default, unless AE_PREFILL_PRESCALE is in the environment): True builds the
+    pipelined fp16 softmax kernel WITHOUT the score scale folded into its Q fragments."""
     extra = []
     if softmax is None and elementwise:
         extra = ["#define AE_PIPE_KIND 1"]
@@ -685,8 +691,10 @@ def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, h
                  f"#define AE_SM_R {softmax[2]}"]
         # The pipelined kernel folds the score scale into its fp16 Q fragments (one rounding of q*c*log2e
         # to fp16: a score moves by about 2^-12 of its size, i.e. lse by < 1e-3 while |score*c| stays below
-        # ~20).  AE_PREFILL_PRESCALE=0 keeps Q as it is and multiplies every score in fp32 instead.
-        if os.environ.get("AE_PREFILL_PRESCALE", "") in ("0", "1"):
+        # ~20).  exact_scale=True (AE_PREFILL_PRESCALE=0) keeps Q as it is and multiplies every score in fp32 instead.
+        if exact_scale is not None:
+            extra.append(f"#define AE_PRESCALE {0 if exact_scale else 1}")
+        elif os.environ.get("AE_PREFILL_PRESCALE", "") in ("0", "1"):
             extra.append(f"#define AE_PRESCALE {os.environ['AE_PREFILL_PRESCALE']}")
     return "\n".join([
         "// generated by core/lower/lower.py -- do not edit",

@@ -28,11 +28,15 @@ class PrefillOp:
     def __init__(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
                  extern_block_mask=False, split_kv=False, target_workgroups=256,
-                 tiles=None, tune=False, tune_file="", tune_bwd=False, tune_file_bwd=""):
+                 tiles=None, tune=False, tune_file="", tune_bwd=False, tune_file_bwd="",
+                 exact_scale=None, defer_norm=None):
         self._ctor = ((qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value),
                       dict(infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
                            infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
-                           split_kv=split_kv, target_workgroups=target_workgroups))
+                           split_kv=split_kv, target_workgroups=target_workgroups,
+                           exact_scale=exact_scale, defer_norm=defer_norm))
+        # numerics switches (see AttentionEngine): None = the default of the kernel / lowering
+        self.exact_scale = exact_scale
         q_meta, k_meta, v_meta = qkv_meta
         self.dtype = q_meta.dtype
         self.D = int(q_meta.shape[3])
@@ -57,7 +61,7 @@ class PrefillOp:
         self.extern_block_mask = bool(extern_block_mask)
         self.mask_block = (int(infer_mask_block_M), int(infer_mask_block_N))
         self.functors = L.trace_functors(score_mod, mask_mod, online_func, custom_fwd_inputs,
-                                         self.dtype, mask_value)
+                                         self.dtype, mask_value, defer_norm=defer_norm)
         self._graph = (score_mod, online_func, custom_fwd_inputs)     # the backward traces score_mod again
         self.functor_src = L.render_functors(self.functors)
         # what the software-pipelined kernel can run: the proven online softmax, or an elementwise graph
@@ -264,7 +268,8 @@ class PrefillOp:
             cfg_src = L.render_config(self.D, self.DV_launch, self.dtype, self.tiles, mask_mode, has_mask_mod,
                                       self.n_rowscales, self.functors.o_scale_one, even_q, even_kv,
                                       self._pipe_softmax if self.tiles.rows_per_wave == 64 else None,
-                                      elementwise=self._pipe_elementwise and self.tiles.rows_per_wave == 64)
+                                      elementwise=self._pipe_elementwise and self.tiles.rows_per_wave == 64,
+                                      exact_scale=self.exact_scale)
             if self.mask_value_zero:
                 cfg_src += "#define AE_MASK_VALUE_ZERO 1\n"
             if mask_mode == 2:
@@ -406,12 +411,21 @@ class _PrefillFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, op, q, k, v, *extra):
         # `extra`: the block mask the engine inferred from mask_mod, which it appends to every call (the
-        # backward applies mask_mod per element instead); custom inputs and external masks are refused
-        bwd = op.backward_op()                 # raises now if this graph has no backward
+        # backward applies mask_mod per element instead); custom inputs and external masks are refused.
+        # A graph without a backward still runs forward on tensors that require gradients -- a caller who
+        # only wants `out` from leaf tensors gets it -- and says so when .backward() is called, as the
+        # reference does (its generated _attention.backward is where a missing rule surfaces,
+        # attn_tl.py:582-640).
+        try:
+            bwd, ctx.no_backward = op.backward_op(), None
+        except NotImplementedError as e:
+            bwd, ctx.no_backward = None, e
         with torch.no_grad():
             out = op._forward(q.detach(), k.detach(), v.detach(), *extra)
         ctx.op = op
         ctx.n_extra = len(extra)
+        if bwd is None:
+            return out
         ctx.customs = tuple(extra[:len(op.functors.customs)])       # scalar CustomIO tensors of score_mod
         lse = op.final_rowscales[bwd.lse_name] if bwd.lse_name is not None else q.new_empty(0)
         ctx.save_for_backward(q, k, v, out, lse)
@@ -419,6 +433,8 @@ class _PrefillFunction(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dout):
+        if ctx.no_backward is not None:
+            raise NotImplementedError(str(ctx.no_backward)) from ctx.no_backward
         q, k, v, out, lse = ctx.saved_tensors
         dq, dk, dv = ctx.op.backward_op()(q, k, v, out, lse, dout, ctx.customs)
         return (None, dq, dk, dv) + (None,) * ctx.n_extra

@@ -1,4 +1,5 @@
-// Matrix-pipe ceiling probe: nothing but mfma_f32_32x32x16_f16 in a loop, with clock stamps.
+// Matrix-pipe ceiling probe: nothing but MFMAs in a loop (optionally with the least other work a flash
+// attention loop needs per MFMA), with clock stamps.
 //
 // It exists to put a measured number next to the published dense fp16 peak of the chip: the rate a wave
 // per SIMD reaches when it issues MFMAs back to back with no memory traffic, no LDS traffic and no other
@@ -9,8 +10,18 @@
 // Every workgroup reports two counter differences taken around its loop: shader-clock cycles (s_memtime)
 // and constant-rate ticks (s_memrealtime, 100 MHz).  Their ratio is the shader clock during the loop.
 //
-// Configuration ("ae_config.h", may be empty): AE_PROBE_WAVES_PER_SIMD (1 or 2) waves per SIMD; AE_PROBE_EXTRA_VALU independent v_fma_f32 per MFMA
-// interleaved into the loop (0 by default: the pure matrix ceiling).
+// Configuration ("ae_config.h", may be empty):
+//   AE_PROBE_WAVES_PER_SIMD  1 or 2 waves per SIMD
+//   AE_PROBE_BF16            1: bf16 operands (the pool is read as bf16), else fp16
+//   AE_PROBE_EXTRA_VALU      independent v_fma_f32 per MFMA, issued between the MFMAs (0: the pure ceiling)
+//   AE_PROBE_EXP             v_exp_f32 per MFMA, likewise
+//   AE_PROBE_LDS             1: every second MFMA takes a fresh A fragment (1 KiB per wave) from LDS, read two
+//                            fragments ahead - the LDS traffic of a kernel whose every fragment feeds two MFMAs
+// A flash attention forward at head dim 128 spends one 32x32x16 MFMA per 64 scores, i.e. per score and lane:
+// one exponential, a maximum, a sum and half a packed conversion at the very least, and half a fragment read.
+// AE_PROBE_EXTRA_VALU 2 + AE_PROBE_EXP 1 (an exponential and the v_fma that consumes it) + AE_PROBE_LDS 1 is that
+// mix - three plain VALU instructions, one transcendental and half a fragment read per MFMA - with nothing else
+// around it: no accumulator read-outs, no tile loads, no barriers, no masks.
 #ifndef __HIPCC_RTC__
 #include <hip/hip_runtime.h>
 #endif
@@ -22,39 +33,71 @@
 #ifndef AE_PROBE_EXTRA_VALU
 #define AE_PROBE_EXTRA_VALU 0
 #endif
+#ifndef AE_PROBE_EXP
+#define AE_PROBE_EXP 0
+#endif
+#ifndef AE_PROBE_LDS
+#define AE_PROBE_LDS 0
+#endif
+#ifndef AE_PROBE_BF16
+#define AE_PROBE_BF16 0
+#endif
 
-typedef _Float16 ae_probe_half8 __attribute__((ext_vector_type(8)));
+#if AE_PROBE_BF16
+typedef __bf16 ae_probe_elem;
+#else
+typedef _Float16 ae_probe_elem;
+#endif
+typedef ae_probe_elem ae_probe_half8 __attribute__((ext_vector_type(8)));
 typedef float ae_probe_f32x16 __attribute__((ext_vector_type(16)));
 
 struct ae_mfma_probe_params {
-  const _Float16* src;            // operand pool, n_src elements (a power of two, at least 32768)
-  float* sink;                    // never written in practice (keeps the accumulators alive)
+  const void* src;                // operand pool, n_src 16-bit elements (a power of two, at least 32768)
+  float* sink;                    // never written in practice (keeps the results alive)
   unsigned long long* stamps;     // [gridDim.x][2]: shader-clock cycles, 100 MHz ticks of the loop
   unsigned n_src;
   int iters;                      // loop trips; one trip = 32 MFMAs per wave
 };
 
+__device__ inline ae_probe_f32x16 ae_probe_mfma(ae_probe_half8 a, ae_probe_half8 b, ae_probe_f32x16 c) {
+#if AE_PROBE_BF16
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
 extern "C" __global__ __launch_bounds__(256 * AE_PROBE_WAVES_PER_SIMD)
 __attribute__((amdgpu_waves_per_eu(AE_PROBE_WAVES_PER_SIMD, AE_PROBE_WAVES_PER_SIMD)))
 void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   const unsigned tid = threadIdx.x;
+  const ae_probe_elem* src = (const ae_probe_elem*)p.src;
   // four A and four B fragments per lane, each lane and workgroup at its own place of the pool
   ae_probe_half8 a[4], b[4];
   const unsigned base = (blockIdx.x * 8191u + tid * 64u) & (p.n_src - 1);
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    a[i] = *(const ae_probe_half8*)(p.src + ((base + i * 8) & (p.n_src - 8)));
-    b[i] = *(const ae_probe_half8*)(p.src + ((base + 32 + i * 8) & (p.n_src - 8)));
+    a[i] = *(const ae_probe_half8*)(src + ((base + i * 8) & (p.n_src - 8)));
+    b[i] = *(const ae_probe_half8*)(src + ((base + 32 + i * 8) & (p.n_src - 8)));
   }
+#if AE_PROBE_LDS
+  // 16 fragments of pool data per wave in LDS (16 KiB a wave), lane-contiguous 16-byte pieces: conflict-free reads
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[4 * AE_PROBE_WAVES_PER_SIMD * 16 * 1024];
+  typedef __attribute__((address_space(3))) ae_probe_half8 lds_frag;
+  lds_frag* mine = (lds_frag*)((__attribute__((address_space(3))) unsigned char*)lds_raw) + (tid >> 6) * 16 * 64 + (tid & 63);
+#pragma unroll
+  for (int f = 0; f < 16; f++)
+    mine[f * 64] = *(const ae_probe_half8*)(src + ((base + 4096 + f * 520) & (p.n_src - 8)));
+#endif
   ae_probe_f32x16 c[8];
 #pragma unroll
   for (int i = 0; i < 8; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) c[i][r] = 0.f;
-#if AE_PROBE_EXTRA_VALU
+#if AE_PROBE_EXTRA_VALU || AE_PROBE_EXP
   float x[8];
 #pragma unroll
-  for (int i = 0; i < 8; i++) x[i] = (float)a[i & 3][i];
+  for (int i = 0; i < 8; i++) x[i] = (float)a[i & 3][i] * 0.25f;
 #endif
   // the operands have arrived before the first stamp is taken
 #pragma unroll
@@ -65,12 +108,25 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   for (int it = 0; it < p.iters; it++) {
 #pragma unroll
     for (int j = 0; j < 32; j++) {
-      c[j & 7] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[j & 3], b[(j >> 2) & 3], c[j & 7], 0, 0, 0);
+#if AE_PROBE_LDS
+      // fragment for the MFMAs j + 4, j + 5 (a[] is a ring of four: one in use, two on their way)
+      if ((j & 1) == 0) a[((j >> 1) + 2) & 3] = mine[((j >> 1) & 15) * 64];
+      c[j & 7] = ae_probe_mfma(a[(j >> 1) & 3], b[j & 3], c[j & 7]);
+#else
+      c[j & 7] = ae_probe_mfma(a[j & 3], b[(j >> 2) & 3], c[j & 7]);
+#endif
 #if AE_PROBE_EXTRA_VALU
 #pragma unroll
       for (int e = 0; e < AE_PROBE_EXTRA_VALU; e++)
         x[(j + e) & 7] = __builtin_fmaf(x[(j + e) & 7], 0.999f, 0.001f);
-      __builtin_amdgcn_sched_barrier(0);      // keep the arithmetic between the MFMAs, where a kernel has it
+#endif
+#if AE_PROBE_EXP
+#pragma unroll
+      for (int e = 0; e < AE_PROBE_EXP; e++)
+        x[(j + 4 + e) & 7] = __builtin_amdgcn_exp2f(x[(j + 4 + e) & 7]) * 0.5f - 0.75f;   // stays in (-0.75, 0.1)
+#endif
+#if AE_PROBE_EXTRA_VALU || AE_PROBE_EXP || AE_PROBE_LDS
+      __builtin_amdgcn_sched_barrier(0);      // keep the other work between the MFMAs, where a kernel has it
 #endif
     }
   }
@@ -83,7 +139,7 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   float acc = 0.f;
 #pragma unroll
   for (int i = 0; i < 8; i++) acc += c[i][tid & 15];
-#if AE_PROBE_EXTRA_VALU
+#if AE_PROBE_EXTRA_VALU || AE_PROBE_EXP
 #pragma unroll
   for (int i = 0; i < 8; i++) acc += x[i];
 #endif

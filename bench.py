@@ -258,11 +258,31 @@ def _clock_mhz(stamps):
     return float(st[:, 0].sum() / st[:, 1].sum() * 100.0) if len(st) else float("nan")
 
 
-def mfma_probe(waves_per_simd=1, extra_valu=0, launches=20, iters=250):
-    """The matrix-pipe ceiling of this chip, measured: ae_mfma_probe_kernel (nothing but fp16 32x32x16 MFMAs,
-    one or two waves per SIMD) on all-zero and on N(0,1) operands -- the same code object, so the difference
-    is the chip's power management reacting to the operand data.  Returns {operands: {tflops, clock_mhz,
-    cycles_per_mfma}}; clock from the kernel's own s_memtime / s_memrealtime stamps."""
+# (label, configuration of ae_mfma_probe.hip) of the cases `--mfma-probe` reports; the first is the pure ceiling
+PROBE_CASES = [
+    ("fp16 MFMA only, 1 wave/SIMD", {}),
+    ("fp16 MFMA only, 2 waves/SIMD", {"AE_PROBE_WAVES_PER_SIMD": 2}),
+    ("bf16 MFMA only, 1 wave/SIMD", {"AE_PROBE_BF16": 1}),
+    ("fp16 MFMA + 4 v_fma per MFMA", {"AE_PROBE_EXTRA_VALU": 4}),
+    ("fp16 MFMA + half a 1 KiB LDS fragment read per MFMA", {"AE_PROBE_LDS": 1}),
+    ("fp16 flash-attention mix per MFMA: 1 v_exp + 3 VALU + half a fragment read, 1 wave/SIMD",
+     {"AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1}),
+    ("fp16 flash-attention mix per MFMA, 2 waves/SIMD",
+     {"AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_WAVES_PER_SIMD": 2}),
+    ("bf16 flash-attention mix per MFMA, 1 wave/SIMD",
+     {"AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_BF16": 1}),
+]
+
+
+def probe_config_text(cfg):
+    return "// configuration of ae_mfma_probe.hip\n" + "".join(f"#define {k} {v}\n" for k, v in sorted(cfg.items()))
+
+
+def mfma_probe(cfg=None, launches=20, iters=250):
+    """The matrix-pipe ceiling of this chip, measured: ae_mfma_probe_kernel (32x32x16 MFMAs back to back, with
+    the other work ``cfg`` asks for between them) on all-zero and on N(0,1) operands -- the same code object, so
+    the difference is the chip's power management reacting to the operand data.  Returns {operands: {tflops,
+    clock_mhz, cycles_per_mfma}}; clock from the kernel's own s_memtime / s_memrealtime stamps."""
     import ctypes
     import torch
     from core.runtime import hip_rt as rt
@@ -270,14 +290,16 @@ def mfma_probe(waves_per_simd=1, extra_valu=0, launches=20, iters=250):
     class ProbeParams(ctypes.Structure):
         _fields_ = [("src", ctypes.c_void_p), ("sink", ctypes.c_void_p), ("stamps", ctypes.c_void_p),
                     ("n_src", ctypes.c_uint32), ("iters", ctypes.c_int32)]
-    cfg = f"#define AE_PROBE_WAVES_PER_SIMD {waves_per_simd}\n#define AE_PROBE_EXTRA_VALU {extra_valu}\n"
-    kern = rt.compile_module("ae_mfma_probe.hip", {"ae_config.h": cfg}).kernel("ae_mfma_probe_kernel")
+    cfg = dict(cfg or {})
+    waves_per_simd = int(cfg.get("AE_PROBE_WAVES_PER_SIMD", 1))
+    kern = rt.compile_module("ae_mfma_probe.hip", {"ae_config.h": probe_config_text(cfg)}).kernel("ae_mfma_probe_kernel")
     dev = torch.device("cuda:0")
     n_src = 1 << 20
     grid = 256 * 8
     g = torch.Generator().manual_seed(0)
-    pools = {"zeros": torch.zeros(n_src, dtype=torch.float16, device=dev),
-             "randn": torch.randn(n_src, generator=g, dtype=torch.float32).half().to(dev)}
+    dt = torch.bfloat16 if cfg.get("AE_PROBE_BF16") else torch.float16
+    pools = {"zeros": torch.zeros(n_src, dtype=dt, device=dev),
+             "randn": torch.randn(n_src, generator=g, dtype=torch.float32).to(dt).to(dev)}
     sink = torch.zeros(1024, dtype=torch.float32, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
     out = {}
@@ -311,13 +333,13 @@ def mfma_probe_report(steps, warmup):
     and without other arithmetic between the MFMAs) and, beside it, the prefill and MLA kernels of the
     benchmark built with clock stamps: their TFLOP/s, the shader clock they ran at, and what the matrix pipes
     could deliver at that clock."""
-    lines = ["# matrix-pipe ceiling probe (ae_mfma_probe_kernel: fp16 32x32x16 MFMAs only) and the clock the attention kernels run at",
+    lines = ["# matrix-pipe ceiling probe (ae_mfma_probe_kernel: 32x32x16 MFMAs back to back, alone or with the named other work "
+             "between them) and the clock the attention kernels run at",
              "# columns: case, operands, TFLOP/s, shader clock MHz (s_memtime / s_memrealtime inside the kernel), "
              "cycles per MFMA and wave, share of 2500 TFLOP/s"]
     rec = {}
-    for wps, extra in ((1, 0), (2, 0), (1, 4)):
-        r = mfma_probe(wps, extra)
-        tag = f"probe {wps} wave(s)/SIMD" + (f" + {extra} v_fma per MFMA" if extra else "")
+    for tag, cfg in PROBE_CASES:
+        r = mfma_probe(cfg)
         rec[tag] = r
         for ops, v in r.items():
             lines.append(f"{tag}, {ops}, {v['tflops']:.0f}, {v['clock_mhz']:.0f}, {v['cycles_per_mfma']:.1f}, "
@@ -458,7 +480,7 @@ def main():
     if head["roofline"]["bound"] == "mfma":
         # beside (never instead of) the fraction of the published peak: what a pure MFMA loop reaches on this
         # chip on the same kind of operand data, and on zeros
-        pr = mfma_probe(launches=10)
+        pr = mfma_probe({}, launches=10)
         line["mfma_ceiling_measured"] = {k: {"tflops": v["tflops"], "clock_mhz": v["clock_mhz"]} for k, v in pr.items()}
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.workload)

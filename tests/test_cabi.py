@@ -67,6 +67,29 @@ def test_struct_layout_matches_the_header():
     assert rc != 0 and "ae_attn_params.k2 offset" in rt.lib().ae_last_error().decode()
 
 
+def test_the_binding_sketch_in_the_integration_notes_matches_the_header():
+    """INTEGRATION.md shows the ctypes structures a maintainer of the reference would copy.  They are executed
+    here as written (the two class statements only) and must have the size of ae_attn_params / ae_tile_cfg,
+    with every field the ctypes mirror of the library also has at the same offset; a sketch that is one ABI
+    behind hands the launch functions a short struct."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    start = text.index("class AttnParams(C.Structure):")
+    end = text.index("assert _lib.ae_abi_version()", start)
+    ns = {"C": ctypes}
+    exec(text[start:end], ns)
+    version = int(re.search(r"assert _lib\.ae_abi_version\(\) == (\d+)", text).group(1))
+    assert version == rt.lib().ae_abi_version()
+    for doc, mirror in ((ns["AttnParams"], rt.AttnParams), (ns["TileCfg"], rt.TileCfg)):
+        assert ctypes.sizeof(doc) == ctypes.sizeof(mirror)
+        mine = {n: getattr(mirror, n).offset for n, _ in mirror._fields_}
+        for name, _ in doc._fields_:
+            if name == "strides":          # the sketch folds the 18 strides into one array
+                assert doc.strides.offset == mirror.q_stride_b.offset and doc.strides.size == 18 * 8
+            else:
+                assert getattr(doc, name).offset == mine[name], name
+        assert doc._fields_[-1][0] == mirror._fields_[-1][0]
+
+
 def _compile(src, opts=()):
     lib = rt.lib()
     handle = ctypes.c_void_p()

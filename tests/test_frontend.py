@@ -594,3 +594,31 @@ def test_decode_kernel_cache_is_keyed_by_the_merge_form(monkeypatch):
     monkeypatch.setenv("AE_DECODE_MERGE_IN_WG", "0")
     assert op._variant(n_split, False, op.merges_in_workgroup(n_split)) is plain
     assert set(op._variants) == {(4, False, True), (4, False, False)}
+
+
+def test_numerics_keywords_of_the_constructor(monkeypatch):
+    """``exact_scale`` / ``defer_norm`` reach the generated configuration; left at None they follow the defaults
+    (and the environment switches the tests use)."""
+    monkeypatch.delenv("AE_PREFILL_PRESCALE", raising=False)
+    monkeypatch.delenv("AE_DEFER_NORM", raising=False)
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    f16 = torch.float16
+    sm = C.make_scale_score_mod(0.1)
+    meta = _meta(2, 32, 32, 1024, 1024, 128, 128, f16)
+    default = AttentionEngine(meta, CustomIO({}), sm, C.causal_mask, C.OnlineSoftmax())
+    exact = AttentionEngine(meta, CustomIO({}), sm, C.causal_mask, C.OnlineSoftmax(), exact_scale=True)
+    folded = AttentionEngine(meta, CustomIO({}), sm, C.causal_mask, C.OnlineSoftmax(), exact_scale=False)
+    assert default._op.tiles.template == "ae_prefill_pipe.hip"
+    assert "AE_PRESCALE" not in default.tl_code
+    assert "#define AE_PRESCALE 0" in exact.tl_code and "#define AE_PRESCALE 1" in folded.tl_code
+    monkeypatch.setenv("AE_PREFILL_PRESCALE", "0")          # the keyword wins over the environment
+    assert "#define AE_PRESCALE 1" in AttentionEngine(meta, CustomIO({}), sm, None, C.OnlineSoftmax(),
+                                                      exact_scale=False).tl_code
+    monkeypatch.delenv("AE_PREFILL_KERNEL")
+    rmeta = _meta(1, 2, 2, 256, 256, 64, 64, f16)
+    args = (rmeta, C.retention_custom_inputs(), C.retention_score_mod, C.causal_mask, C.OnlineRetention())
+    assert AttentionEngine(*args, mask_value="0").attention.functors.deferred_norm == "r"
+    assert AttentionEngine(*args, mask_value="0", defer_norm=False).attention.functors.deferred_norm is None
+    monkeypatch.setenv("AE_DEFER_NORM", "0")
+    assert AttentionEngine(*args, mask_value="0").attention.functors.deferred_norm is None
+    assert AttentionEngine(*args, mask_value="0", defer_norm=True).attention.functors.deferred_norm == "r"

@@ -207,11 +207,18 @@ def test_retention_backward(cuda_device, B, H, Hkv, S, D, DV, dtype):
 
 def test_backward_of_other_graphs_is_refused(cuda_device):
     """An online function that keeps row scales of its own but defines no forward() / backward() rules
-    (here: the running sum of |s| without them) says it has no backward."""
+    (here: the running sum of |s| without them) has no backward.  Its forward still runs on tensors that
+    require gradients, with the result of the plain call; the missing rule is reported by .backward(), where the
+    reference reports it."""
     B, H, S, D = 1, 2, 128, 64
     meta = (meta_tensor(B, H, S, D, dtype=torch.float16),) * 3
     mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(0.125), mask_mod=None,
                           online_func=C.OnlineAbsNorm())
-    q, k, v = (t.cuda().requires_grad_(True) for t in C.make_inputs(B, S, S, H, H, D, D, torch.float16))
-    with pytest.raises(NotImplementedError):
-        mod(q, k, v)
+    q, k, v = (t.cuda() for t in C.make_inputs(B, S, S, H, H, D, D, torch.float16))
+    plain = mod(q, k, v)
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = mod(qg, kg, vg)
+    assert out.requires_grad and torch.equal(out.detach(), plain)
+    with pytest.raises(NotImplementedError, match="no backward for this engine"):
+        out.sum().backward()
+    assert qg.grad is None

@@ -409,7 +409,7 @@ def test_retention_with_decay_mask_input(cuda_device, monkeypatch, B, H, S, D, D
     per score, fetched a tile ahead), abs-sum normalisation clamped at 1, mask_value="0".  With the
     per-tile renormalisation deferred to the epilogue (the default) and as the script writes it."""
     print(f"case retention B{B} H{H} S{S} D{D} DV{DV} {dtype} defer={defer}", flush=True)
-    monkeypatch.setenv("AE_DEFER_NORM", defer)
+    monkeypatch.delenv("AE_DEFER_NORM", raising=False)
     q, k, v = C.make_inputs(B, S, S, H, H, D, DV, dtype)
     q = (q.float() * (1 / D) ** 0.5).to(dtype)                       # bench_utils.py:1034-1036
     g = torch.Generator().manual_seed(5)
@@ -417,13 +417,46 @@ def test_retention_with_decay_mask_input(cuda_device, monkeypatch, B, H, S, D, D
     meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, H, S, D, dtype=dtype),
             meta_tensor(B, H, S, DV, dtype=dtype))
     mod = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
-                          mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0")
+                          mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0",
+                          defer_norm=None if defer == "1" else False)      # the constructor keyword
     assert mod.attention.functors.deferred_norm == ("r" if defer == "1" else None)
     out = mod(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).float().cpu()
     ref, r = R.retention_attention(q, k, v, mask)
     assert (r > 1.0).any()
     assert (mod.final_rowscales["r"].cpu() - r).abs().max().item() <= 2e-3 * r.max().item()
     assert (out - ref).abs().max().item() <= OUT_TOL
+
+
+def test_retention_scores_beyond_the_fp16_range(cuda_device, monkeypatch):
+    """Scores of 65504 and more, fp16: the script's per-tile form ``scores / r_new`` keeps the operand of the
+    second product at |X / r| <= 1 and stays finite -- ``defer_norm=False`` builds exactly that and matches the
+    oracle.  The default (normalisation deferred to the epilogue) holds the unnormalised |X| in fp16 P, which
+    overflows to inf here: a documented limit of the faster form, not of the path (bf16 has fp32's range)."""
+    monkeypatch.delenv("AE_DEFER_NORM", raising=False)
+    B, H, S, D, dtype = 1, 2, 256, 64, torch.float16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=3)
+    q, k = (q.float() * 40.0).to(dtype), (k.float() * 40.0).to(dtype)      # |q k| up to ~ 1e5
+    g = torch.Generator().manual_seed(5)
+    mask = (torch.rand(1, H, S, S, generator=g) * 4.0).tril().to(dtype).contiguous()
+    ref, r = R.retention_attention(q, k, v, mask)
+    scores = torch.einsum("bqhd,bkhd->bhqk", q.float(), k.float()) * mask.float()
+    assert scores.abs().max().item() > 65504.0 and torch.isfinite(ref).all()
+    meta = (meta_tensor(B, H, S, D, dtype=dtype),) * 3
+    exact = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
+                            mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0", defer_norm=False)
+    assert exact.attention.functors.deferred_norm is None
+    out = exact(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).float().cpu()
+    assert torch.isfinite(out).all()
+    assert (out - ref).abs().max().item() <= OUT_TOL
+    assert (exact.final_rowscales["r"].cpu() - r).abs().max().item() <= 2e-3 * r.max().item()
+    fast = AttentionEngine(meta, C.retention_custom_inputs(), score_mod=C.retention_score_mod,
+                           mask_mod=C.causal_mask, online_func=C.OnlineAbsNorm(), mask_value="0")
+    assert fast.attention.functors.deferred_norm == "r"
+    out_fast = fast(q.cuda(), k.cuda(), v.cuda(), mask.cuda()).float().cpu()
+    # rows whose scores all stay inside the fp16 range agree with the oracle in the default form too
+    small = (scores.abs().amax(-1) < 60000.0).permute(0, 2, 1)             # [B, S, H]
+    assert small.any()
+    assert (out_fast - ref)[small].abs().max().item() <= OUT_TOL
 
 
 def test_affine_of_tanh_score_mod(cuda_device):
@@ -539,18 +572,25 @@ def test_head_dims_whose_rows_are_not_a_power_of_two(cuda_device, B, H, Hkv, Sq,
     assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
-def test_pipelined_kernel_exact_scale_switch(cuda_device, monkeypatch):
-    """AE_PREFILL_PRESCALE=0: the pipelined kernel leaves Q alone and scales every score in fp32; lse then
-    holds 1e-3 (+ fp32 rounding) also for scores of size 60."""
+@pytest.mark.parametrize("how", ["keyword", "environment"])
+def test_pipelined_kernel_exact_scale_switch(cuda_device, monkeypatch, how):
+    """``AttentionEngine(..., exact_scale=True)`` (or AE_PREFILL_PRESCALE=0 in the environment): the pipelined
+    kernel leaves Q alone and scales every score in fp32; lse then holds 1e-3 (+ fp32 rounding) also for scores
+    of size 60."""
     monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
-    monkeypatch.setenv("AE_PREFILL_PRESCALE", "0")
+    monkeypatch.delenv("AE_PREFILL_PRESCALE", raising=False)
+    kw = {}
+    if how == "keyword":
+        kw["exact_scale"] = True
+    else:
+        monkeypatch.setenv("AE_PREFILL_PRESCALE", "0")
     B, H, S, D, dtype = 1, 2, 1536, 128, torch.float16
     q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=31)
     k = k.float()
     k[:, S // 2:] *= 12.0
     k = k.to(dtype)
     for mask_mod in (None, C.causal_mask):
-        mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod, C.OnlineSoftmax())
+        mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod, C.OnlineSoftmax(), **kw)
         assert mod._op.tiles.template == "ae_prefill_pipe.hip" and "#define AE_PRESCALE 0" in mod.tl_code
         out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
         ref, lse = R.softmax_attention(q, k, v, causal=mask_mod is not None)
@@ -589,15 +629,20 @@ def test_pipelined_kernel_odd_shapes_and_masks(cuda_device, monkeypatch):
         assert (got[vis] - lse[vis]).abs().max().item() <= LSE_TOL, (B, H, S, D, n)
 
 
-def test_pipelined_kernel_scores_far_above_the_first_tiles(cuda_device, monkeypatch):
-    """Running maxima that keep moving: later keys score far above the first tiles' (for all rows, for the
+@pytest.mark.parametrize("exact_scale", [None, True])
+def test_pipelined_kernel_scores_far_above_the_first_tiles(cuda_device, monkeypatch, exact_scale):
+    """(exact_scale=True: the same cases with the flat 1e-3 bar on lse, which that build holds for fp16 too.)
+    Running maxima that keep moving: later keys score far above the first tiles' (for all rows, for the
     rows of one wave only, growing slowly, and in one jump of three keys), so the lazy refresh of the
     reference and the rescale of O outside the hot loop are taken many times, by some waves of a
     workgroup and not by others.  (bf16 only where |out| stays small enough for the 2e-2 bar: a one-hot
     softmax returns single rows of V, and bf16 rounds a value of 4 by 8e-3.)"""
     monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    monkeypatch.delenv("AE_PREFILL_PRESCALE", raising=False)
     B, H, S, D = 1, 2, 1536, 128
     for dtype in (torch.float16, torch.bfloat16):
+        if exact_scale and dtype == torch.bfloat16:
+            continue                                  # bf16 never pre-scales: nothing to switch
         for case in ("all_rows", "one_wave", "slow_growth", "late_jump"):
             if dtype == torch.bfloat16 and case in ("all_rows", "slow_growth"):
                 continue
@@ -617,8 +662,9 @@ def test_pipelined_kernel_scores_far_above_the_first_tiles(cuda_device, monkeypa
                 q, k = q.to(dtype), k.to(dtype)
                 mask_mod = C.causal_mask if causal else None
                 mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), mask_mod,
-                              C.OnlineSoftmax())
+                              C.OnlineSoftmax(), exact_scale=exact_scale)
                 assert mod._op.tiles.template == "ae_prefill_pipe.hip"
+                assert ("#define AE_PRESCALE 0" in mod.tl_code) == bool(exact_scale)
                 out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
                 dense = _dense(mask_mod, B, H, S, S) if causal else None
                 ref, lse = R.softmax_attention(q, k, v, mask=dense)
@@ -630,7 +676,7 @@ def test_pipelined_kernel_scores_far_above_the_first_tiles(cuda_device, monkeypa
                 # (several hundred here; 2e-2 measured, typical errors are sqrt(D) below the bound; at the
                 # benchmark shapes the effect on lse is below 3e-4).  bf16 keeps Q and scales in fp32.
                 tol = LSE_TOL + 2e-6 * lse.abs()
-                if dtype == torch.float16:
+                if dtype == torch.float16 and not exact_scale:
                     sc = torch.einsum("bqhd,bkhd->bhqk", q.float().abs(), k.float().abs()) / math.sqrt(D)
                     if causal:
                         sc = sc.masked_fill(~dense, 0.0)
