@@ -74,7 +74,7 @@ class AttentionEngine:
                  mask_value="-inf", device=None, backend="tl",
                  tune=False, tune_file="", tune_bwd=False, tune_file_bwd="",
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
-                 extern_block_mask=False, kv_shared=False, exact_scale=None, defer_norm=None):
+                 extern_block_mask=False, kv_shared=False, exact_scale=None, defer_norm=None, allow_spills=None):
         """The reference's constructor (attn_engine.py:109-115) plus two numerics switches of this build, both
         None by default (= the faster form) and both only meaningful for prefill engines:
 
@@ -89,7 +89,14 @@ class AttentionEngine:
         (retention) keep that per-tile form.  By default the lowering accumulates the unnormalised scores and
         divides once in the epilogue (the factors telescope); P, the fp16 operand of the second product, then
         holds |X| instead of |X / r| <= 1, so scores of 65504 and more overflow where the script's form stays
-        finite (bf16 has the range of fp32)."""
+        finite (bf16 has the range of fp32).
+
+        ``allow_spills`` (all engines): what to do with a kernel whose compiled code moves register tuples through
+        scratch memory or spills heavily -- one such build of the compiler in use returned wrong output columns,
+        see ``core.runtime.hip_rt.check_spills``.  None: a RuntimeWarning names it (the builds of the family in
+        which the wrong columns were seen are refused); False: it is refused (``hip_rt.SpillError``; a prefill
+        engine whose own choice was the software-pipelined kernel switches to the generic kernel instead); True:
+        it runs unchecked."""
         if backend not in ("tl", "cute", "hip"):
             raise ValueError(f"unknown backend {backend!r}")
         if mask_value not in ("-inf", "0"):
@@ -108,7 +115,7 @@ class AttentionEngine:
             infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
             kv_shared=kv_shared,
             tune=dict(tune=bool(tune), tune_file=tune_file, tune_bwd=bool(tune_bwd), tune_file_bwd=tune_file_bwd),
-            numerics=dict(exact_scale=exact_scale, defer_norm=defer_norm))
+            numerics=dict(exact_scale=exact_scale, defer_norm=defer_norm), allow_spills=allow_spills)
         # generated device source, under the attribute name scripts read
         # (attn_script/reluattn.py:75-76)
         self.tl_code = self._op.source
@@ -119,7 +126,7 @@ class AttentionEngine:
     # same dispatch order as attn_engine.py:218-332
     def _select_lower_template(self, qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
                                mask_value, infer_mask, infer_mask_block_M, infer_mask_block_N,
-                               extern_block_mask, kv_shared, tune=None, numerics=None):
+                               extern_block_mask, kv_shared, tune=None, numerics=None, allow_spills=None):
         dtype_map = {torch.float16: "float16", torch.bfloat16: "bfloat16"}
         q_meta, k_meta, v_meta = qkv_meta
         dtype_map[q_meta.dtype]  # KeyError for unsupported dtypes, as in the reference (225-228, 304)
@@ -133,13 +140,14 @@ class AttentionEngine:
         if kv_shared:
             from core.lower.lower_decode import MLADecodeOp
             return MLADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func,
-                               mask_value, cute_convention=(self.backend == "cute"), **decode_tune)
+                               mask_value, cute_convention=(self.backend == "cute"), allow_spills=allow_spills,
+                               **decode_tune)
         if not dynamic and q_seqlen != kv_len and head > head_kv:
             assert q_seqlen < kv_len
             assert q_seqlen == 1
             from core.lower.lower_decode import GQADecodeOp
             return GQADecodeOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
-                               **decode_tune)
+                               allow_spills=allow_spills, **decode_tune)
         # MHA decode (attn_engine.py:273-290 of the reference): a few query tokens against a long KV,
         # split over the kv axis and merged with the user's combine()
         # (an online function that does not override combine() cannot merge splits: it runs unsplit)
@@ -151,7 +159,7 @@ class AttentionEngine:
         return PrefillOp(qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value,
                          infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
                          infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
-                         split_kv=split_kv, **(tune or {}), **(numerics or {}))
+                         split_kv=split_kv, allow_spills=allow_spills, **(tune or {}), **(numerics or {}))
 
     def __call__(self, *args, **kargs):
         if kargs.get("block_mask") is not None:

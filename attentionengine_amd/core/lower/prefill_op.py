@@ -29,14 +29,19 @@ class PrefillOp:
                  infer_mask=True, infer_mask_block_M=128, infer_mask_block_N=128,
                  extern_block_mask=False, split_kv=False, target_workgroups=256,
                  tiles=None, tune=False, tune_file="", tune_bwd=False, tune_file_bwd="",
-                 exact_scale=None, defer_norm=None):
+                 exact_scale=None, defer_norm=None, allow_spills=None):
         self._ctor = ((qkv_meta, custom_fwd_inputs, score_mod, mask_mod, online_func, mask_value),
                       dict(infer_mask=infer_mask, infer_mask_block_M=infer_mask_block_M,
                            infer_mask_block_N=infer_mask_block_N, extern_block_mask=extern_block_mask,
                            split_kv=split_kv, target_workgroups=target_workgroups,
-                           exact_scale=exact_scale, defer_norm=defer_norm))
+                           exact_scale=exact_scale, defer_norm=defer_norm, allow_spills=allow_spills))
         # numerics switches (see AttentionEngine): None = the default of the kernel / lowering
         self.exact_scale = exact_scale
+        # None: a build that moves register tuples through scratch memory is reported, False: it is refused
+        # (hip_rt.check_spills); where the pipelined kernel was this operator's own choice it then gives way to the
+        # generic one, see _gives_way_to_the_generic_kernel
+        self.allow_spills = allow_spills
+        self._tiles_given = tiles is not None
         q_meta, k_meta, v_meta = qkv_meta
         self.dtype = q_meta.dtype
         self.D = int(q_meta.shape[3])
@@ -140,15 +145,38 @@ class PrefillOp:
         B, H, Sq, Skv = self.meta_shape
         self.source = self.functor_src
         if Sq > 0:
-            plan = self._plan(B, H, Sq, Skv, device=None)
-            mode = 2 if self.extern_block_mask else plan.mode
-            n_split, _ = self.plan_splits(B, H, Sq, Skv)
-            _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split,
-                                          self._table_rows(self.mask_block[0] if self.extern_block_mask else plan.block_m),
-                                          plan.heavy_last and not self.extern_block_mask)
-            self.source = cfg_src + "\n" + self.functor_src
-            if infer_mask and mask_mod is not None and not self.extern_block_mask:
-                self.block_mask = self._reference_block_mask(B, H, Sq, Skv)
+            try:
+                self._compile_declared_shape(B, H, Sq, Skv, infer_mask, mask_mod)
+            except rt.SpillError:
+                if not self._gives_way_to_the_generic_kernel():
+                    raise
+                self._compile_declared_shape(B, H, Sq, Skv, infer_mask, mask_mod)
+
+    def _gives_way_to_the_generic_kernel(self) -> bool:
+        """A build of the software-pipelined kernel that spills registers is refused (hip_rt.check_spills).  Where
+        that kernel was this operator's own choice -- not the caller's (``tiles=``, the tuner) -- the operator
+        switches to the generic kernel, whose two waves per SIMD leave the compiler room, for every later launch:
+        True if it did.  (The pipelined kernel holds 64 query rows per wave in one wave per SIMD and fills the
+        register file; its fp16 builds fit, some bf16 builds at head dim 128 spill a few values.)"""
+        if self._tiles_given or self.tiles.template != "ae_prefill_pipe.hip":
+            return False
+        self.tiles = L.PrefillTiles()
+        self._variants.clear()
+        self._plans.clear()
+        self._bwd = None            # (the backward reads this operator's mask plans: built again on demand)
+        self.gave_way_to_generic = True
+        return True
+
+    def _compile_declared_shape(self, B, H, Sq, Skv, infer_mask, mask_mod):
+        plan = self._plan(B, H, Sq, Skv, device=None)
+        mode = 2 if self.extern_block_mask else plan.mode
+        n_split, _ = self.plan_splits(B, H, Sq, Skv)
+        _, _, cfg_src = self._variant(mode, Sq % self.tiles.block_m == 0, Skv % self.tiles.block_n == 0, n_split,
+                                      self._table_rows(self.mask_block[0] if self.extern_block_mask else plan.block_m),
+                                      plan.heavy_last and not self.extern_block_mask)
+        self.source = cfg_src + "\n" + self.functor_src
+        if infer_mask and mask_mod is not None and not self.extern_block_mask:
+            self.block_mask = self._reference_block_mask(B, H, Sq, Skv)
 
     def _probe_mask_mode(self, q_meta, v_meta):
         """Mode of the mask plan at the declared sequence lengths (4096 where they are dynamic), for batch entry
@@ -279,7 +307,10 @@ class PrefillOp:
             if self._clock_stamps():
                 cfg_src += "#define AE_CLOCK_STAMPS 1\n"
             module = rt.compile_module(self.tiles.template, {"ae_config.h": cfg_src,
-                                                          "ae_functors.h": self.functor_src})
+                                                          "ae_functors.h": self.functor_src},
+                                       allow_spills=self.allow_spills,
+                                       # the builds in which a spilled tuple came back wrong: 256 accumulator registers
+                                       strict_spills=self.tiles.template == "ae_prefill.hip" and self.DV_launch > 256)
             cfg = rt.TileCfg(block_m=self.tiles.block_m, block_n=self.tiles.block_n,
                              threads=64 * self.tiles.n_waves,
                              lds_bytes=self.tiles.lds_bytes(self.D, self.DV_launch) + self._kv_custom_scratch(), head_dim=self.D,
@@ -299,10 +330,20 @@ class PrefillOp:
     def backward_op(self):
         if getattr(self, "_bwd", None) is None:
             from .prefill_bwd_op import PrefillBwdOp
-            self._bwd = PrefillBwdOp(self, *self._graph, tune=self._tune_bwd[0], tune_file=self._tune_bwd[1])
+            self._bwd = PrefillBwdOp(self, *self._graph, tune=self._tune_bwd[0], tune_file=self._tune_bwd[1],
+                                     allow_spills=self.allow_spills)
         return self._bwd
 
     def _forward(self, q, k, v, *extra):
+        try:
+            return self._forward_once(q, k, v, *extra)
+        except rt.SpillError:
+            # (raised by the compilation of a variant, before anything was launched)
+            if not self._gives_way_to_the_generic_kernel():
+                raise
+            return self._forward_once(q, k, v, *extra)
+
+    def _forward_once(self, q, k, v, *extra):
         if self._tune_pending:
             self._tune(q, k, v, *extra)
         n_custom = len(self.functors.customs)
@@ -427,14 +468,19 @@ class _PrefillFunction(torch.autograd.Function):
         if bwd is None:
             return out
         ctx.customs = tuple(extra[:len(op.functors.customs)])       # scalar CustomIO tensors of score_mod
-        lse = op.final_rowscales[bwd.lse_name] if bwd.lse_name is not None else q.new_empty(0)
-        ctx.save_for_backward(q, k, v, out, lse)
+        # the user's block mask of this call (engines built with extern_block_mask=True): last positional
+        ctx.block_mask = extra[-1] if (op.extern_block_mask and len(extra) == len(op.functors.customs) + 1) else None
+        # the final row scales the backward reads: lse, or every final row scale of an online function whose
+        # forward() / backward() are traced
+        scales = [op.final_rowscales[n] for n in bwd.rowscale_names] or [q.new_empty(0)]
+        ctx.save_for_backward(q, k, v, out, *scales)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         if ctx.no_backward is not None:
             raise NotImplementedError(str(ctx.no_backward)) from ctx.no_backward
-        q, k, v, out, lse = ctx.saved_tensors
-        dq, dk, dv = ctx.op.backward_op()(q, k, v, out, lse, dout, ctx.customs)
+        q, k, v, out, *scales = ctx.saved_tensors
+        lse = scales[0] if len(scales) == 1 else scales
+        dq, dk, dv = ctx.op.backward_op()(q, k, v, out, lse, dout, ctx.customs, ctx.block_mask)
         return (None, dq, dk, dv) + (None,) * ctx.n_extra

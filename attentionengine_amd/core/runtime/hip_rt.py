@@ -73,10 +73,12 @@ class AttnBwdParams(C.Structure):
     _fields_ = (
         [(n, C.c_void_p) for n in ("q", "k", "v", "out", "dout", "lse", "delta", "dq", "dk", "dv",
                                    "mask_dq", "mask_dkv")]
-        + [("custom", C.c_void_p * AE_MAX_CUSTOM)]
+        + [("custom", C.c_void_p * AE_MAX_CUSTOM), ("block_mask", C.c_void_p),
+           ("more_rowscales", C.c_void_p * (AE_MAX_ROWSCALES - 1))]
         + [(f"{t}_stride_{a}", C.c_int64) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for a in "bsh"]
         + [("batch", C.c_int32), ("heads_q", C.c_int32), ("heads_kv", C.c_int32),
            ("seqlen_q", C.c_int32), ("seqlen_kv", C.c_int32), ("mask_b", C.c_int32), ("mask_h", C.c_int32),
+           ("mask_nq", C.c_int32), ("mask_nkv", C.c_int32), ("mask_block_m", C.c_int32), ("mask_block_n", C.c_int32),
            ("reserved", C.c_int32 * 1)]
     )
 
@@ -272,6 +274,32 @@ class Module:
                     return {k[".name"]: k for k in md.get("amdhsa.kernels", [])}
         raise AEError("code object without an AMDGPU metadata note")
 
+    def scratch_accesses(self) -> dict:
+        """{"single": n, "wide": m}: scratch-memory instructions in the code object's .text that move one
+        dword, and those that move two to four (``scratch_load/store_dwordx2/x3/x4``) -- the form in which the
+        compiler spills and reloads register TUPLES (matrix accumulators, MFMA operands).  Found by matching
+        the instruction words (FLAT encoding, scratch segment); no disassembler is involved."""
+        import struct
+        f = self.code()
+        shoff = struct.unpack_from("<Q", f, 0x28)[0]
+        shentsize, shnum, shstrndx = struct.unpack_from("<HHH", f, 0x3A)
+        secs = [struct.unpack_from("<IIQQQQ", f, shoff + i * shentsize) for i in range(shnum)]
+        strtab = secs[shstrndx][4]
+        out = {"single": 0, "wide": 0}
+        for name_off, typ, _, _, offset, size in secs:
+            name = f[strtab + name_off:f.index(b"\0", strtab + name_off)]
+            if name != b".text":
+                continue
+            for (w,) in struct.iter_unpack("<I", f[offset:offset + (size & ~3)]):
+                if (w & 0xFC00C000) != 0xDC004000:        # FLAT encoding, segment = scratch
+                    continue
+                op = (w >> 18) & 0x7F
+                if op in (20, 28):                          # scratch_load_dword, scratch_store_dword
+                    out["single"] += 1
+                elif op in (21, 22, 23, 29, 30, 31):        # ..._dwordx2, x3, x4
+                    out["wide"] += 1
+        return out
+
     def kernel(self, name: str) -> Kernel:
         k = self._kernels.get(name)
         if k is None:
@@ -291,13 +319,76 @@ _modules = {}
 _modules_lock = threading.Lock()
 
 
-def compile_module(template: str, headers: dict, arch: str = None, use_cache: bool = True) -> Module:
+class SpillError(AEError):
+    """A compiled kernel keeps part of its vector registers in scratch memory (see ``check_spills``)."""
+
+
+# scratch bytes per lane beyond which a build counts as spilling heavily (slow, and refused)
+MAX_SCRATCH_BYTES = 128
+
+
+def check_spills(module: "Module", what: str, allow_spills=None, strict=False):
+    """Warns about -- or, where asked to be strict, refuses -- a code object that moves register TUPLES through
+    scratch memory or spills heavily.
+
+    Every attention template holds its matrix accumulators as 16-register tuples, several of them pinned to the
+    accumulator file by ``asm`` statements.  One build of the compiler in use (wide value heads, tile table, ragged
+    tiles: 16 spilled values) spilled such a tuple -- twelve registers with three ``scratch_store_dwordx4``, a
+    thirteenth alone, three kept in other registers -- and, where it put the tuple together again, never emitted
+    the copy of one of the three: the reloaded tuple carried a stale register and the kernel returned one wrong
+    pair of output columns, silently (found by reading that build's code; the kernel has since been changed so
+    that the build no longer spills).  Builds that spill a few single values (a row's running maximum, a lane
+    index: plain ``scratch_store_dword`` / ``scratch_load_dword``) take none of that path.
+
+    A build is SUSPECT when its code contains scratch accesses wider than one dword, or when it keeps more than
+    MAX_SCRATCH_BYTES per lane in scratch memory.  Many of the less common configurations (odd head-dim pairs,
+    decode shapes with few heads, backward launches under elementwise masks) are suspect builds that pass their
+    parity tests, so by default a suspect build only raises a RuntimeWarning naming the kernel.  It is refused
+    (SpillError) when ``strict`` is set -- the operators set it for the family of builds in which the wrong
+    columns were seen, the wide value heads of ae_prefill.hip, which do not spill as the kernel stands -- when
+    ``allow_spills`` is False (``AttentionEngine(..., allow_spills=False)``), or with AE_ALLOW_SPILLS=0 in the
+    environment, which refuses every build that spills at all.  ``allow_spills=True`` / AE_ALLOW_SPILLS=1
+    switch the check off."""
+    env = os.environ.get("AE_ALLOW_SPILLS", "")
+    if allow_spills is True or (allow_spills is None and env == "1"):
+        return
+    info = module.kernel_info()
+    spilling = {name: (k.get(".vgpr_spill_count", 0), k.get(".private_segment_fixed_size", 0))
+                for name, k in info.items() if k.get(".vgpr_spill_count", 0)}
+    if not spilling:
+        return
+    acc = module.scratch_accesses()
+    heavy = any(b > MAX_SCRATCH_BYTES for _, b in spilling.values())
+    if not (acc["wide"] or heavy or env == "0"):
+        return
+    text = ", ".join(f"{n}: {c} spilled registers, {b} bytes of scratch per lane" for n, (c, b) in sorted(spilling.items()))
+    why = (f"{acc['wide']} scratch accesses wider than one dword: a register tuple goes through scratch memory"
+           if acc["wide"] else "it spills heavily" if heavy else "AE_ALLOW_SPILLS=0")
+    msg = (f"{what}: the compiled kernel spills vector registers ({text}; {why}).  One such build has returned wrong "
+           "results (a register tuple put together again from scratch memory lost a register)")
+    if strict or allow_spills is False or env == "0":
+        raise SpillError(msg + "; this build is refused -- choose other head dims / tiles, or pass allow_spills=True "
+                               "(AE_ALLOW_SPILLS=1) to run it anyway")
+    import warnings
+    warnings.warn(msg + "; check its results, or pass allow_spills=False to refuse such builds", RuntimeWarning,
+                  stacklevel=3)
+
+
+def compile_module(template: str, headers: dict, arch: str = None, use_cache: bool = True,
+                   allow_spills=None, strict_spills=False) -> Module:
     """Compile kernel template ``template`` (a file name under csrc/kernels) with the generated
     in-memory ``headers`` ({"ae_config.h": text, "ae_functors.h": text}).
 
     The code object is cached on disk under a key that covers the template text, every header,
-    the architecture and the compiler options, and in memory for the life of the process.
+    the architecture and the compiler options, and in memory for the life of the process.  A code object
+    that moves register tuples through scratch memory is reported or refused (``check_spills``).
     """
+    m = _compile_module(template, headers, arch, use_cache)
+    check_spills(m, template, allow_spills, strict_spills)
+    return m
+
+
+def _compile_module(template: str, headers: dict, arch: str = None, use_cache: bool = True) -> Module:
     arch = arch or os.environ.get("AE_HIP_ARCH", "gfx950")
     src = _read(osp.join(KERNEL_DIR, template))
     all_headers = {

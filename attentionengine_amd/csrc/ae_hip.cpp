@@ -638,6 +638,14 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
     if ((p->mask_b != 1 && p->mask_b != p->batch) || (p->mask_h != 1 && p->mask_h != p->heads_q))
       return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: table batch/head extent (%d,%d) must be 1 or (B,Hq)",
                   p->mask_b, p->mask_h);
+    // a block mask of the user's (kernels built with AE_EXT_BLOCK_MASK 1 read it per element on partly visible tiles)
+    if (p->block_mask && (p->mask_nq <= 0 || p->mask_nkv <= 0 || p->mask_block_m <= 0 || p->mask_block_n <= 0 ||
+                          (int64_t)p->mask_nq * p->mask_block_m < p->seqlen_q ||
+                          (int64_t)p->mask_nkv * p->mask_block_n < p->seqlen_kv))
+      return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: block mask [%d x %d] of %dx%d blocks does not cover %d x %d",
+                  p->mask_nq, p->mask_nkv, p->mask_block_m, p->mask_block_n, p->seqlen_q, p->seqlen_kv);
+  } else if (p->block_mask) {
+    return fail(AE_ERR_INVALID_ARG, "ae_prefill_bwd: a block mask was passed to kernels built without tile-class tables");
   }
   const uint64_t rows = (uint64_t)p->batch * p->seqlen_q * p->heads_q;
   const uint64_t rows_per_wg = 256u / (uint32_t)(cfg->head_dim_v / 8);

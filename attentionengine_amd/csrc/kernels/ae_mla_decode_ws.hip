@@ -85,7 +85,9 @@ static_assert(AE_NSTAGE >= 3, "a tile is multiplied by K one trip before it is m
 #endif
 // 1 (single-split builds only, a measurement switch): every workgroup reports the shader-clock cycles (s_memtime)
 // and the constant-rate 100 MHz ticks (s_memrealtime) between its entry and its last store, as two 64-bit values
-// at ((unsigned long long*)p.partial_o)[2 * blockIdx.x] - a buffer a single-split launch does not otherwise use.
+// at ((unsigned long long*)p.partial_o)[2 * blockIdx.x] - a buffer a single-split launch does not otherwise use -
+// and, behind the pairs of all workgroups (at index 2 * gridDim.x + 4 * blockIdx.x), four more tick values of one
+// value wave: entry, first tile landed, last trip done, last store acknowledged (absolute 100 MHz ticks).
 #ifndef AE_CLOCK_STAMPS
 #define AE_CLOCK_STAMPS 0
 #endif
@@ -487,6 +489,9 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
   for (int t = 0; t < AE_NSTAGE - 1; t++) load_tile(t);
   __builtin_amdgcn_s_waitcnt(AE_VMCNT((AE_NSTAGE - 2) * AE_LOADS));
   __syncthreads();
+#if AE_CLOCK_STAMPS
+  const unsigned long long ae_w1 = __builtin_amdgcn_s_memrealtime();     // tile 0 (and Q) have landed
+#endif
 
   // V^T fragment (k-step kk, dv block db): A[m = dv][k = kv]: lane i of a 16-lane group supplies the
   // address of row 16*kk + 8*hf + i/4 (+4 for slots 4..7), 8 bytes at value column
@@ -575,6 +580,9 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
     end_trip(n_tiles);
   }
   __builtin_amdgcn_s_waitcnt(AE_VMCNT(0));   // (the last barrier also made the final (m, r) of every head visible)
+#if AE_CLOCK_STAMPS
+  const unsigned long long ae_w2 = __builtin_amdgcn_s_memrealtime();     // the last trip is done
+#endif
 
   // ---- per-split epilogue: lane owns head 32*hb + l32, value columns AE_DVW*dvw + 32*db + 8*(r/4) + 4*hf + r%4
 #pragma unroll
@@ -651,6 +659,12 @@ void ae_mla_decode_split_kernel(const ae_attn_params p) {
       unsigned long long* st = (unsigned long long*)p.partial_o + 2 * (unsigned long long)blockIdx.x;
       st[0] = t1 - ae_t0;
       st[1] = w1 - ae_w0;
+      unsigned long long* ph = (unsigned long long*)p.partial_o + 2 * (unsigned long long)gridDim.x +
+                               4 * (unsigned long long)blockIdx.x;
+      ph[0] = ae_w0;
+      ph[1] = ae_w1;
+      ph[2] = ae_w2;
+      ph[3] = w1;
     }
   }
 #endif

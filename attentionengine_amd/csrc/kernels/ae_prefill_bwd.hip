@@ -28,6 +28,9 @@
 // tile-class tables built on the host from mask_mod (0 skip, 1 test per element, 2 fully visible), one
 // per launch because the two tile shapes differ: [q tiles of 32*AE_BWD_NWAVES][kv tiles of 64] for dq,
 // [q tiles of 64][kv tiles of 128] for dk/dv (role of blockattn_tl.py's block mask in the backward).
+// AE_EXT_BLOCK_MASK 1: the forward ran on a block mask the user supplied (blockattn_tl.py:195-470 is the
+// reference's backward for it); the two tables are then made from that mask, and a tile of class 1 - one that
+// straddles blocks of both kinds - looks every element up in the user's mask (ae_attn_bwd_params.block_mask).
 //
 // Waves per workgroup (AE_BWD_NWAVES, 32 resident rows each): dk/dv runs four, one per SIMD with the
 // whole register file (two accumulators). dq has one accumulator and fits 256 registers, so it runs
@@ -45,7 +48,8 @@
 // generated ae_bwd_pd (f' by symbolic differentiation of the traced score_mod); no row scales, scale 1.
 //
 // Configuration ("ae_config.h"): AE_D AE_DV AE_DTYPE_BF16 AE_MASK_MODE (0, 1, 2) AE_HAS_MASK_MOD
-// AE_SM_SCALE AE_BWD_ROLE AE_BWD_KIND, optional AE_BWD_NWAVES (4 or 8) AE_BWD_WAVES_PER_EU AE_AHEAD.  Functors used ("ae_functors.h"): ae_mask_mod; kind 1: ae_bwd_pd,
+// AE_SM_SCALE AE_BWD_ROLE AE_BWD_KIND, optional AE_BWD_NWAVES (4 or 8) AE_BWD_WAVES_PER_EU AE_AHEAD AE_BWD_NRS (kind 2:
+// final row scales of the online function, 1 .. AE_MAX_ROWSCALES).  Functors used ("ae_functors.h"): ae_mask_mod; kind 1: ae_bwd_pd,
 // ae_bwd_load_custom; kind 2: ae_bwd_pd2.
 
 #include "ae_hip.h"
@@ -54,6 +58,9 @@
 #include "ae_functors.h"
 #ifndef AE_HEAVY_LAST
 #define AE_HEAVY_LAST 0
+#endif
+#ifndef AE_EXT_BLOCK_MASK
+#define AE_EXT_BLOCK_MASK 0
 #endif
 
 #ifndef AE_BWD_NWAVES
@@ -69,7 +76,15 @@
 #define AE_CPR2 (AE_DV / 8)
 #define AE_T1_BYTES (AE_BS * AE_STR1)
 #define AE_T2_BYTES (AE_BS * AE_STR2)
-#define AE_STAGE_BYTES (AE_T1_BYTES + AE_T2_BYTES + 2 * AE_BS * 4)   // + lse, rowsum(do*o) of the streamed rows
+// per-row values that travel with a streamed tile of the dk / dv launch: rowsum(do*o), and lse - or, kind 2, the
+// AE_BWD_NRS final row scales of the online function (planes of the work buffer `delta`: 0 = rowsum(do*o), 1 + i =
+// row scale i).  In LDS, behind the tile: row scale 0 first, rowsum(do*o) second, further row scales after them.
+#ifndef AE_BWD_NRS
+#define AE_BWD_NRS 1
+#endif
+#define AE_RS_PLANES (1 + AE_BWD_NRS)
+#define AE_RS_SLOT(plane) ((plane) == 0 ? 1 : ((plane) == 1 ? 0 : (plane)))
+#define AE_STAGE_BYTES (AE_T1_BYTES + AE_T2_BYTES + AE_RS_PLANES * AE_BS * 4)
 #define AE_NKS1 (AE_D / 16)        // k-steps of S
 #define AE_NKS2 (AE_DV / 16)       // k-steps of dP
 #define AE_NDB1 (AE_D / 32)        // 32-wide output blocks of dQ / dK
@@ -82,7 +97,8 @@
 #ifndef AE_BWD_WAVES_PER_EU
 #define AE_BWD_WAVES_PER_EU 1
 #endif
-#define AE_NLOADS (AE_L1 + AE_L2 + (AE_BWD_ROLE == 1 ? 1 : 0))   // load instructions per wave and tile
+#define AE_RSL ((AE_RS_PLANES + AE_NWAVES - 1) / AE_NWAVES)      // row-value loads per wave and tile (dk / dv launch)
+#define AE_NLOADS (AE_L1 + AE_L2 + (AE_BWD_ROLE == 1 ? AE_RSL : 0))   // load instructions per wave and tile
 #define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
 #ifndef AE_AHEAD
 #define AE_AHEAD 4                 // LDS fragments in flight ahead of the MFMA that uses them
@@ -244,6 +260,9 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #if AE_BWD_ROLE == 0
   // row scales of the lane's q row: lse in log2 units (+inf for a row without a visible key: p = 0)
   float lse2_r, delta_r;
+#if AE_BWD_KIND == 2 && AE_BWD_NRS > 1
+  float rs_more[AE_BWD_NRS - 1];      // the online function's further final row scales of the lane's row
+#endif
   {
     const int64_t ri = ((int64_t)b * p.heads_q + h) * p.seqlen_q + rrow_c;
 #if AE_BWD_FUSE_DELTA
@@ -253,6 +272,10 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #else
     delta_r = p.delta[ri];
     lse2_r = p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri];
+#endif
+#if AE_BWD_KIND == 2 && AE_BWD_NRS > 1
+#pragma unroll
+    for (int i = 1; i < AE_BWD_NRS; i++) rs_more[i - 1] = p.delta[(int64_t)(1 + i) * p.batch * p.heads_q * p.seqlen_q + ri];
 #endif
   }
 #endif
@@ -391,13 +414,17 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
     ae_load_lds16_burst_base<AE_L2>(x2 - 4096, g2, t2 + (wave * AE_L2 + AE_L2 / 2) * 1024);
 #if AE_BWD_ROLE == 1
     {
-      // lse (log2 units) and rowsum(do * o) of the tile's 64 q rows: even waves fetch the one, odd waves
-      // the other (twice each, so that every wave issues the same number of loads)
+      // rowsum(do * o) and lse in log2 units (kind 2: the final row scales) of the tile's 64 q rows: the waves share
+      // the planes out, every wave issuing the same number of loads (planes are fetched more than once where there
+      // are fewer of them than waves)
       int row = s0 + lane;
       row = row < n_str ? row : n_str - 1;
-      const int plane = (wave & 1) ^ 1;                // plane 0: rowsum(do * o), plane 1: lse
-      const float* src = p.delta + ((int64_t)plane * p.batch * p.heads_q + (int64_t)b * p.heads_q + hq) * p.seqlen_q + row;
-      ae_load_lds4(src, t2 + AE_T2_BYTES + (wave & 1) * AE_BS * 4);
+#pragma unroll
+      for (int i = 0; i < AE_RSL; i++) {
+        const int plane = (wave + AE_NWAVES * i) % AE_RS_PLANES;
+        const float* src = p.delta + ((int64_t)plane * p.batch * p.heads_q + (int64_t)b * p.heads_q + hq) * p.seqlen_q + row;
+        ae_load_lds4(src, t2 + AE_T2_BYTES + AE_RS_SLOT(plane) * AE_BS * 4);
+      }
     }
 #endif
   };
@@ -545,7 +572,7 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #if AE_MASK_MODE == 2
     bool need_vis = cls0 != 2 || s0 + AE_BS > n_str || r0w + 32 > n_res;
 #else
-    bool need_vis = (AE_HAS_MASK_MOD != 0) || s0 + AE_BS > n_str || r0w + 32 > n_res;
+    bool need_vis = (AE_HAS_MASK_MOD != 0) || (AE_EXT_BLOCK_MASK != 0) || s0 + AE_BS > n_str || r0w + 32 > n_res;
 #endif
 #if AE_MASK_MODE == 1
     need_vis = need_vis || (AE_BWD_ROLE == 0 ? s0 + AE_BS - 1 > r0w : s0 < r0w + 31);
@@ -599,9 +626,20 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
         dfac *= pacc[r];
         (void)l2; (void)dl;
 #else
-        // traced OnlineFunc.forward / backward: l2 is the row's final row scale as the forward wrote it
+        // traced OnlineFunc.forward / backward: l2 is the row's (first) final row scale as the forward wrote it
         float pv, dfac;
-        ae_bwd_pd2(sacc[r], pacc[r], l2, dl, b, hq, qi, ki, p, pv, dfac);
+        float rsv[AE_BWD_NRS];
+        rsv[0] = l2;
+#if AE_BWD_NRS > 1
+#pragma unroll
+        for (int i = 1; i < AE_BWD_NRS; i++)
+#if AE_BWD_ROLE == 0
+          rsv[i] = rs_more[i - 1];
+#else
+          rsv[i] = rs_l[(1 + i) * AE_BS + sl];
+#endif
+#endif
+        ae_bwd_pd2(sacc[r], pacc[r], rsv, dl, b, hq, qi, ki, p, pv, dfac);
 #endif
         bool vis = true;
         if (decltype(masked)::value) {
@@ -611,6 +649,16 @@ void AE_BWD_KERNEL(const ae_attn_bwd_params p) {
 #endif
 #if AE_HAS_MASK_MOD
           vis = vis && ae_mask_mod(b, hq, qi, ki);
+#endif
+#if AE_EXT_BLOCK_MASK
+          {
+            // the user's block of this (q, kv) position (positions past the end are invisible anyway: clamped)
+            int mr = qi / p.mask_block_m, mc = ki / p.mask_block_n;
+            mr = mr < p.mask_nq ? mr : p.mask_nq - 1;
+            mc = mc < p.mask_nkv ? mc : p.mask_nkv - 1;
+            const int64_t mbh = (int64_t)(p.mask_b == 1 ? 0 : b) * p.mask_h + (p.mask_h == 1 ? 0 : hq);
+            vis = vis && p.block_mask[(mbh * p.mask_nq + mr) * p.mask_nkv + mc] != 0;
+          }
 #endif
           pv = vis ? pv : 0.f;
         }
@@ -812,8 +860,11 @@ void ae_bwd_delta_kernel(const ae_attn_bwd_params p) {
     const float l = p.lse ? p.lse[ri] : 0.f;
     p.delta[ri] = acc;
 #if AE_BWD_KIND == 2
-    // second plane: the online function's final row scale, as the forward wrote it
+    // further planes: the online function's final row scales, as the forward wrote them
     p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = l;
+#pragma unroll
+    for (int i = 1; i < AE_BWD_NRS; i++)
+      p.delta[(int64_t)(1 + i) * p.batch * p.heads_q * p.seqlen_q + ri] = p.more_rowscales[i - 1][ri];
 #else
     // second plane: lse in log2 units, +inf for a row without a visible key (its p is 0 everywhere)
     p.delta[(int64_t)p.batch * p.heads_q * p.seqlen_q + ri] = (l == AE_NEG_INF) ? __builtin_inff() : l * AE_LOG2E;

@@ -109,6 +109,12 @@
 
 typedef __attribute__((address_space(3))) unsigned char ae_lds_byte;
 #define AE_SB() __builtin_amdgcn_sched_barrier(0)
+// C operand of a tile's first k-step for q block qb
+#if AE_PRESCALE
+#define AE_C0(qb) negc[qb]
+#else
+#define AE_C0(qb) zero16
+#endif
 
 struct ae_tag_true { static constexpr bool value = true; };
 struct ae_tag_false { static constexpr bool value = false; };
@@ -333,7 +339,15 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // thr is what a tile maximum (relative to the reference) must exceed before the reference moves: 8
   // (p stays below 256), or -inf while the row has not seen a visible key and its reference is unset.
   float m2[2], r_run[2], thr[2];
+#if AE_PRESCALE
   ae_f32x16 negc[2];
+#else
+  // (the first k-step starts from the constant 0, an operand the MFMA encodes itself: sixteen registers of
+  // zeros per q block in the accumulator file, and the copies out of them, are what made the bf16 builds spill)
+  ae_f32x16 zero16;
+#pragma unroll
+  for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+#endif
   ae_elem8 zero8;
 #pragma unroll
   for (int i = 0; i < 8; i++) zero8[i] = (ae_elem)0.f;
@@ -355,7 +369,9 @@ void ae_prefill_kernel(const ae_attn_params p) {
     m2[qb] = 0.f;
     thr[qb] = AE_NEG_INF;
     r_run[qb] = 0.f;                  // per-lane partial sum; the two halves of a row meet in the epilogue
+#if AE_PRESCALE
     negc[qb] = acc_splat(0.f);
+#endif
 #pragma unroll
     for (int db = 0; db < AE_NDB; db++)
 #pragma unroll
@@ -585,7 +601,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
       const ae_elem8 kf = read_kfrag(f, lds);
 #pragma unroll
       for (int qb = 0; qb < 2; qb++) {
-        sacc[f & 1][qb] = ae_mfma32(kf, qf[qb][f >> 1], f < 2 ? negc[qb] : sacc[f & 1][qb]);
+        sacc[f & 1][qb] = ae_mfma32(kf, qf[qb][f >> 1], f < 2 ? AE_C0(qb) : sacc[f & 1][qb]);
       }
     }
     mx[0] = mx[1] = AE_NEG_INF;
@@ -655,7 +671,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
         if (f + AE_AHEAD < NF) ring[(f + AE_AHEAD) % AE_RING] = read_frag(f + AE_AHEAD);
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
-          sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], f < 2 ? negc[qb] : sacc[f & 1][qb]);
+          sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], f < 2 ? AE_C0(qb) : sacc[f & 1][qb]);
           exp_slot(2 * f + qb);
           if (2 * f + qb == AE_KLOAD_SLOT) load_k(j2l, n & 1);
           if (2 * f + qb == AE_VLOAD_SLOT) load_v(j1, (n + 1) & 1);

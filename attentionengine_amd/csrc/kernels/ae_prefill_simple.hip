@@ -251,6 +251,12 @@ void ae_prefill_kernel(const ae_attn_params p) {
   int j = next_tile(0);
   bool any_tile = j < j_end;
   int cls[AE_RB];          // class of tile j for this lane's row of each row block
+  // 1 once this lane's row of a row block has met a key it may see.  A row that never does - inside a q tile whose
+  // other rows do: block masks finer than the q tile, masks such as q - 100 >= kv - ends with out = 0 and row
+  // scales of -inf, like the rows of a q tile without any tile (not with the 0 / 0 its epilogue would make of it)
+  float seen[AE_RB];
+#pragma unroll
+  for (int rb = 0; rb < AE_RB; rb++) seen[rb] = 0.f;
 #pragma unroll
   for (int rb = 0; rb < AE_RB; rb++) cls[rb] = row_class(j, rb);
   if (any_tile) {
@@ -310,13 +316,16 @@ void ae_prefill_kernel(const ae_attn_params p) {
       const int kvb = ctx[rb].kv_base;
 
       // ---- mask (additive -inf before score_mod, attn_tl.py:124-137) --------------------------
+      bool masked_here = false;    // some score of this row block was tested on this tile
 #if AE_MASK_MODE == 1
       if (kv0 + AE_BN - 1 > q0w + rb * 32) {  // tile crosses the diagonal of this row block
+        masked_here = true;
 #pragma unroll
         for (int e = 0; e < AE_NS; e++) s[e] = (qrow[rb] >= kvb + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
       }
 #elif AE_MASK_MODE == 2 && !(defined(AE_MASK_VALUE_ZERO) && AE_MASK_VALUE_ZERO)
       if (__builtin_amdgcn_ballot_w64(cls[rb] != 2) != 0) {   // some row of this block does not see the whole tile
+        masked_here = true;
 #pragma unroll
         for (int e = 0; e < AE_NS; e++) {
 #if AE_HAS_MASK_MOD
@@ -329,6 +338,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
       }
 #elif AE_HAS_MASK_MOD
       {
+        masked_here = true;
 #pragma unroll
         for (int e = 0; e < AE_NS; e++)
           s[e] = ae_mask_mod(b, h, qrow[rb], kvb + ae_kv_off(e)) ? s[e] : AE_NEG_INF;
@@ -336,10 +346,19 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #endif
 #if !AE_EVEN_KV
       if (kv0 + AE_BN > p.seqlen_kv) {
+        masked_here = true;
 #pragma unroll
         for (int e = 0; e < AE_NS; e++) s[e] = (kvb + ae_kv_off(e) < p.seqlen_kv) ? s[e] : AE_KV_PAD;
       }
 #endif
+      if (masked_here) {           // (an untested tile is visible to every row)
+        float top = s[0];
+#pragma unroll
+        for (int e = 1; e < AE_NS; e++) top = __builtin_fmaxf(top, s[e]);
+        seen[rb] = top > AE_NEG_INF ? 1.f : seen[rb];
+      } else {
+        seen[rb] = 1.f;
+      }
 
       // ---- user functors ----------------------------------------------------------------------
       ae_score_mod<AE_NS>(s, ctx[rb], cust[rb]);
@@ -413,10 +432,14 @@ void ae_prefill_kernel(const ae_attn_params p) {
       for (int r = 0; r < 16; r++) o[db * 16 + r] = oacc[rb][db][r];
     float frs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
     frs[0] = 0.f;
-    if (any_tile) {
+    const bool row_seen = ae_group_max(seen[rb]) > 0.f;     // (both lanes of a row, or neither)
+    if (any_tile && row_seen) {
       ae_epilogue<AE_NO>(o, st[rb], frs, ctx[rb], cust[rb]);
     } else {
-      // no visible kv block for this q-tile: out = 0 (blockattn_tl.py:153-160), rowscales = -inf
+      // no visible kv block for this q-tile, or no visible key for this row: out = 0 (blockattn_tl.py:153-160),
+      // rowscales = -inf
+#pragma unroll
+      for (int e = 0; e < AE_NO; e++) o[e] = 0.f;
 #pragma unroll
       for (int i = 0; i < AE_N_ROWSCALES; i++) frs[i] = AE_NEG_INF;
     }

@@ -146,6 +146,19 @@ def measure(name, steps, warmup):
     stamps = getattr(getattr(mod, "_op", None), "clock_stamps", None)     # builds with AE_CLOCK_STAMPS=1 only
     if stamps is not None:
         res["clock_mhz"] = _clock_mhz(stamps)
+        ph = getattr(getattr(mod, "_op", None), "phase_ticks", None)
+        if ph is not None:
+            # where a workgroup's time goes, microseconds (100 MHz ticks): launch start = the earliest entry
+            t = ph.cpu().double()
+            t = t[t[:, 3] > 0]
+            t0 = t[:, 0].min()
+            res["phases_us"] = {"first_entry_to_last_exit": float((t[:, 3].max() - t0) / 100.0),
+                                "entry_after_launch_start_max": float((t[:, 0].max() - t0) / 100.0),
+                                "prologue_median": float((t[:, 1] - t[:, 0]).median() / 100.0),
+                                "loop_median": float((t[:, 2] - t[:, 1]).median() / 100.0),
+                                "epilogue_median": float((t[:, 3] - t[:, 2]).median() / 100.0),
+                                "workgroup_median": float((t[:, 3] - t[:, 0]).median() / 100.0),
+                                "workgroup_max": float((t[:, 3] - t[:, 0]).max() / 100.0)}
     if kind in ("prefill", "prefill_bwd"):
         ach = info["flops"] / (ev_ms * 1e-3) / 1e12
         res["roofline"] = {"bound": "mfma", "achieved": ach, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
@@ -353,6 +366,10 @@ def mfma_probe_report(steps, warmup):
         tf = r["flops"] / (r["kernel_ms"] * 1e-3) / 1e12
         at_clock = MFMA_FLOP_PER_CLK * clk * 1e6 / 1e12
         rec[name] = {"tflops": tf, "ms": r["kernel_ms"], "clock_mhz": clk}
+        if "phases_us" in r:
+            rec[name]["phases_us"] = r["phases_us"]
+            lines.append(f"#   {name} workgroup phases, microseconds: " +
+                         ", ".join(f"{k} {v:.1f}" for k, v in r["phases_us"].items()))
         lines.append(f"{name}, {tf:.0f}, {r['kernel_ms']:.4f}, {clk:.0f}, {at_clock:.0f}, {tf / at_clock:.3f}, "
                      f"{tf / PEAK_MFMA_TFLOPS:.3f}")
     print("\n".join(lines))

@@ -143,7 +143,8 @@ typedef struct ae_tile_cfg {
  * Kernel argument block of the backward kernels (softmax attention, prefill shapes). Same layouts as
  * ae_attn_params; dout [B,Sq,Hq,DV] is the gradient of `out`, dq/dk/dv have the shapes of q/k/v, lse
  * is the forward's natural-log row scale fp32 [B,Hq,Sq] (NULL for graphs without row scales), delta a caller-allocated fp32 [2,B,Hq,Sq]
- * work buffer (the first launch fills it: rowsum(dout * out), and lse in log2 units). Stands where the reference passes Q, K, V, dO, lse
+ * work buffer (the first launch fills it: rowsum(dout * out), and lse in log2 units; [1 + AE_BWD_NRS,B,Hq,Sq] for kernels that read
+ * several final row scales). Stands where the reference passes Q, K, V, dO, lse
  * and Delta to flashattn_bwd (core/template/tl_template/attn/attn_tl.py:271-295).
  */
 typedef struct ae_attn_bwd_params {
@@ -160,6 +161,16 @@ typedef struct ae_attn_bwd_params {
   const int8_t* mask_dq;   /* mask mode 2: tile classes [mask_b,mask_h,ceil(Sq/128),ceil(Skv/64)], else NULL */
   const int8_t* mask_dkv;  /* mask mode 2: tile classes [mask_b,mask_h,ceil(Sq/64),ceil(Skv/128)], else NULL */
   const void* custom[AE_MAX_CUSTOM]; /* scalar CustomIO tensors (fp32 [1]) of score_mod, in dict order   */
+  /* kernels compiled with AE_EXT_BLOCK_MASK 1 (the forward ran on a block mask the user supplied, the
+   * reference's blockattn_tl.py:195-470): that mask, int8 [mask_b,mask_h,mask_nq,mask_nkv] with blocks of
+   * mask_block_m x mask_block_n positions (0 = invisible); tiles of class 1 in the two tables above test
+   * their elements against it.  NULL otherwise. */
+  const int8_t* block_mask;
+  /* kernels compiled with AE_BWD_KIND 2 and AE_BWD_NRS > 1 (an online function that hands more than one final
+   * row scale to its traced forward() / backward(), the reference's core/lower/lower.py:413-453): row scales
+   * 1 .. AE_BWD_NRS - 1, fp32 [B,Hq,Sq] each; `lse` carries row scale 0 and `delta` has 1 + AE_BWD_NRS planes.
+   * NULL otherwise. */
+  const float* more_rowscales[AE_MAX_ROWSCALES - 1];
   int64_t q_stride_b, q_stride_s, q_stride_h;
   int64_t k_stride_b, k_stride_s, k_stride_h;
   int64_t v_stride_b, v_stride_s, v_stride_h;
@@ -169,7 +180,8 @@ typedef struct ae_attn_bwd_params {
   int64_t dk_stride_b, dk_stride_s, dk_stride_h;
   int64_t dv_stride_b, dv_stride_s, dv_stride_h;
   int32_t batch, heads_q, heads_kv, seqlen_q, seqlen_kv;
-  int32_t mask_b, mask_h;  /* batch / head extents of the two tables: 1 or (B, Hq) */
+  int32_t mask_b, mask_h;  /* batch / head extents of the two tables (and of block_mask): 1 or (B, Hq) */
+  int32_t mask_nq, mask_nkv, mask_block_m, mask_block_n;  /* geometry of block_mask (0 without one)   */
   int32_t reserved[1];
 } ae_attn_bwd_params;
 

@@ -44,8 +44,8 @@ def test_struct_layout_matches_the_header():
     # 4 + 4 + 4 + 1 + 2 + 2 pointers, 18 strides, 13 + 3 ints, then the paged-cache part: 2 pointers, 3 + 1 ints
     assert ctypes.sizeof(rt.AttnParams) == 8 * 17 + 8 * 18 + 4 * 16 + 8 * 2 + 4 * 4
     assert ctypes.sizeof(rt.TileCfg) == 4 * 12
-    # backward: 12 + 4 pointers, 8 tensors x 3 strides, 7 + 1 ints
-    assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 16 + 8 * 24 + 4 * 8
+    # backward: 12 + 4 + 1 + 3 pointers, 8 tensors x 3 strides, 7 + 4 + 1 ints
+    assert ctypes.sizeof(rt.AttnBwdParams) == 8 * 20 + 8 * 24 + 4 * 12
     lines = ['#include "ae_hip.h"']
     n_fields = 0
     for cname, mirror in (("ae_attn_params", rt.AttnParams), ("ae_tile_cfg", rt.TileCfg),
@@ -387,8 +387,10 @@ def test_benchmarked_kernels_do_not_spill_registers():
 @pytest.mark.parametrize("causal", [True, False])
 def test_prefill_kernels_keep_their_arrays_in_registers(dtype, D, causal):
     """The pipelined and the generic kernel of the softmax prefill, both input types: no scratch memory beyond a few
-    spilled values.  (A lambda of a kernel that the inliner leaves as a function keeps the arrays it captures by reference
-    in scratch memory: the larger bf16 builds of the pipelined kernel once ran 30 times slower for it.)"""
+    spilled single values (some bf16 builds of the pipelined kernel at head dim 128), and never a register tuple in
+    scratch memory -- the form of spill that once returned wrong columns (hip_rt.check_spills refuses it).  (A lambda
+    of a kernel that the inliner leaves as a function keeps the arrays it captures by reference in scratch memory:
+    the larger bf16 builds of the pipelined kernel once ran 30 times slower for it.)"""
     import attn_cases as C
     from core import CustomIO, meta_tensor
     from core.lower.prefill_op import PrefillOp
@@ -401,6 +403,143 @@ def test_prefill_kernels_keep_their_arrays_in_registers(dtype, D, causal):
         for key, (module, _, _) in op._variants.items():
             for kname, k in module.kernel_info().items():
                 assert k[".private_segment_fixed_size"] <= 64, (t, key, kname, k[".private_segment_fixed_size"])
+            assert module.scratch_accesses()["wide"] == 0, (t, key)
+            if dtype == torch.float16:
+                assert module.scratch_accesses() == {"single": 0, "wide": 0}, (t, key)
+
+
+def test_a_kernel_that_spills_registers_is_refused():
+    """hip_rt.check_spills: a code object that keeps vector registers in scratch memory is refused after
+    compilation when the caller is strict about it (``allow_spills=False``, ``strict_spills``, AE_ALLOW_SPILLS=0) and
+    reported with a warning otherwise; ``allow_spills=True`` / AE_ALLOW_SPILLS=1 switch the check off.  The kernel here
+    is register-hungry on purpose: 600 values live across a barrier under a launch bound that leaves a wave 128
+    registers."""
+    src_dir = rt.KERNEL_DIR
+    name = "_x_spill_guard_probe.hip"                      # (git-ignored name pattern of scratch kernels)
+    path = os.path.join(src_dir, name)
+    body = """
+#ifndef __HIPCC_RTC__
+#include <hip/hip_runtime.h>
+#endif
+#include "ae_config.h"
+extern "C" __global__ __launch_bounds__(1024) void ae_hungry_kernel(float* p) {
+  float x[AE_LIVE];
+#pragma unroll
+  for (int i = 0; i < AE_LIVE; i++) x[i] = p[threadIdx.x + 1024 * i];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < AE_LIVE; i++) p[threadIdx.x + 1024 * ((i * 7) % AE_LIVE)] += x[i] * x[(i * 13) % AE_LIVE];
+}
+"""
+    with open(path, "w") as f:
+        f.write(body)
+
+    def small_spill(name):
+        """A build that spills, however little (found by raising the number of live values)."""
+        for live in (130, 140, 160, 200, 260):
+            m = rt.compile_module(name, {"ae_config.h": f"#define AE_LIVE {live}\n"}, use_cache=False, allow_spills=True)
+            if m.kernel_info()["ae_hungry_kernel"][".vgpr_spill_count"] > 0:
+                return m
+        pytest.skip("no spilling build found")
+    try:
+        small = rt.compile_module(name, {"ae_config.h": "#define AE_LIVE 8\n"}, use_cache=False)
+        assert small.kernel_info()["ae_hungry_kernel"][".vgpr_spill_count"] == 0
+        big = {"ae_config.h": "#define AE_LIVE 600\n"}
+        with pytest.raises(rt.SpillError, match="spills vector registers") as e:
+            rt.compile_module(name, big, use_cache=False, allow_spills=False)
+        assert "ae_hungry_kernel" in str(e.value) and "allow_spills=True" in str(e.value)
+        assert isinstance(e.value, rt.AEError)
+        with pytest.raises(rt.SpillError):                       # the family of builds the operators mark
+            rt.compile_module(name, big, use_cache=False, strict_spills=True)
+        with pytest.warns(RuntimeWarning, match="spills vector registers"):     # the default: reported, not refused
+            m = rt.compile_module(name, big, use_cache=False)
+        assert m.kernel_info()["ae_hungry_kernel"][".vgpr_spill_count"] > 0 and m.scratch_accesses()["single"] > 0
+        import warnings
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            rt.check_spills(m, name, allow_spills=True)
+            os.environ["AE_ALLOW_SPILLS"] = "1"
+            try:
+                rt.check_spills(m, name)
+            finally:
+                os.environ["AE_ALLOW_SPILLS"] = "0"
+            try:
+                with pytest.raises(rt.SpillError):
+                    rt.check_spills(m, name)
+                with pytest.raises(rt.SpillError):               # ... and with it any spill at all
+                    rt.check_spills(small_spill(name), name)
+            finally:
+                del os.environ["AE_ALLOW_SPILLS"]
+    finally:
+        os.remove(path)
+        rt._modules.clear()
+
+
+def test_a_prefill_engine_gives_way_to_the_generic_kernel_rather_than_spill(monkeypatch):
+    """A build of the software-pipelined kernel that the spill guard refuses (``allow_spills=False``): where that
+    kernel was the engine's own choice the engine compiles the generic kernel instead and says so; asked for explicitly
+    (``tiles=``, as the tuner does) the refused build is an error, which the tuner passes over.  The case: bf16, head
+    dim 128, causal -- a build that spills seven single values, which the guard accepts as it stands and objects to
+    here because the test sets its limit on scratch bytes to zero."""
+    import attn_cases as C
+    from attn_engine import AttentionEngine
+    from core import CustomIO, meta_tensor
+    from core.lower import lower as L
+    from core.lower.prefill_op import PrefillOp
+    dtype = torch.bfloat16
+    meta = (meta_tensor(2, 32, 4096, 128, dtype=dtype),) * 3
+    args = (meta, CustomIO({}), C.make_scale_score_mod(128 ** -0.5), C.causal_mask, C.OnlineSoftmax())
+    assert L.choose_prefill_tiles(128, 128, 4096, (0.1, "m", "r"), 64).template == "ae_prefill_pipe.hip"
+    accepted = AttentionEngine(*args)
+    assert accepted._op.tiles.template == "ae_prefill_pipe.hip"
+    (module, _, _), = accepted._op._variants.values()
+    acc = module.scratch_accesses()
+    assert acc["wide"] == 0 and 0 < acc["single"] < 40
+    monkeypatch.setattr(rt, "MAX_SCRATCH_BYTES", 0)
+    rt._modules.clear()
+    mod = AttentionEngine(*args, allow_spills=False)
+    assert mod._op.tiles.template == "ae_prefill.hip" and mod._op.gave_way_to_generic
+    assert "#define AE_WAVES_PER_EU 2" in mod.tl_code
+    pipe = L.PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)
+    with pytest.raises(rt.SpillError, match="spills heavily"):
+        PrefillOp(*args, "-inf", tiles=pipe, allow_spills=False)
+    with pytest.warns(RuntimeWarning, match="spills heavily"):       # the default: reported, and the kernel stays
+        assert AttentionEngine(*args)._op.tiles.template == "ae_prefill_pipe.hip"
+    forced = AttentionEngine(*args, allow_spills=True)
+    assert forced._op.tiles.template == "ae_prefill_pipe.hip"
+    # fp16 fits the registers: nothing gives way
+    f16 = AttentionEngine((meta_tensor(2, 32, 4096, 128, dtype=torch.float16),) * 3, *args[1:])
+    assert f16._op.tiles.template == "ae_prefill_pipe.hip" and not getattr(f16._op, "gave_way_to_generic", False)
+    rt._modules.clear()
+
+
+def test_wide_value_head_builds_are_compiled_strictly(monkeypatch):
+    """The configuration whose compiled code once returned a wrong pair of output columns (head dim 256, value head
+    dim 512, sliding window, ragged tiles: a 16-register accumulator tuple went through scratch memory and came back
+    with a stale register) does not spill as the kernel stands, and PrefillOp compiles that family of builds -- one
+    launch over more than 256 value columns -- with the spill check set to refuse: a compiler that spills a tuple
+    there again is an error, not a warning."""
+    import attn_cases as C
+    from core import CustomIO, meta_tensor
+    from core.lower.prefill_op import PrefillOp
+    seen = []
+    real = rt.compile_module
+
+    def spy(template, headers, *a, **kw):
+        seen.append((template, kw.get("strict_spills", False)))
+        return real(template, headers, *a, **kw)
+    monkeypatch.setattr(rt, "compile_module", spy)
+    S, D, DV, dt = 100, 256, 512, torch.float16
+    meta = (meta_tensor(1, 1, S, D, dtype=dt), meta_tensor(1, 1, S, D, dtype=dt), meta_tensor(1, 1, S, DV, dtype=dt))
+    op = PrefillOp(meta, CustomIO({}), C.make_scale_score_mod(D ** -0.5), C.make_sliding_window_mask(70),
+                   C.OnlineSoftmax(), "-inf")
+    (module, _, _), = op._variants.values()
+    assert module.kernel_info()["ae_prefill_kernel"][".vgpr_spill_count"] == 0
+    assert op.DV_launch == 512 and seen == [("ae_prefill.hip", True)]
+    seen.clear()
+    meta = (meta_tensor(1, 1, S, 128, dtype=dt),) * 3
+    PrefillOp(meta, CustomIO({}), C.make_scale_score_mod(128 ** -0.5), C.causal_mask, C.OnlineSoftmax(), "-inf")
+    assert seen and all(not strict for _, strict in seen)
 
 
 @pytest.mark.parametrize("mask", [None, "causal", "window"])

@@ -622,3 +622,25 @@ def test_numerics_keywords_of_the_constructor(monkeypatch):
     monkeypatch.setenv("AE_DEFER_NORM", "0")
     assert AttentionEngine(*args, mask_value="0").attention.functors.deferred_norm is None
     assert AttentionEngine(*args, mask_value="0", defer_norm=True).attention.functors.deferred_norm == "r"
+
+
+def test_tile_classes_of_a_user_block_mask():
+    """PrefillBwdOp.block_mask_tile_classes (the tables the backward launches read when the forward ran on a block
+    mask the user supplied) against brute force over the expanded mask, for block sizes below, equal to and above
+    the tile sizes and sequence lengths that are not multiples of either."""
+    from core.lower.prefill_bwd_op import PrefillBwdOp
+    g = torch.Generator().manual_seed(2)
+    for bm, bn, Sq, Skv in ((128, 128, 1024, 1024), (32, 64, 640, 576), (64, 128, 448, 450), (256, 32, 700, 333),
+                            (48, 96, 500, 400)):
+        nq, nk = -(-Sq // bm), -(-Skv // bn)
+        blocks = (torch.rand(2, 3, nq, nk, generator=g) < 0.5).to(torch.int8)
+        dense = blocks.bool().repeat_interleave(bm, 2).repeat_interleave(bn, 3)[:, :, :Sq, :Skv]
+        for tm, tn in ((128, 64), (256, 64), (64, 128)):
+            got = PrefillBwdOp.block_mask_tile_classes(blocks, bm, bn, Sq, Skv, tm, tn)
+            assert got.shape == (2, 3, -(-Sq // tm), -(-Skv // tn)) and got.dtype == torch.int8
+            for i in range(got.shape[2]):
+                for j in range(got.shape[3]):
+                    t = dense[:, :, i * tm:(i + 1) * tm, j * tn:(j + 1) * tn]
+                    some, every = t.any(-1).any(-1), t.all(-1).all(-1)
+                    want = some.to(torch.int8) + (some & every).to(torch.int8)
+                    assert torch.equal(got[:, :, i, j], want), (bm, bn, Sq, Skv, tm, tn, i, j)

@@ -17,6 +17,31 @@ from oracle import masks as M
 pytestmark = pytest.mark.gpu
 
 
+class OnlineSoftmaxTwoScales(C.OnlineSoftmax):
+    """The online softmax of attn_script/mha.py with its reference point and its row sum exported as TWO final row
+    scales (instead of their combination lse), and the recompute / backward rules written against both, in the
+    protocol of the reference (attn_engine/attn_engine.py:75-93; every final row scale is handed to forward() and
+    backward(), core/lower/lower.py:413-453).  The lowering cannot take it for the softmax it has a fixed backward
+    for, so both rules are traced; the function it computes is still softmax attention."""
+
+    def __init__(self):
+        super().__init__()
+        from core import SymbolScalar, Var
+        self.final_rowscales = {"m": SymbolScalar("m", Var("0.0")), "r": SymbolScalar("r", Var("0.0"))}
+
+    @staticmethod
+    def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+        return o / online_rowscales["r"], {"m": online_rowscales["m"], "r": online_rowscales["r"]}
+
+    @staticmethod
+    def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+        return (scores - final_rowscales["m"]).exp() / final_rowscales["r"]
+
+    @staticmethod
+    def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+        return scores * (dp - doosum_rowscales)
+
+
 def _engine(B, H, Hkv, S, D, DV, dtype, mask_mod, scale):
     meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
             meta_tensor(B, Hkv, S, DV, dtype=dtype))
@@ -200,6 +225,142 @@ def test_retention_backward(cuda_device, B, H, Hkv, S, D, DV, dtype):
     out.backward(do.cuda())
     dq, dk, dv = R.retention_attention_grads(q, k, v, mask, do)
     case = (B, H, Hkv, S, D, DV, dtype)
+    _check(qd.grad, dq, "dq", case)
+    _check(kd.grad, dk, "dk", case)
+    _check(vd.grad, dv, "dv", case)
+
+
+@pytest.mark.parametrize("bm,bn,S,Hkv,dtype", [
+    (128, 128, 1024, 3, torch.float16),    # attn_script/blocksparseattn.py's granularity: every backward tile lies in ONE block
+    (128, 64, 512, 3, torch.float16),      # the geometry of the reference's tests/test_blockmask.py
+    (32, 64, 640, 1, torch.bfloat16),      # finer than the backward's 64- and 128-row tiles: tiles straddle blocks of both
+                                           # kinds and test every element against the mask; grouped heads
+    (64, 128, 448, 3, torch.float16),      # ragged last tiles of both launches (448 = 3.5 x 128)
+])
+def test_backward_with_an_external_block_mask(cuda_device, bm, bn, S, Hkv, dtype):
+    """attn_script/blocksparseattn.py with gradients (the reference's block-sparse backward,
+    blockattn_tl.py:195-470): the user's int8 block mask [B,H,S/bm,S/bn] reaches the two backward launches as
+    tile-class tables made from it on the GPU, and tiles that straddle visible and invisible blocks look every
+    element up in the mask itself.  Against the oracle's gradients under the expanded dense mask; one q block
+    row sees nothing at all (out 0, gradients 0)."""
+    print(f"case bwd extern block mask {bm}x{bn} S{S} Hkv{Hkv} {dtype}", flush=True)
+    B, H, D = 2, 3, 64
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator().manual_seed(11)
+    nq, nk = -(-S // bm), -(-S // bn)
+    blocks = torch.rand(B, H, nq, nk, generator=g) < 0.45
+    blocks[..., 0] = True                         # every row sees something ...
+    blocks[0, 1, nq - 1] = False                  # ... except one block row of one head
+    q, k, v = C.make_inputs(B, S, S, H, Hkv, D, D, dtype, seed=5)
+    do = torch.randn(B, S, H, D, generator=g).to(dtype)
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+            meta_tensor(B, Hkv, S, D, dtype=dtype))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(scale), mask_mod=None,
+                          online_func=C.OnlineSoftmax(), infer_mask=True, extern_block_mask=True,
+                          infer_mask_block_M=bm, infer_mask_block_N=bn)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = mod(qd, kd, vd, block_mask=blocks.to(torch.int8).cuda())
+    out.backward(do.cuda())
+    dense = blocks.repeat_interleave(bm, 2).repeat_interleave(bn, 3)[:, :, :S, :S]
+    ref_out, _ = R.softmax_attention(q, k, v, scale=scale, mask=dense)
+    assert (out.detach().float().cpu() - ref_out).abs().max().item() <= 2e-2
+    dq, dk, dv = R.softmax_attention_grads(q, k, v, do, scale=scale, mask=dense)
+    case = (bm, bn, S, Hkv, dtype)
+    _check(qd.grad, dq, "dq", case)
+    _check(kd.grad, dk, "dk", case)
+    _check(vd.grad, dv, "dv", case)
+    r0 = (nq - 1) * bm
+    assert qd.grad[0, r0:, 1].abs().max().item() == 0.0          # the rows that see nothing
+    # a second call with another mask: the tables follow the mask of the call
+    blocks2 = torch.ones_like(blocks)
+    qd.grad = kd.grad = vd.grad = None
+    mod(qd, kd, vd, block_mask=blocks2.to(torch.int8).cuda()).backward(do.cuda())
+    dq, dk, dv = R.softmax_attention_grads(q, k, v, do, scale=scale)
+    _check(qd.grad, dq, "dq", case + ("all",))
+    _check(kd.grad, dk, "dk", case + ("all",))
+
+
+@pytest.mark.parametrize("mask_name", ["causal", "window", "plus_one", "head_dependent"])
+def test_backward_masks_are_bit_exact(cuda_device, mask_name):
+    """One-hot probes of the masks the two backward launches apply (tiles skipped by index or by their tile-class
+    tables, elements tested where a tile is partly visible), at 4300 positions -- more than 64 streamed items per
+    resident tile, so the tables are read in several chunks of ballots, ragged last tiles in both launches -- and
+    two q heads per kv head.  Integers, compared exactly:
+      * dk / dv launch: the graph out = sum_kv f(s) v with f = 1 on every finite score and 0 on a masked one;
+        dO holds one-hot rows (q -> column q mod DV), so dv[kv, j] = dO^T p counts the queries of residue class j
+        that see key kv (summed over the group's q heads);
+      * dq launch: f(s) = s, so ds = dp on visible scores and 0 on masked ones; with v and dO all equal to the
+        first unit vector dp = 1, and K one-hot rows make dq[q, j] = ds K count the visible keys of class j."""
+    mask_mod = {"causal": C.causal_mask, "window": C.make_sliding_window_mask(100),
+                "plus_one": C.causal_plus_one_mask, "head_dependent": C.head_dependent_mask}[mask_name]
+    B, H, Hkv, S, D = 1, 2, 1, 4300, 64
+    dtype = torch.float16
+    print(f"case bwd mask probe {mask_name}", flush=True)
+    dense = torch.from_numpy(M.dense_mask_grid(mask_mod, B, H, S, S)).float()        # [B,H,S,S]
+    onehot = torch.zeros(S, D)
+    onehot[torch.arange(S), torch.arange(S) % D] = 1.0
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+            meta_tensor(B, Hkv, S, D, dtype=dtype))
+
+    def ones_score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+        return ((score * 0.001 + 50.0).tanh() + 1.0) * 0.5
+
+    def plain_score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+        return score * 1.0
+
+    q, k, v = C.make_inputs(B, S, S, H, Hkv, D, D, dtype)
+    # dk / dv launch
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=ones_score_mod, mask_mod=mask_mod, online_func=C.OnlineIdentity())
+    bwd = mod._op.backward_op()
+    assert bwd.kind == 1
+    do = onehot.to(dtype).view(1, S, 1, D).expand(B, S, H, D).contiguous()
+    out = torch.zeros(B, S, H, D, dtype=dtype)
+    _, _, dv = bwd(q.cuda(), k.cuda(), v.cuda(), out.cuda(), None, do.cuda())
+    expect = torch.einsum("bhqk,qd->bkd", dense, onehot).view(B, S, Hkv, D)
+    assert expect.max().item() >= {"causal": 100, "plus_one": 100, "window": 4, "head_dependent": 5}[mask_name]
+    assert torch.equal(dv.float().cpu(), expect), mask_name
+    # dq launch
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=plain_score_mod, mask_mod=mask_mod, online_func=C.OnlineIdentity())
+    bwd = mod._op.backward_op()
+    e0 = torch.zeros(D, dtype=dtype)
+    e0[0] = 1.0
+    kk = onehot.to(dtype).view(1, S, 1, D).expand(B, S, Hkv, D).contiguous()
+    vv = e0.view(1, 1, 1, D).expand(B, S, Hkv, D).contiguous()
+    do = e0.view(1, 1, 1, D).expand(B, S, H, D).contiguous()
+    dq, _, _ = bwd(q.cuda(), kk.cuda(), vv.cuda(), out.cuda(), None, do.cuda())
+    expect = torch.einsum("bhqk,kd->bqhd", dense, onehot)
+    assert torch.equal(dq.float().cpu(), expect), mask_name
+
+
+@pytest.mark.parametrize("B,H,Hkv,S,D,dtype,causal", [
+    (1, 2, 2, 256, 64, torch.float16, False),
+    (2, 4, 2, 333, 128, torch.bfloat16, True),      # grouped heads, ragged tiles, causal
+    (1, 3, 1, 200, 64, torch.float16, True),
+])
+def test_traced_backward_with_two_final_row_scales(cuda_device, B, H, Hkv, S, D, dtype, causal):
+    """An online function with TWO final row scales whose forward() / backward() rules read both: the rules are
+    traced (no fixed gradient applies), the backward launches carry both row scales per q row, and since the
+    function is softmax attention written differently its gradients must be those of the oracle
+    (softmax_attention_grads, pinned by float64 autograd).  The exported scales themselves: m + log r = lse."""
+    print(f"case two row scales B{B} H{H} Hkv{Hkv} S{S} D{D} {dtype} causal={causal}", flush=True)
+    scale = 1 / math.sqrt(D)
+    q, k, v = C.make_inputs(B, S, S, H, Hkv, D, D, dtype, seed=13)
+    do = torch.randn(B, S, H, D, generator=torch.Generator().manual_seed(113)).to(dtype)
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, Hkv, S, D, dtype=dtype),
+            meta_tensor(B, Hkv, S, D, dtype=dtype))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(scale),
+                          mask_mod=C.causal_mask if causal else None, online_func=OnlineSoftmaxTwoScales())
+    bwd = mod._op.backward_op()
+    assert bwd.kind == 2 and bwd.rowscale_names == ["m", "r"] and bwd.n_rs == 2
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = mod(qd, kd, vd)
+    out.backward(do.cuda())
+    ref_out, lse = R.softmax_attention(q, k, v, scale=scale, causal=causal)
+    assert (out.detach().float().cpu() - ref_out).abs().max().item() <= 2e-2
+    m, r = mod.final_rowscales["m"].cpu(), mod.final_rowscales["r"].cpu()
+    assert (m + r.log() - lse).abs().max().item() <= 1e-3
+    dq, dk, dv = R.softmax_attention_grads(q, k, v, do, scale=scale, causal=causal)
+    case = (B, H, Hkv, S, D, dtype, causal)
     _check(qd.grad, dq, "dq", case)
     _check(kd.grad, dk, "dk", case)
     _check(vd.grad, dv, "dv", case)

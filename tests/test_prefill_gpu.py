@@ -265,6 +265,44 @@ def test_mask_is_bit_exact(cuda_device):
         assert torch.equal(out, expect), mask_mod.__name__
 
 
+def _ones_score_mod(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+    """Every finite score -> exactly 1, a masked (-inf) score -> exactly 0 (tanh saturates)."""
+    return ((score * 0.001 + 50.0).tanh() + 1.0) * 0.5
+
+
+def _one_hot_rows(S, D, dtype):
+    """[S, D]: row i is the unit vector of column i mod D."""
+    x = torch.zeros(S, D, dtype=dtype)
+    x[torch.arange(S), torch.arange(S) % D] = 1.0
+    return x
+
+
+@pytest.mark.parametrize("mask_name", ["causal", "window", "plus_one", "head_dependent"])
+def test_mask_is_bit_exact_in_the_pipelined_kernel(cuda_device, monkeypatch, mask_name):
+    """The one-hot probe of test_mask_is_bit_exact where the headline kernel runs: the software-pipelined kernel
+    (here with the generated functor of an elementwise graph), 4700 keys -- more than 64 kv tiles, so the tile
+    classes are read in two chunks of ballots, and a ragged last q tile of 256 rows -- under the analytic causal
+    mask with its per-wave cut-off at the diagonal, and under three masks that reach the kernel as a tile-class
+    table.  out[q, j] counts the visible keys of residue class j: integers, compared exactly."""
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    mask_mod = {"causal": C.causal_mask, "window": C.make_sliding_window_mask(100),
+                "plus_one": C.causal_plus_one_mask, "head_dependent": C.head_dependent_mask}[mask_name]
+    B, H, S, D = 1, 2, 4700, 64
+    dtype = torch.float16
+    print(f"case pipelined mask probe {mask_name}", flush=True)
+    q, k, _ = C.make_inputs(B, S, S, H, H, D, D, dtype)
+    onehot = _one_hot_rows(S, D, dtype)
+    v = onehot.view(1, S, 1, D).expand(B, S, H, D).contiguous()
+    mod = _engine(B, H, S, D, D, dtype, _ones_score_mod, mask_mod, C.OnlineIdentity())
+    assert mod._op.tiles.template == "ae_prefill_pipe.hip" and "#define AE_PIPE_KIND 1" in mod.tl_code
+    assert ("#define AE_MASK_MODE 1" in mod.tl_code) == (mask_name == "causal")
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    dense = _dense(mask_mod, B, H, S, S).float()                  # [B,H,S,S]
+    expect = torch.einsum("bhqk,kd->bqhd", dense, onehot.float())
+    assert expect.max().item() >= {"causal": 60, "plus_one": 60, "window": 2, "head_dependent": 3}[mask_name]
+    assert torch.equal(out, expect), mask_name
+
+
 @pytest.mark.parametrize("kernel,bm,bn,S", [
     ("generic", 128, 128, 1024),       # attn_script/blocksparseattn.py: blocks of 128 x 128
     ("pipelined", 128, 128, 1024),     # two table rows per 256-row q tile
@@ -310,6 +348,70 @@ def test_score_mod_with_indices(cuda_device):
     s = s.masked_fill(~torch.ones(S, S, dtype=torch.bool).tril(), float("-inf"))
     ref = torch.einsum("bhqk,bkhd->bqhd", torch.softmax(s, -1), v.float())
     assert (out - ref).abs().max().item() <= OUT_TOL
+
+
+@pytest.mark.parametrize("kernel", ["generic", "simple"])
+def test_rows_without_a_visible_key_inside_a_visited_tile(cuda_device, kernel):
+    """``q_idx - 100 >= kv_idx``: rows 0..99 see no key at all, rows 100..127 of the same q tile do, so the tile
+    is visited and the first hundred rows meet nothing but masked scores.  They end like the rows of a q tile
+    without any tile: out = 0 and lse = -inf (the convention of the reference's CuTe kernels, flash_fwd_kernel.h:
+    180-183; its TileLang scripts guard the division with r + 1e-30, attn_script/sparseattn.py:68) -- not the
+    0 / 0 the softmax epilogue makes of an empty row.  Also under a user block mask finer than the q tile."""
+    def late_mask(b, h, q_idx, kv_idx):
+        return q_idx - 100 >= kv_idx
+    B, H, S, dtype = 1, 2, 384, torch.float16
+    D, DV = (128, 128) if kernel == "generic" else (96, 160)     # (96 / 160: head dims of the register-staged kernel)
+    print(f"case empty rows {kernel} D{D} DV{DV}", flush=True)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, DV, dtype)
+    mod = _engine(B, H, S, D, DV, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), late_mask, C.OnlineSoftmax())
+    assert mod._op.tiles.template == ("ae_prefill.hip" if kernel == "generic" else "ae_prefill_simple.hip")
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    lse = mod.final_rowscales["lse"].cpu()
+    ref, lref = R.softmax_attention(q, k, v, mask=_dense(late_mask, B, H, S, S))
+    assert torch.isfinite(out).all()
+    assert out[:, :100].abs().max().item() == 0.0 and torch.isinf(lse[:, :, :100]).all() and (lse[:, :, :100] < 0).all()
+    assert (out[:, 100:] - ref[:, 100:]).abs().max().item() <= OUT_TOL
+    assert (lse[:, :, 100:] - lref[:, :, 100:]).abs().max().item() <= LSE_TOL
+    if kernel == "generic":
+        blocks = torch.ones(B, H, S // 32, S // 64, dtype=torch.bool)
+        blocks[0, 1, 5] = False                      # rows 160..191 of head 1: inside the q tile 128..255
+        mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), None, C.OnlineSoftmax(),
+                      infer_mask=True, extern_block_mask=True, infer_mask_block_M=32, infer_mask_block_N=64)
+        out = mod(q.cuda(), k.cuda(), v.cuda(), block_mask=blocks.to(torch.int8).cuda()).float().cpu()
+        lse = mod.final_rowscales["lse"].cpu()
+        dense = blocks.repeat_interleave(32, 2).repeat_interleave(64, 3)
+        ref, lref = R.softmax_attention(q, k, v, mask=dense)
+        assert torch.isfinite(out).all()
+        assert out[0, 160:192, 1].abs().max().item() == 0.0 and (lse[0, 1, 160:192] == float("-inf")).all()
+        keep = torch.ones(B, S, H, dtype=torch.bool)
+        keep[0, 160:192, 1] = False
+        assert (out - ref)[keep].abs().max().item() <= OUT_TOL
+        assert (lse - lref).permute(0, 2, 1)[keep].abs().max().item() <= LSE_TOL
+
+
+def test_dynamic_extents(cuda_device, tmp_path):
+    """attn_script/mha.py:90-95 declares its shapes with names, ``meta_tensor("batch", H, "seq_len", D)`` (the
+    reference turns them into symbolic extents, core/lower/lower.py:627-629): one engine then serves any batch
+    size and sequence length.  Here the extents are runtime parameters of the kernels anyway; the engine is
+    built without a shape, compiles what a call needs at that call, and is checked against the oracle at three
+    shapes, with the tuner's record looked up under the reference's defaults for dynamic dims
+    (attn_tl.py:465-472)."""
+    H, D, dtype = 4, 128, torch.float16
+    meta = (meta_tensor("batch", H, "seq_len", D, dtype=dtype),) * 3
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)),
+                          mask_mod=C.causal_mask, online_func=C.OnlineSoftmax(), tune=True,
+                          tune_file=str(tmp_path / "tuned.json"))
+    assert mod._op.meta_shape[2] == 0                     # nothing was compiled for a declared shape
+    for B, S in ((2, 512), (1, 1000), (3, 77)):
+        print(f"case dynamic extents B{B} S{S}", flush=True)
+        q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=B)
+        out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+        ref, lse = R.softmax_attention(q, k, v, causal=True)
+        assert (out - ref).abs().max().item() <= OUT_TOL
+        assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+    import json
+    (rec,) = json.load(open(tmp_path / "tuned.json"))
+    assert (rec["batch"], rec["heads"], rec["seq_len"], rec["dim"]) == (4, H, 2048, D)
 
 
 def test_gqa_prefill(cuda_device):
