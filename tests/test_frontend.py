@@ -398,14 +398,43 @@ def test_traced_backward_of_an_online_function_with_its_own_row_scale():
     derivative of score_mod (the decay mask, read per score); an online function that keeps row scales
     without defining them gets no backward."""
     from core.lower.prefill_bwd_op import lower_traced_backward
-    src, name = lower_traced_backward(C.retention_score_mod, C.OnlineRetention(), C.retention_custom_inputs(),
-                                      torch.float16)
-    assert name == "r" and "ae_bwd_pd2" in src
+    src, names = lower_traced_backward(C.retention_score_mod, C.OnlineRetention(), C.retention_custom_inputs(),
+                                       torch.float16)
+    assert names == ["r"] and "ae_bwd_pd2" in src
     assert "p.custom[0]" in src and "p.seqlen_kv" in src          # the mask element of (head, q, kv)
     body = src.split("ae_bwd_pd2", 2)[-1]
-    assert "rs0" in body and "cv_mask" in body and "dp" in body
+    assert "const float (&rs)[1]" in body and "rs[0]" in body and "cv_mask" in body and "dp" in body
     with pytest.raises(NotImplementedError, match="forward"):
         lower_traced_backward(C.retention_score_mod, C.OnlineAbsNorm(), C.retention_custom_inputs(), torch.float16)
+
+
+def test_traced_backward_reads_every_final_row_scale():
+    """An online function with two final row scales whose forward() / backward() read both (the reference hands
+    every final row scale to them, core/lower/lower.py:413-453): both arrive in the functor, in declaration order."""
+    from core.lower.prefill_bwd_op import lower_traced_backward
+
+    class TwoScales(C.OnlineSoftmax):
+        def __init__(self):
+            super().__init__()
+            self.final_rowscales = {"m": SymbolScalar("m", Var("0.0")), "r": SymbolScalar("r", Var("0.0"))}
+
+        @staticmethod
+        def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+            return o / online_rowscales["r"], {"m": online_rowscales["m"], "r": online_rowscales["r"]}
+
+        @staticmethod
+        def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+            return (scores - final_rowscales["m"]).exp() / final_rowscales["r"]
+
+        @staticmethod
+        def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+            return scores * (dp - doosum_rowscales)
+    src, names = lower_traced_backward(C.make_scale_score_mod(0.125), TwoScales(), CustomIO({}), torch.float16)
+    assert names == ["m", "r"]
+    body = src.split("ae_bwd_pd2", 2)[-1]
+    assert "const float (&rs)[2]" in body and "rs[0]" in body and "rs[1]" in body and "doosum" in body
+    lf = L.trace_functors(C.make_scale_score_mod(0.125), None, TwoScales(), CustomIO({}), torch.float16)
+    assert lf.softmax is None and lf.final_rowscale_names == ["m", "r"]     # not the graph with the fixed backward
 
 
 def test_symbol_backward_leaves_gradient_expressions_on_the_leaves():
