@@ -588,13 +588,14 @@ class PrefillTiles:
     k_pad: int = 0
     v_pad: int = 0
     rows_per_wave: int = 32
+    kv_stages: int = 2                 # K / V tile stages in LDS (AE_KV_STAGES of the pipelined kernel: 2 or 3)
 
     @property
     def block_m(self):
         return self.rows_per_wave * self.n_waves
 
     def lds_bytes(self, d: int, dv: int) -> int:
-        stages = 2 * self.block_n * ((2 * d + self.k_pad) + (2 * dv + self.v_pad))
+        stages = self.kv_stages * self.block_n * ((2 * d + self.k_pad) + (2 * dv + self.v_pad))
         if self.template == "ae_prefill_pipe.hip":
             # behind the tile stages every wave has room for its 64 Q rows (later its 64 O rows), which travel
             # through LDS as whole rows (AE_QO_BYTES of the kernel)
@@ -618,6 +619,19 @@ def direct_tile_ok(d: int, dv: int, block_n: int, n_waves: int = 4) -> bool:
     a wave and tile (one burst of direct loads)."""
     nt = 64 * n_waves
     return all((block_n * x // 8) % nt == 0 and (block_n * x // 8) // nt <= 8 for x in (d, dv))
+
+
+PIPE_KV_STAGES = 2      # default number of K / V stages of the pipelined kernel (AE_PIPE_STAGES=2|3 overrides)
+
+
+def pipelined_tiles(d: int, dv: int) -> PrefillTiles:
+    """The software-pipelined kernel's tile configuration: 256-row q tiles, one wave per SIMD, and as many K / V
+    stages as asked for while they fit the 160 KiB of LDS beside the waves' Q / O rows."""
+    stages = int(os.environ.get("AE_PIPE_STAGES", "") or PIPE_KV_STAGES)
+    t = PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64, kv_stages=stages)
+    if stages != 2 and t.lds_bytes(d, dv) > 160 * 1024:
+        t.kv_stages = 2
+    return t
 
 
 def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch_heads: int = 0,
@@ -655,7 +669,7 @@ def choose_prefill_tiles(d: int, dv: int, seqlen_q: int = 0, softmax=None, batch
             fits = False
         if d in (64, 128) and (softmax is not None or elementwise) and force != "generic" and (
                 force == "pipelined" or (fits and n_tiles >= (3 * _MI355X_CUS) // 4)):
-            return PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64)
+            return pipelined_tiles(d, dv)
         return PrefillTiles()
     t = PrefillTiles(template="ae_prefill_simple.hip", k_pad=16)
     if max(d, dv) > 128:
@@ -712,6 +726,10 @@ def render_config(d: int, dv: int, dtype, tiles: PrefillTiles, mask_mode: int, h
         f"#define AE_WAVES_PER_EU {tiles.waves_per_eu}",
         f"#define AE_K_PAD {tiles.k_pad}",
         f"#define AE_V_PAD {tiles.v_pad}",
+        *([f"#define AE_KV_STAGES {tiles.kv_stages}"] if tiles.template == "ae_prefill_pipe.hip" else []),
+        # (measurement switch of the pipelined kernel: the order of a causal launch's workgroups)
+        *([f"#define AE_CAUSAL_ORDER {os.environ['AE_CAUSAL_ORDER']}"]
+          if tiles.template == "ae_prefill_pipe.hip" and os.environ.get("AE_CAUSAL_ORDER", "") in ("0", "1") else []),
         *extra,
         "",
     ])

@@ -102,7 +102,7 @@ def prefill_candidates(d, dv, softmax, elementwise):
     if d in L.DIRECT_D and dv in L.DIRECT_DV:
         c = []
         if d in (64, 128) and dv in (64, 128) and (softmax is not None or elementwise):
-            c.append(L.PrefillTiles(template="ae_prefill_pipe.hip", waves_per_eu=1, rows_per_wave=64))
+            c.append(L.pipelined_tiles(d, dv))
         # two waves per SIMD while a wave may fit 256 registers (Q fragments of up to 192 columns, 128 value columns)
         shapes = [(2, 64), (2, 32), (1, 64)] if d <= 192 and dv <= 128 else [(1, 64), (1, 32)]
         if d > 128 and dv <= 128:
@@ -121,7 +121,7 @@ def prefill_candidates(d, dv, softmax, elementwise):
 
 
 def encode_tiles(t):
-    return [t.block_m, t.block_n, 2, 64 * t.n_waves, t.waves_per_eu, t.template]
+    return [t.block_m, t.block_n, t.kv_stages, 64 * t.n_waves, t.waves_per_eu, t.template]
 
 
 def decode_tiles(tuned_config, candidates):

@@ -76,6 +76,23 @@
 #ifndef AE_EXP_SPAN
 #define AE_EXP_SPAN (2 * AE_NKF + 8)   // MFMA slots over which the 32 exponentiation units of a tile start
 #endif
+// K / V tile stages in LDS.  2: a tile is requested in the iteration before the one that multiplies it and waited
+// for (vmcnt(0)) at that iteration's end, i.e. it has about three quarters of an iteration to arrive.  3: it is
+// requested one iteration earlier still, and an iteration ends by waiting only until its OWN requests are the
+// ones outstanding - the tile it waits for has had a whole further iteration.
+#ifndef AE_KV_STAGES
+#define AE_KV_STAGES 2
+#endif
+// order of a causal launch's workgroups: 0 = heaviest q tile first across ALL heads (longest job first),
+// 1 = head by head (see below)
+#ifndef AE_CAUSAL_ORDER
+#define AE_CAUSAL_ORDER 0
+#endif
+static_assert(AE_KV_STAGES == 2 || AE_KV_STAGES == 3, "two or three K / V stages");
+// s_waitcnt with vmcnt(n) and the other counters left alone (vmcnt is six bits wide: 3:0 and 15:14)
+#define AE_VMCNT(n) (0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+// tile loads a wave may leave in flight across the end of an iteration: its own requests of that iteration
+#define AE_INFLIGHT (AE_KV_STAGES == 3 ? AE_K_LOADS + AE_V_LOADS : 0)
 #ifndef AE_KLOAD_SLOT
 #define AE_KLOAD_SLOT 7            // phase-1 MFMA slots after which the K and the V tile loads go out
 #define AE_VLOAD_SLOT (AE_NKF + 7)
@@ -122,7 +139,7 @@ struct ae_tag_false { static constexpr bool value = false; };
 extern "C" __global__ __launch_bounds__(AE_NT) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void ae_prefill_kernel(const ae_attn_params p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char ae_smem[];
-  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // [2][K tile], [2][V tile], then AE_QO_BYTES per wave (its Q rows, later its O rows)
+  ae_lds_byte* lds = (ae_lds_byte*)ae_smem;   // [AE_KV_STAGES][K tile], [AE_KV_STAGES][V tile], then AE_QO_BYTES per wave (its Q rows, later its O rows)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -147,8 +164,16 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // late q tiles are the long ones (AE_HEAVY_LAST, found on the host: causal variants, long sliding windows)
   // takes the same order: B2 H32 S4096, "kv <= q + 1": 0.40 -> 0.35 ms.
   const int n_bg = (n_bh + 7) >> 3;
+#if AE_CAUSAL_ORDER == 0
   const int qt = n_qt - 1 - slot / n_bg;
   const int bh = (slot % n_bg) * 8 + xcd;
+#else
+  // (measurement switch) head by head: the q tiles of one (batch, head) are adjacent in time, heaviest first, so
+  // that its K / V stay in the XCD's L2 while they are used - at the price of a longer tail
+  const int qt = n_qt - 1 - slot % n_qt;
+  const int bh = (slot / n_qt) * 8 + xcd;
+  (void)n_bg;
+#endif
 #else
   const int qt = slot % n_qt;
   const int bh = (slot / n_qt) * 8 + xcd;
@@ -178,7 +203,7 @@ void ae_prefill_kernel(const ae_attn_params p) {
   // until the first tile could be multiplied), swizzled like a K tile, into a region of the wave's own behind
   // the tile stages; the fragments are read from there once the first tiles have landed too.
   ae_elem8 qf[2][AE_NKS];
-  ae_lds_byte* qo = lds + 2 * AE_K_BYTES + 2 * AE_V_BYTES + wave * AE_QO_BYTES;
+  ae_lds_byte* qo = lds + AE_KV_STAGES * (AE_K_BYTES + AE_V_BYTES) + wave * AE_QO_BYTES;
   {
     const int q0c = q0w < p.seqlen_q ? q0w : p.seqlen_q - 1;
     const char* qg = (const char*)((const ae_elem*)p.q + (int64_t)b * p.q_stride_b + (int64_t)q0c * p.q_stride_s +
@@ -307,24 +332,35 @@ void ae_prefill_kernel(const ae_attn_params p) {
       gp[i] = off;
     }
     ae_load_lds16_burst_base<AE_V_LOADS>(
-        g, gp, lds + 2 * AE_K_BYTES + stage * AE_V_BYTES + (wave * AE_V_LOADS + AE_V_LOADS / 2) * 1024);
+        g, gp, lds + AE_KV_STAGES * AE_K_BYTES + stage * AE_V_BYTES + (wave * AE_V_LOADS + AE_V_LOADS / 2) * 1024);
   };
 
   // ---- the first tiles are requested before anything else is set up: the zeroing of the accumulators, the
   // constants and the address arithmetic below (about a thousand instructions of one wave per SIMD) then run
   // while they and the Q rows travel ----
   int j0 = next_tile(0);                  // tile whose scores are in sv (exp + PV next)
-  int tc0[2], tc1[2], tc2[2];             // ... and what tiles j0, j1, j2 mean to this wave (tile_info)
-  bool tnm0, tnm1, tnm2 = false;
+  int tc0[2], tc1[2], tc2[2], tcn[2];     // ... and what tiles j0, j1, j2, jn mean to this wave (tile_info)
+  bool tnm0, tnm1, tnm2 = false, tnmn = false;
   tile_info(j0, tc0, tnm0);
-  tc2[0] = tc2[1] = 2;
+  tc2[0] = tc2[1] = tcn[0] = tcn[1] = 2;
   const bool any_tile = j0 < j_end;
   int j1 = any_tile ? next_tile(j0 + 1) : j_end;   // tile multiplied by Q next
   tile_info(j1, tc1, tnm1);
+#if AE_KV_STAGES == 3
+  int j2 = j1 < j_end ? next_tile(j1 + 1) : j_end;  // with three stages the tile after it is on its way as well
+  tile_info(j2, tc2, tnm2);
+#endif
   if (any_tile) {
     load_k(j0, 0);
     load_v(j0, 0);
+#if AE_KV_STAGES == 2
     if (j1 < j_end) load_k(j1, 1);
+#else
+    // (tiles past the end: the last tile again, so that every wave's requests can be counted)
+    load_k(j1 < j_end ? j1 : j_end - 1, 1);
+    load_v(j1 < j_end ? j1 : j_end - 1, 1);
+    load_k(j2 < j_end ? j2 : j_end - 1, 2);
+#endif
   }
 
   // ---- state ------------------------------------------------------------------------------
@@ -571,7 +607,9 @@ void ae_prefill_kernel(const ae_attn_params p) {
   };
 
   // ---- prologue: first tile's scores ------------------------------------------------------------
-  __builtin_amdgcn_s_waitcnt(0);
+  // (three stages: V of the second tile and K of the third, requested last, may still be travelling)
+  if (AE_KV_STAGES == 3 && any_tile) __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_INFLIGHT) & 0xF0FF);   // ... and lgkmcnt(0)
+  else __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 #pragma unroll
   for (int qb = 0; qb < 2; qb++)
@@ -613,17 +651,19 @@ void ae_prefill_kernel(const ae_attn_params p) {
   __syncthreads();                         // everyone is done with K stage 0 before it is refilled
 
   // ---- main loop ----------------------------------------------------------------------------------
-  // iteration n: loads K(n+2) -> K stage n%2, V(n+1) -> V stage (n+1)%2;
+  // iteration n (two stages): loads K(n+2) -> K stage n%2, V(n+1) -> V stage (n+1)%2;
   //              phase 1 multiplies K(n+1) (K stage (n+1)%2), phase 2 multiplies V(n) (V stage n%2).
+  // With three stages the loads are K(n+3) -> K stage n%3 and V(n+2) -> V stage (n+2)%3.
   int n = 0;
+  int sg = 0;     // n % AE_KV_STAGES: the stage of V(j0); K(j1) sits in the next one
   // first AE_AHEAD fragments of iteration n's stream: K(j1) if it has a next tile, else V(j0)
   auto prefetch_ring = [&]() AE_LAMBDA {
     if (j1 < j_end) {
-      const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
+      const ae_lds_byte* kt = lds + (sg + 1 == AE_KV_STAGES ? 0 : sg + 1) * AE_K_BYTES;
 #pragma unroll
       for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_kfrag(f, kt);
     } else {
-      const ae_lds_byte* vt = lds + 2 * AE_K_BYTES + (n & 1) * AE_V_BYTES;
+      const ae_lds_byte* vt = lds + AE_KV_STAGES * AE_K_BYTES + sg * AE_V_BYTES;
 #pragma unroll
       for (int f = 0; f < AE_AHEAD; f++) ring[f] = read_vfrag(f, vt);
     }
@@ -636,18 +676,26 @@ void ae_prefill_kernel(const ae_attn_params p) {
   auto iteration = [&](auto has_next_tag, auto tail_loads_tag) AE_LAMBDA {
     constexpr bool HN = decltype(has_next_tag)::value;
     constexpr bool TL = decltype(tail_loads_tag)::value;
-    const ae_lds_byte* kt = lds + ((n + 1) & 1) * AE_K_BYTES;
-    const ae_lds_byte* vt = lds + 2 * AE_K_BYTES + (n & 1) * AE_V_BYTES;
-    const int j2 = (HN || TL) ? next_tile(j1 + 1) : j_end;
-    tile_info(j2, tc2, tnm2);
-    // Nothing is in flight here on the back edge (the iteration ends with vmcnt(0)); saying so
-    // also clears loads still pending on loop ENTRY (Q fragments, spill reloads), which the
+    const int sg1 = sg + 1 == AE_KV_STAGES ? 0 : sg + 1;              // stage of K(j1), V(j1)
+    const int sgv = AE_KV_STAGES == 2 ? sg1 : (sg1 + 1 == 3 ? 0 : sg1 + 1);   // stage of the V tile requested now
+    const ae_lds_byte* kt = lds + sg1 * AE_K_BYTES;
+    const ae_lds_byte* vt = lds + AE_KV_STAGES * AE_K_BYTES + sg * AE_V_BYTES;
+#if AE_KV_STAGES == 2
+    const int jlast = j1;
+#else
+    const int jlast = j2;
+#endif
+    const int jn = (HN || TL) ? next_tile(jlast + 1) : j_end;        // the tile whose K is requested now
+    tile_info(jn, tcn, tnmn);
+    // Only this wave's requests of the previous iteration (none with two stages) are in flight here on the back
+    // edge; saying so also clears loads still pending on loop ENTRY (Q fragments, spill reloads), which the
     // compiler's wait-count insertion would otherwise wait for after this iteration's tile loads
     // have been issued, i.e. with a vmcnt(0) that serialises them.
-    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);
-    // The tile loads of this iteration, K(j2) and V(j1), are issued as two bursts from phase-1 slots
-    // below.  When there is no tile j2 the K stage is refilled with the last tile, which nobody reads.
-    const int j2l = j2 < j_end ? j2 : j_end - 1;
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_INFLIGHT));
+    // The tile loads of this iteration, K(jn) and V(jlast), are issued as two bursts from phase-1 slots
+    // below.  When there is no such tile the stage is refilled with the last tile, which nobody reads.
+    const int j2l = jn < j_end ? jn : j_end - 1;
+    const int jvl = jlast < j_end ? jlast : j_end - 1;
     // fragment stream of this iteration: K fragments 0..NKF-1 (if HN) then V fragments
     constexpr int NF1 = HN ? AE_NKF : 0;
     constexpr int NF = NF1 + AE_NVF;
@@ -673,15 +721,15 @@ void ae_prefill_kernel(const ae_attn_params p) {
         for (int qb = 0; qb < 2; qb++) {
           sacc[f & 1][qb] = ae_mfma32(ring[f % AE_RING], qf[qb][f >> 1], f < 2 ? AE_C0(qb) : sacc[f & 1][qb]);
           exp_slot(2 * f + qb);
-          if (2 * f + qb == AE_KLOAD_SLOT) load_k(j2l, n & 1);
-          if (2 * f + qb == AE_VLOAD_SLOT) load_v(j1, (n + 1) & 1);
+          if (2 * f + qb == AE_KLOAD_SLOT) load_k(j2l, sg);
+          if (2 * f + qb == AE_VLOAD_SLOT) load_v(jvl, sgv);
           AE_SB();
         }
       }
     } else {
       if (TL) {
-        load_k(j2l, n & 1);
-        load_v(j1, (n + 1) & 1);
+        load_k(j2l, sg);
+        load_v(jvl, sgv);
       }
       exp_all();
     }
@@ -708,13 +756,22 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #if !AE_TOP_PREFETCH
     if (HN) finish_scores(j1, tc1, tnm1);
 #endif
-    // tiles for the next iteration must have landed, and everyone must be done with this one's
-    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);   // vmcnt(0)
+    // tiles for the next iteration must have landed (with three stages they were requested an iteration ago: only
+    // this iteration's own requests may still travel), and everyone must be done with this one's
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT((HN || TL) ? AE_INFLIGHT : 0));
     __syncthreads();
     j0 = j1;
-    j1 = j2;
     tc0[0] = tc1[0], tc0[1] = tc1[1], tnm0 = tnm1;
+#if AE_KV_STAGES == 2
+    j1 = jn;
+    tc1[0] = tcn[0], tc1[1] = tcn[1], tnm1 = tnmn;
+#else
+    j1 = j2;
     tc1[0] = tc2[0], tc1[1] = tc2[1], tnm1 = tnm2;
+    j2 = jn;
+    tc2[0] = tcn[0], tc2[1] = tcn[1], tnm2 = tnmn;
+#endif
+    sg = sg1;
     n++;
 #if AE_TOP_PREFETCH
     if (HN) {
@@ -749,14 +806,26 @@ void ae_prefill_kernel(const ae_attn_params p) {
 #if AE_MASK_MODE == 1
   // an iteration of a wave that is done with its own tiles: its share of the tile loads, and the barrier
   auto drain = [&]() AE_LAMBDA {
-    const int j2 = next_tile(j1 + 1);
-    const int j2l = j2 < j_end ? j2 : j_end - 1;
-    load_k(j2l, n & 1);
-    load_v(j1, (n + 1) & 1);
-    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);   // vmcnt(0)
+    const int sg1 = sg + 1 == AE_KV_STAGES ? 0 : sg + 1;
+    const int sgv = AE_KV_STAGES == 2 ? sg1 : (sg1 + 1 == 3 ? 0 : sg1 + 1);
+#if AE_KV_STAGES == 2
+    const int jlast = j1;
+#else
+    const int jlast = j2;
+#endif
+    const int jn = next_tile(jlast + 1);
+    load_k(jn < j_end ? jn : j_end - 1, sg);
+    load_v(jlast < j_end ? jlast : j_end - 1, sgv);
+    __builtin_amdgcn_s_waitcnt(AE_VMCNT(AE_INFLIGHT));
     __syncthreads();
     j0 = j1;
+#if AE_KV_STAGES == 2
+    j1 = jn;
+#else
     j1 = j2;
+    j2 = jn;
+#endif
+    sg = sg1;
     n++;      // (a wave that only requests tiles no longer looks at their classes)
   };
   if (any_tile) {

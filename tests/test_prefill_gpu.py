@@ -529,6 +529,27 @@ def test_retention_with_decay_mask_input(cuda_device, monkeypatch, B, H, S, D, D
     assert (out - ref).abs().max().item() <= OUT_TOL
 
 
+@pytest.mark.parametrize("D,dtype,causal", [(128, torch.float16, True), (128, torch.float16, False),
+                                            (64, torch.bfloat16, True)])
+def test_pipelined_kernel_with_three_tile_stages(cuda_device, monkeypatch, D, dtype, causal):
+    """AE_PIPE_STAGES=3: the pipelined kernel with a third K / V stage in LDS (tiles requested an iteration
+    earlier, the end of an iteration waits only until its own requests are the ones outstanding).  It measures
+    the same as two stages on the benchmark shapes and is not the default; this keeps it correct: ragged
+    sequence, several q tiles per head, against the oracle."""
+    monkeypatch.setenv("AE_PREFILL_KERNEL", "pipelined")
+    monkeypatch.setenv("AE_PIPE_STAGES", "3")
+    B, H, S = 2, 3, 1100
+    print(f"case three stages D{D} {dtype} causal={causal}", flush=True)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=17)
+    mod = _engine(B, H, S, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.causal_mask if causal else None,
+                  C.OnlineSoftmax())
+    assert mod._op.tiles.template == "ae_prefill_pipe.hip" and "#define AE_KV_STAGES 3" in mod.tl_code
+    out = mod(q.cuda(), k.cuda(), v.cuda()).float().cpu()
+    ref, lse = R.softmax_attention(q, k, v, causal=causal)
+    assert (out - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
 def test_retention_scores_beyond_the_fp16_range(cuda_device, monkeypatch):
     """Scores of 65504 and more, fp16: the script's per-tile form ``scores / r_new`` keeps the operand of the
     second product at |X / r| <= 1 and stays finite -- ``defer_norm=False`` builds exactly that and matches the
