@@ -295,7 +295,8 @@ def mfma_probe(cfg=None, launches=20, iters=250):
     """The matrix-pipe ceiling of this chip, measured: ae_mfma_probe_kernel (32x32x16 MFMAs back to back, with
     the other work ``cfg`` asks for between them) on all-zero and on N(0,1) operands -- the same code object, so
     the difference is the chip's power management reacting to the operand data.  Returns {operands: {tflops,
-    clock_mhz, cycles_per_mfma}}; clock from the kernel's own s_memtime / s_memrealtime stamps."""
+    clock_mhz, cycles_per_mfma}}; clock from the kernel's own s_memtime / s_memrealtime stamps, cycles_per_mfma =
+    the cycles of that clock one SIMD spent per MFMA over the launch (32 when the matrix pipe never idles)."""
     import ctypes
     import torch
     from core.runtime import hip_rt as rt
@@ -335,9 +336,10 @@ def mfma_probe(cfg=None, launches=20, iters=250):
         e1.record(stream)
         ms = e0.elapsed_ms(e1) / launches
         flop = grid * 4.0 * waves_per_simd * iters * 32 * 32768.0
-        st = stamps.cpu().double()
-        out[name] = {"tflops": flop / (ms * 1e-3) / 1e12, "ms": ms, "clock_mhz": _clock_mhz(stamps),
-                     "cycles_per_mfma": float(st[:, 0].mean() / (iters * 32.0 * waves_per_simd))}
+        tflops, clock = flop / (ms * 1e-3) / 1e12, _clock_mhz(stamps)
+        # cycles one SIMD spends per MFMA over the whole launch: 32768 flop per MFMA, 1024 SIMDs
+        out[name] = {"tflops": tflops, "ms": ms, "clock_mhz": clock,
+                     "cycles_per_mfma": 32768.0 * 1024 * clock * 1e6 / (tflops * 1e12)}
     return out
 
 
@@ -349,7 +351,7 @@ def mfma_probe_report(steps, warmup):
     lines = ["# matrix-pipe ceiling probe (ae_mfma_probe_kernel: 32x32x16 MFMAs back to back, alone or with the named other work "
              "between them) and the clock the attention kernels run at",
              "# columns: case, operands, TFLOP/s, shader clock MHz (s_memtime / s_memrealtime inside the kernel), "
-             "cycles per MFMA and wave, share of 2500 TFLOP/s"]
+             "SIMD cycles per MFMA, share of 2500 TFLOP/s"]
     rec = {}
     for tag, cfg in PROBE_CASES:
         r = mfma_probe(cfg)
