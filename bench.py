@@ -291,7 +291,7 @@ def probe_config_text(cfg):
     return "// configuration of ae_mfma_probe.hip\n" + "".join(f"#define {k} {v}\n" for k, v in sorted(cfg.items()))
 
 
-def mfma_probe(cfg=None, launches=20, iters=250):
+def mfma_probe(cfg=None, launches=20, iters=250, operands=("zeros", "randn")):
     """The matrix-pipe ceiling of this chip, measured: ae_mfma_probe_kernel (32x32x16 MFMAs back to back, with
     the other work ``cfg`` asks for between them) on all-zero and on N(0,1) operands -- the same code object, so
     the difference is the chip's power management reacting to the operand data.  Returns {operands: {tflops,
@@ -318,6 +318,8 @@ def mfma_probe(cfg=None, launches=20, iters=250):
     stream = torch.cuda.current_stream(dev).cuda_stream
     out = {}
     for name, pool in pools.items():
+        if name not in operands:
+            continue
         stamps = torch.zeros((grid, 2), dtype=torch.int64, device=dev)
         prm = ProbeParams(pool.data_ptr(), sink.data_ptr(), stamps.data_ptr(), n_src, iters)
         threads = 256 * waves_per_simd
@@ -459,6 +461,10 @@ def main():
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of the benchmark line: measure the matrix-pipe ceiling (a pure MFMA loop on zero and "
                          "on N(0,1) operands) and the shader clock the prefill / MLA kernels run at")
+    ap.add_argument("--probe-case", type=int, default=None, metavar="I",
+                    help="with --mfma-probe: only case I of PROBE_CASES, on --probe-operands, --steps launches of ~1 ms "
+                         "back to back (a steady load to read socket power and clocks against, e.g. with amd-smi metric -p)")
+    ap.add_argument("--probe-operands", default="randn", choices=["zeros", "randn"])
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain 256 MiB copy kernel (ae_copy_probe_kernel) so that a "
                          "hardware-counter run can scale FETCH_SIZE / WRITE_SIZE by a known transfer")
@@ -474,6 +480,11 @@ def main():
         sys.exit(3)
     from core.runtime import hip_rt as rt
     info = rt.device_info(0)
+    if a.mfma_probe and a.probe_case is not None:
+        tag, cfg = PROBE_CASES[a.probe_case]
+        r = mfma_probe(cfg, launches=a.steps, operands=(a.probe_operands,))[a.probe_operands]
+        print(json.dumps({"mfma_probe_case": tag, "operands": a.probe_operands, "launches": a.steps, **r}), flush=True)
+        return
     if a.mfma_probe:
         mfma_probe_report(a.steps, a.warmup)
         return
