@@ -11,8 +11,12 @@
 // and constant-rate ticks (s_memrealtime, 100 MHz).  Their ratio is the shader clock during the loop.
 //
 // Configuration ("ae_config.h", may be empty):
-//   AE_PROBE_WAVES_PER_SIMD  1 or 2 waves per SIMD
+//   AE_PROBE_WAVES_PER_SIMD  1 or 2 waves per SIMD (one: the accumulators sit in the accumulator file; two: each wave has
+//                            256 registers and the compiler picks the form of the MFMA whose accumulators are ordinary
+//                            registers -- the rates of the two forms do not differ)
 //   AE_PROBE_BF16            1: bf16 operands (the pool is read as bf16), else fp16
+//   AE_PROBE_M16             1: the 16x16x32 shape, two MFMAs where the other builds have one 32x32x16 (same flops,
+//                            half the accumulator registers read and written per flop, twice the operand registers)
 //   AE_PROBE_EXTRA_VALU      independent v_fma_f32 per MFMA, issued between the MFMAs (0: the pure ceiling)
 //   AE_PROBE_EXP             v_exp_f32 per MFMA, likewise
 //   AE_PROBE_LDS             1: every second MFMA takes a fresh A fragment (1 KiB per wave) from LDS, read two
@@ -42,6 +46,10 @@
 #ifndef AE_PROBE_BF16
 #define AE_PROBE_BF16 0
 #endif
+#ifndef AE_PROBE_M16
+#define AE_PROBE_M16 0
+#endif
+#define AE_PROBE_NACC 8   // accumulator tuples the MFMAs rotate over
 
 #if AE_PROBE_BF16
 typedef __bf16 ae_probe_elem;
@@ -59,10 +67,27 @@ struct ae_mfma_probe_params {
   int iters;                      // loop trips; one trip = 32 MFMAs per wave
 };
 
-__device__ inline ae_probe_f32x16 ae_probe_mfma(ae_probe_half8 a, ae_probe_half8 b, ae_probe_f32x16 c) {
+__device__ __attribute__((always_inline)) inline ae_probe_f32x16 ae_probe_mfma(const int QP, ae_probe_half8 a, ae_probe_half8 b, ae_probe_half8 b2,
+                                                                              ae_probe_f32x16 c) {
+#if AE_PROBE_M16
+  // two 16x16x32 MFMAs on registers 8 QP .. 8 QP + 7 of the accumulator tuple
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  f32x4 lo = {c[8 * QP], c[8 * QP + 1], c[8 * QP + 2], c[8 * QP + 3]}, hi = {c[8 * QP + 4], c[8 * QP + 5], c[8 * QP + 6], c[8 * QP + 7]};
 #if AE_PROBE_BF16
+  lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, lo, 0, 0, 0);
+  hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, hi, 0, 0, 0);
+#else
+  lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, lo, 0, 0, 0);
+  hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b2, hi, 0, 0, 0);
+#endif
+#pragma unroll
+  for (int i = 0; i < 4; i++) c[8 * QP + i] = lo[i], c[8 * QP + 4 + i] = hi[i];
+  return c;
+#elif AE_PROBE_BF16
+  (void)QP, (void)b2;
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 #else
+  (void)QP, (void)b2;
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
 #endif
 }
@@ -89,11 +114,12 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   for (int f = 0; f < 16; f++)
     mine[f * 64] = *(const ae_probe_half8*)(src + ((base + 4096 + f * 520) & (p.n_src - 8)));
 #endif
-  ae_probe_f32x16 c[8];
+  ae_probe_f32x16 c[AE_PROBE_NACC];
 #pragma unroll
-  for (int i = 0; i < 8; i++)
+  for (int i = 0; i < AE_PROBE_NACC; i++) {
 #pragma unroll
     for (int r = 0; r < 16; r++) c[i][r] = 0.f;
+  }
 #if AE_PROBE_EXTRA_VALU || AE_PROBE_EXP
   float x[8];
 #pragma unroll
@@ -111,9 +137,9 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
 #if AE_PROBE_LDS
       // fragment for the MFMAs j + 4, j + 5 (a[] is a ring of four: one in use, two on their way)
       if ((j & 1) == 0) a[((j >> 1) + 2) & 3] = mine[((j >> 1) & 15) * 64];
-      c[j & 7] = ae_probe_mfma(a[(j >> 1) & 3], b[j & 3], c[j & 7]);
+      c[j % AE_PROBE_NACC] = ae_probe_mfma((j / AE_PROBE_NACC) & 1, a[(j >> 1) & 3], b[j & 3], b[(j + 1) & 3], c[j % AE_PROBE_NACC]);
 #else
-      c[j & 7] = ae_probe_mfma(a[j & 3], b[(j >> 2) & 3], c[j & 7]);
+      c[j % AE_PROBE_NACC] = ae_probe_mfma((j / AE_PROBE_NACC) & 1, a[j & 3], b[(j >> 2) & 3], b[((j >> 2) + 1) & 3], c[j % AE_PROBE_NACC]);
 #endif
 #if AE_PROBE_EXTRA_VALU
 #pragma unroll
@@ -138,7 +164,7 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   }
   float acc = 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; i++) acc += c[i][tid & 15];
+  for (int i = 0; i < AE_PROBE_NACC; i++) acc += c[i][tid & 15];
 #if AE_PROBE_EXTRA_VALU || AE_PROBE_EXP
 #pragma unroll
   for (int i = 0; i < 8; i++) acc += x[i];

@@ -284,6 +284,12 @@ PROBE_CASES = [
      {"AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_WAVES_PER_SIMD": 2}),
     ("bf16 flash-attention mix per MFMA, 1 wave/SIMD",
      {"AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_BF16": 1}),
+    ("fp16 MFMA only, 16x16x32 shape (two per 32x32x16), 1 wave/SIMD", {"AE_PROBE_M16": 1}),
+    ("fp16 MFMA only, 16x16x32 shape, 2 waves/SIMD", {"AE_PROBE_M16": 1, "AE_PROBE_WAVES_PER_SIMD": 2}),
+    ("fp16 flash-attention mix per two 16x16x32 MFMAs, 1 wave/SIMD",
+     {"AE_PROBE_M16": 1, "AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1}),
+    ("fp16 flash-attention mix per two 16x16x32 MFMAs, 2 waves/SIMD",
+     {"AE_PROBE_M16": 1, "AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_WAVES_PER_SIMD": 2}),
 ]
 
 
