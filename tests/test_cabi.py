@@ -68,8 +68,9 @@ def test_struct_layout_matches_the_header():
 
 
 def test_the_binding_sketch_in_the_integration_notes_matches_the_header():
-    """INTEGRATION.md shows the ctypes structures a maintainer of the reference would copy.  They are executed
-    here as written (the two class statements only) and must have the size of ae_attn_params / ae_tile_cfg,
+    """The integration notes at the repository root show the ctypes structures a maintainer of the reference would
+    copy.  They are executed here as written (the two class statements only) and must have the size of
+    ae_attn_params / ae_tile_cfg,
     with every field the ctypes mirror of the library also has at the same offset; a sketch that is one ABI
     behind hands the launch functions a short struct."""
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
