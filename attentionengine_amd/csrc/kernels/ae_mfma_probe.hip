@@ -20,7 +20,14 @@
 //   AE_PROBE_EXTRA_VALU      independent v_fma_f32 per MFMA, issued between the MFMAs (0: the pure ceiling)
 //   AE_PROBE_EXP             v_exp_f32 per MFMA, likewise
 //   AE_PROBE_LDS             1: every second MFMA takes a fresh A fragment (1 KiB per wave) from LDS, read two
-//                            fragments ahead - the LDS traffic of a kernel whose every fragment feeds two MFMAs
+//                            fragments ahead - the LDS traffic of a kernel whose every fragment feeds two MFMAs;
+//                            2: every 32768 flop take one (a wave of 32 rows: a fragment feeds one 32x32x16 or two 16x16x32)
+//   AE_PROBE_SKELETON        1 (with AE_PROBE_EXP 1, AE_PROBE_LDS 1): what a kernel's loop cannot avoid on top of the mix --
+//                            the exponentials take MFMA RESULTS (read out of the accumulators) and their packed
+//                            results become B operands of later MFMAs, each accumulator starts from zero every trip
+//                            (chains of four MFMAs, values stay bounded), and every trip (32 MFMAs) each wave requests
+//                            4 KiB of the pool straight into LDS, waits for it and meets the workgroup's barrier: the
+//                            tile traffic of a 256-row q tile with 64-key tiles at head dim 128
 // A flash attention forward at head dim 128 spends one 32x32x16 MFMA per 64 scores, i.e. per score and lane:
 // one exponential, a maximum, a sum and half a packed conversion at the very least, and half a fragment read.
 // AE_PROBE_EXTRA_VALU 2 + AE_PROBE_EXP 1 (an exponential and the v_fma that consumes it) + AE_PROBE_LDS 1 is that
@@ -48,6 +55,9 @@
 #endif
 #ifndef AE_PROBE_M16
 #define AE_PROBE_M16 0
+#endif
+#ifndef AE_PROBE_SKELETON
+#define AE_PROBE_SKELETON 0
 #endif
 #define AE_PROBE_NACC 8   // accumulator tuples the MFMAs rotate over
 
@@ -107,7 +117,7 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   }
 #if AE_PROBE_LDS
   // 16 fragments of pool data per wave in LDS (16 KiB a wave), lane-contiguous 16-byte pieces: conflict-free reads
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[4 * AE_PROBE_WAVES_PER_SIMD * 16 * 1024];
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[4 * AE_PROBE_WAVES_PER_SIMD * (16 + 4 * AE_PROBE_SKELETON) * 1024];
   typedef __attribute__((address_space(3))) ae_probe_half8 lds_frag;
   lds_frag* mine = (lds_frag*)((__attribute__((address_space(3))) unsigned char*)lds_raw) + (tid >> 6) * 16 * 64 + (tid & 63);
 #pragma unroll
@@ -132,12 +142,38 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
   const unsigned long long t0 = __builtin_amdgcn_s_memtime();
   const unsigned long long w0 = __builtin_amdgcn_s_memrealtime();
   for (int it = 0; it < p.iters; it++) {
+#if AE_PROBE_SKELETON
+    {
+      // this trip's "tile": four direct loads of 1 KiB per wave behind one write of M0, into the wave's staging area
+      // behind the fragments (the data are never read: the fragments above stand for them)
+      const unsigned m0v = __builtin_amdgcn_readfirstlane(
+          (unsigned)(unsigned long)((__attribute__((address_space(3))) unsigned char*)lds_raw) +
+          4u * AE_PROBE_WAVES_PER_SIMD * 16u * 1024u + (tid >> 6) * 4096u);
+      const char* gsrc = (const char*)src + (((blockIdx.x * 4099u + (unsigned)it * 64u + tid) * 16u) & (p.n_src * 2u - 4096u - 16u));
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                   "global_load_lds_dwordx4 %0, off\n\tglobal_load_lds_dwordx4 %0, off offset:1024\n\t"
+                   "global_load_lds_dwordx4 %0, off offset:2048\n\tglobal_load_lds_dwordx4 %0, off offset:3072"
+                   : : "v"(gsrc), "s"(m0v) : "memory");
+    }
+#endif
 #pragma unroll
     for (int j = 0; j < 32; j++) {
+#if AE_PROBE_SKELETON
+      if (j < AE_PROBE_NACC) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) c[j][r] = 0.f;      // (folds into the MFMA's C operand)
+      }
+#endif
 #if AE_PROBE_LDS
+#if AE_PROBE_LDS == 2
+      // a fresh fragment for every slot, read two slots ahead (a[] is a ring of four)
+      a[(j + 2) & 3] = mine[(j & 15) * 64];
+      c[j % AE_PROBE_NACC] = ae_probe_mfma((j / AE_PROBE_NACC) & 1, a[j & 3], b[j & 3], b[(j + 1) & 3], c[j % AE_PROBE_NACC]);
+#else
       // fragment for the MFMAs j + 4, j + 5 (a[] is a ring of four: one in use, two on their way)
       if ((j & 1) == 0) a[((j >> 1) + 2) & 3] = mine[((j >> 1) & 15) * 64];
       c[j % AE_PROBE_NACC] = ae_probe_mfma((j / AE_PROBE_NACC) & 1, a[(j >> 1) & 3], b[j & 3], b[(j + 1) & 3], c[j % AE_PROBE_NACC]);
+#endif
 #else
       c[j % AE_PROBE_NACC] = ae_probe_mfma((j / AE_PROBE_NACC) & 1, a[j & 3], b[(j >> 2) & 3], b[((j >> 2) + 1) & 3], c[j % AE_PROBE_NACC]);
 #endif
@@ -146,7 +182,14 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
       for (int e = 0; e < AE_PROBE_EXTRA_VALU; e++)
         x[(j + e) & 7] = __builtin_fmaf(x[(j + e) & 7], 0.999f, 0.001f);
 #endif
-#if AE_PROBE_EXP
+#if AE_PROBE_EXP && AE_PROBE_SKELETON
+      {
+        // a result of the MFMA issued four slots ago -> exponent -> packed into a B operand used four slots on
+        const float sres = c[(j + 4) % AE_PROBE_NACC][j & 15];
+        const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sres, 0.125f, -4.0f));
+        b[(j + 2) & 3][j & 7] = (ae_probe_elem)pe;
+      }
+#elif AE_PROBE_EXP
 #pragma unroll
       for (int e = 0; e < AE_PROBE_EXP; e++)
         x[(j + 4 + e) & 7] = __builtin_amdgcn_exp2f(x[(j + 4 + e) & 7]) * 0.5f - 0.75f;   // stays in (-0.75, 0.1)
@@ -155,6 +198,10 @@ void ae_mfma_probe_kernel(const ae_mfma_probe_params p) {
       __builtin_amdgcn_sched_barrier(0);      // keep the other work between the MFMAs, where a kernel has it
 #endif
     }
+#if AE_PROBE_SKELETON
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0f00);      // vmcnt(0): the tile has landed
+    __syncthreads();
+#endif
   }
   const unsigned long long t1 = __builtin_amdgcn_s_memtime();
   const unsigned long long w1 = __builtin_amdgcn_s_memrealtime();

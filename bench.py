@@ -290,6 +290,14 @@ PROBE_CASES = [
      {"AE_PROBE_M16": 1, "AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1}),
     ("fp16 flash-attention mix per two 16x16x32 MFMAs, 2 waves/SIMD",
      {"AE_PROBE_M16": 1, "AE_PROBE_EXTRA_VALU": 2, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_WAVES_PER_SIMD": 2}),
+    ("fp16 loop skeleton: the mix on MFMA results, their exponentials as operands, tile loads and a barrier per 32 MFMAs, "
+     "1 wave/SIMD",
+     {"AE_PROBE_EXTRA_VALU": 1, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 1, "AE_PROBE_SKELETON": 1}),
+    ("fp16 loop skeleton, 2 waves/SIMD of half the rows (a fragment read per MFMA)",
+     {"AE_PROBE_EXTRA_VALU": 1, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 2, "AE_PROBE_SKELETON": 1, "AE_PROBE_WAVES_PER_SIMD": 2}),
+    ("fp16 loop skeleton on 16x16x32 MFMAs, 2 waves/SIMD of half the rows (a fragment read per pair)",
+     {"AE_PROBE_EXTRA_VALU": 1, "AE_PROBE_EXP": 1, "AE_PROBE_LDS": 2, "AE_PROBE_SKELETON": 1, "AE_PROBE_WAVES_PER_SIMD": 2,
+      "AE_PROBE_M16": 1}),
 ]
 
 
