@@ -235,7 +235,7 @@ def find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale
         o_scale = exp(m - m_new)
         scores' = exp(S - m_new)
         r_new = r * o_scale + rowsum(scores')
-        epilogue: o / r  and  lse = log(r) + m
+        epilogue: o / r  (or o / (r + c), c a constant of at most 1e-20)  and  lse = log(r) + m
 
     Every use of m_new must be one of these.  Then m_new may lag behind the true maximum
     (thresholded update, see codegen/hip_gen.py) without changing o or lse.  Anything else: None.
@@ -275,8 +275,18 @@ def find_lazy_softmax(online_func, rowscales, new_scores, new_rowscales, o_scale
         acc = _SA("acc_o", Var("acc_o"), shape_idx=["block_M", "dimv"])
         dummy = SymbolScalar("b", Var("b"), shape_idx=[])
         o_new, finals = online_func.online_fwd_epilogue(acc, rowscales, dummy, dummy, dummy)
-        if not (o_new.code.type == "Div" and o_new.prev[0] is acc and o_new.prev[1] is r):
+        if not (o_new.code.type == "Div" and o_new.prev[0] is acc):
             return None
+        den = o_new.prev[1]
+        if den is not r:
+            # o / (r + c) with a constant 0 <= c <= 1e-20, the guard of attn_script/sparseattn.py:68 ("to avoid division
+            # by zero").  A row with a visible key has r >= 1 whatever the (lagging) reference -- its largest score
+            # contributes exp(0) or more --, so r + c == r in fp32; a row without one has o = 0 and gives 0 either way.
+            if den.code.type != "Add" or len(den.prev) != 2:
+                return None
+            rr, cc = den.prev if den.prev[0] is r else den.prev[::-1]
+            if rr is not r or cc.code.type != "Const" or not 0.0 <= float(cc.code.value) <= 1e-20:
+                return None
         if len(finals) != 1:
             return None
         (lse,) = finals.values()

@@ -325,6 +325,30 @@ def test_softmax_specialisation_needs_the_exact_graph():
             PrefillBwdOp(op, sm, near_miss, CustomIO({}))
 
 
+def test_softmax_proof_takes_the_guarded_division_of_the_sparse_attention_script():
+    """attn_script/sparseattn.py:66-72 divides by r + 1e-30.  A row with a visible key has r >= 1 whatever the lagging
+    reference, so a constant of at most 1e-20 leaves r unchanged in fp32 and the graph is still the online softmax;
+    a constant that can change r (or anything else in the denominator) is not."""
+    sm = C.make_scale_score_mod(0.125)
+
+    def guarded(c, wrong_side=False):
+        class Guarded(C.OnlineSoftmax):
+            @staticmethod
+            def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+                r = online_rowscales["r"]
+                den = (c + r) if wrong_side else (r + c)
+                return o / den, {"lse": r.log() + online_rowscales["m"]}
+        return Guarded()
+    for c in (1e-30, 1e-20, 0.0):
+        assert L.trace_functors(sm, None, guarded(c), CustomIO({}), torch.float16).softmax == (0.125, "m", "r"), c
+    assert L.trace_functors(sm, None, guarded(1e-30, wrong_side=True), CustomIO({}), torch.float16).softmax is not None
+    for c in (1e-6, 1.0, -1e-30):
+        lf = L.trace_functors(sm, None, guarded(c), CustomIO({}), torch.float16)
+        assert lf.softmax is None and "5.545" not in lf.online_fwd_body, c      # neither specialised nor lazy
+    src = L.render_functors(L.trace_functors(sm, None, guarded(1e-30), CustomIO({}), torch.float16))
+    assert "1e-30" in src or "1.0e-30" in src or "9.99999" in src        # the user's epilogue runs as written
+
+
 def test_shapes_broadcast_by_name():
     q = SymbolScalar("q_idx", Var("q_idx"), shape_idx=["block_M"])
     kv = SymbolScalar("kv_idx", Var("kv_idx"), shape_idx=["block_N"])

@@ -915,3 +915,103 @@ def test_tune_measures_at_the_first_call_and_records(cuda_device, tmp_path):
     out2, dq2 = run(second)
     assert second.attention.tune_times is None and second.attention.backward_op().dq_rows == bwd.dq_rows
     assert torch.equal(out1, out2) and torch.equal(dq1, dq2)
+
+
+class _OnlineSoftmaxGuardedDivision(C.OnlineSoftmax):
+    """The online softmax as attn_script/sparseattn.py:28-77 writes it: the epilogue divides by r + 1e-30 "to avoid
+    division by zero".  The lowering still takes the graph for the online softmax (r >= 1 for a row with a visible
+    key, so the guard changes nothing in fp32) and runs the user's epilogue as written."""
+
+    @staticmethod
+    def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+        o_new = o / (online_rowscales["r"] + 1e-30)
+        lse = (online_rowscales["r"]).log() + online_rowscales["m"]
+        return o_new, {"lse": lse}
+
+
+@pytest.mark.gpu
+def test_sliding_window_script(cuda_device):
+    """attn_script/sparseattn.py:87-170 at its own head count and sequence length (batch 2 of its 4): a causal sliding
+    window of 256 written with torch.logical_and, infer_mask=True (the window becomes a tile table plus the
+    elementwise test on its edges), bf16, and the script's own online function with the guarded division.  Against
+    the oracle with the dense window mask; the script prints its difference against a per-row loop."""
+    B, H, S, D, dtype = 2, 32, 2048, 128, torch.bfloat16
+    window = 256
+
+    def block_sparse_mask(b, h, q_idx, kv_idx):
+        return torch.logical_and(q_idx >= kv_idx, q_idx < kv_idx + window)
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=21)
+    meta = (meta_tensor(B, H, S, D, dtype=dtype),) * 3
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)),
+                          mask_mod=block_sparse_mask, online_func=_OnlineSoftmaxGuardedDivision(), infer_mask=True)
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    lse = mod.final_rowscales["lse"]
+    dense = torch.from_numpy(M.dense_mask_grid(block_sparse_mask, 1, 1, S, S))
+    ref, ref_lse = R.softmax_attention(q, k, v, mask=dense)
+    assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
+    assert (lse.cpu() - ref_lse).abs().max().item() <= 1e-3
+    assert mod._op.functors.softmax is not None          # the guarded form is still proven to be the online softmax
+    # the same graph with the plain division must agree
+    plain = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)),
+                            mask_mod=block_sparse_mask, online_func=C.OnlineSoftmax(), infer_mask=True)
+    out2 = plain(q.cuda(), k.cuda(), v.cuda())
+    assert (out2.float() - out.float()).abs().max().item() <= 2e-2
+
+
+class _OnlineSoftmaxRawMaximum(C.OnlineSoftmax):
+    """The online softmax as attn_script/mha_cute.py:29-85 writes it: score_mod is the identity, the running maximum is
+    kept on the RAW scores and the scale sits inside exp2, ((s - m) * c * log2 e).exp2(); lse = log r + m * c."""
+    scale = 0.125
+    k = 0.125 * math.log2(math.e)
+
+    @staticmethod
+    def online_fwd(scores, online_rowscales, b, h, q_idx):
+        k = _OnlineSoftmaxRawMaximum.k
+        m, r = online_rowscales["m"], online_rowscales["r"]
+        m_new = m.max(scores.get_reduce("max"))
+        scale_tmp = ((m - m_new) * k).exp2()
+        r = r * scale_tmp
+        scores = ((scores - m_new) * k).exp2()
+        r = r + scores.get_reduce("sum")
+        return scores, {"m": m_new, "r": r}, scale_tmp
+
+    @staticmethod
+    def online_fwd_epilogue(o, online_rowscales, b, h, q_idx):
+        o_new = o / online_rowscales["r"]
+        lse = (online_rowscales["r"]).log() + online_rowscales["m"] * _OnlineSoftmaxRawMaximum.scale
+        return o_new, {"lse": lse}
+
+    @staticmethod
+    def forward(scores, final_rowscales, b, h, q_idx, kv_idx):
+        return (scores * _OnlineSoftmaxRawMaximum.scale - final_rowscales["lse"]).exp()
+
+    @staticmethod
+    def backward(dp, scores, final_rowscales, doosum_rowscales, b, h, q_idx, kv_idx):
+        return (dp - doosum_rowscales) * scores
+
+
+@pytest.mark.gpu
+def test_softmax_written_with_the_scale_inside_exp2(cuda_device):
+    """attn_script/mha_cute.py at its own shape (B1 H12 S2048 D64 bf16, causal): the scale is not in score_mod but
+    inside the online function, and the exported lse is log r + m * scale.  Forward (out, lse) against the oracle.
+    The script's backward() rule, (dp - doosum) * p, is the gradient with respect to the SCALED score; the reference's
+    CuTe kernels multiply dq and dk by their own softmax_scale argument (cute_template/flash_attn_interface.py:216-233,
+    default head_dim ** -0.5), which has no counterpart here: the rule is traced as written, so dv is the oracle's and
+    dq, dk are the oracle's divided by the scale."""
+    B, H, S, D, dtype = 1, 12, 2048, 64, torch.bfloat16
+    q, k, v = C.make_inputs(B, S, S, H, H, D, D, dtype, seed=5)
+    do = torch.randn(B, S, H, D, generator=torch.Generator().manual_seed(6)).to(dtype)
+    meta = (meta_tensor(B, H, S, D, dtype=dtype),) * 3
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=lambda score, custom, b, h, q_idx, kv_idx: score,
+                          mask_mod=C.causal_mask, online_func=_OnlineSoftmaxRawMaximum(), backend="cute")
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = mod(qd, kd, vd)
+    ref, ref_lse = R.softmax_attention(q, k, v, scale=0.125, causal=True)
+    assert (out.detach().float().cpu() - ref).abs().max().item() <= 2e-2
+    assert (mod.final_rowscales["lse"].cpu() - ref_lse).abs().max().item() <= 1e-3
+    out.backward(do.cuda())
+    dq, dk, dv = R.softmax_attention_grads(q, k, v, do, scale=0.125, causal=True)
+    for got, want, name in ((qd.grad.float().cpu() * 0.125, dq, "dq"), (kd.grad.float().cpu() * 0.125, dk, "dk"),
+                            (vd.grad.float().cpu(), dv, "dv")):
+        tol = 2e-2 + 1e-2 * want.abs().max().item()
+        assert (got - want).abs().max().item() <= tol, name
