@@ -1015,3 +1015,33 @@ def test_softmax_written_with_the_scale_inside_exp2(cuda_device):
                             (vd.grad.float().cpu(), dv, "dv")):
         tol = 2e-2 + 1e-2 * want.abs().max().item()
         assert (got - want).abs().max().item() <= tol, name
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,Hkv,S,D,dtype,causal", [
+    (2, 2, 65536, 128, torch.float16, True),
+    (4, 1, 100003, 64, torch.bfloat16, False),      # grouped heads, a ragged last tile 1563 tiles away
+])
+def test_very_long_sequences(cuda_device, H, Hkv, S, D, dtype, causal):
+    """Sequences far beyond the benchmark's (1024 and more kv tiles, row offsets beyond 2^24 elements): the first,
+    the middle and the last 64 query rows against softmax / logsumexp over all keys in fp32."""
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(1, S, H, D, generator=g).to(dtype)
+    k = torch.randn(1, S, Hkv, D, generator=g).to(dtype)
+    v = torch.randn(1, S, Hkv, D, generator=g).to(dtype)
+    meta = (meta_tensor(1, H, S, D, dtype=dtype), meta_tensor(1, Hkv, S, D, dtype=dtype), meta_tensor(1, Hkv, S, D, dtype=dtype))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)),
+                          mask_mod=C.causal_mask if causal else None, online_func=C.OnlineSoftmax())
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    lse = mod.final_rowscales["lse"]
+    kk = k[0].float().repeat_interleave(H // Hkv, dim=1)
+    vv = v[0].float().repeat_interleave(H // Hkv, dim=1)
+    for r0 in (0, S // 2 - 31, S - 64):
+        rows = slice(r0, r0 + 64)
+        s = torch.einsum("qhd,khd->hqk", q[0, rows].float(), kk) / math.sqrt(D)
+        if causal:
+            vis = torch.arange(r0, r0 + 64)[:, None] >= torch.arange(S)[None, :]
+            s = s.masked_fill(~vis[None], float("-inf"))
+        ref = torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), vv)
+        assert (out[0, rows].float().cpu() - ref).abs().max().item() <= 2e-2, r0
+        assert (lse[0, :, rows].cpu() - torch.logsumexp(s, -1)).abs().max().item() <= 1e-3, r0
