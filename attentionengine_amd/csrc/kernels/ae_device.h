@@ -156,14 +156,21 @@ AE_DEV float ae_swap32_lo_hi(float v, float& hi) {
   hi = __builtin_bit_cast(float, (unsigned)r[1]);
   return __builtin_bit_cast(float, (unsigned)r[0]);
 }
-AE_DEV float ae_xor16(float v) {
-  int lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-  int r = __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, v));
-  return __builtin_bit_cast(float, r);
+// the values of the even and of the odd 16-lane row of a lane's row pair (v_permlane16_swap with both operands
+// equal): an exchange inside the VALU, where ds_bpermute goes through the LDS pipeline and back
+AE_DEV float ae_swap16_even_odd(float v, float& odd) {
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  odd = __builtin_bit_cast(float, (unsigned)r[1]);
+  return __builtin_bit_cast(float, (unsigned)r[0]);
 }
 AE_DEV float ae_group_max(float v) {
 #if AE_LAYOUT == 1
-  v = __builtin_fmaxf(v, ae_xor16(v));
+  {
+    float od;
+    const float ev = ae_swap16_even_odd(v, od);
+    v = __builtin_fmaxf(ev, od);
+  }
 #endif
   float hi;
   float lo = ae_swap32_lo_hi(v, hi);
@@ -171,7 +178,11 @@ AE_DEV float ae_group_max(float v) {
 }
 AE_DEV float ae_group_sum(float v) {
 #if AE_LAYOUT == 1
-  v = v + ae_xor16(v);
+  {
+    float od;
+    const float ev = ae_swap16_even_odd(v, od);
+    v = ev + od;
+  }
 #endif
   float hi;
   float lo = ae_swap32_lo_hi(v, hi);
