@@ -143,6 +143,9 @@ _lib = None
 _lib_lock = threading.Lock()
 
 
+AE_ABI_VERSION = 6      # AE_ABI_VERSION of include/ae_hip.h
+
+
 def lib():
     """Load libae_hip.so once; raise if it has not been built (no fallback)."""
     global _lib
@@ -158,6 +161,10 @@ def lib():
                     fn = getattr(handle, name)
                     fn.restype = res
                     fn.argtypes = args
+                if handle.ae_abi_version() != AE_ABI_VERSION:
+                    # (a library built from another header: its structures may be laid out differently)
+                    raise AEError(f"{LIB_PATH} has C ABI version {handle.ae_abi_version()}, this binding is written for "
+                                  f"{AE_ABI_VERSION}: rebuild it (python -c 'import __graft_entry__ as g; g.build()')")
                 _lib = handle
     return _lib
 

@@ -420,12 +420,21 @@ static int decode_fwd_impl(ae_kernel* split, ae_kernel* combine, const ae_attn_p
   // head tile) merges its waves' partial results itself and writes out; no combine kernel, no work buffers.
   // The host cannot see how a kernel was compiled, so the flag travels with the tile configuration: a kernel
   // built WITHOUT the merge stores its partials through p->partial_o and must never run with NULL buffers.
-  if (cfg->merge_in_wg != 0 && cfg->merge_in_wg != 1)
+  if (cfg->merge_in_wg < 0 || cfg->merge_in_wg > 2)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: merge_in_wg=%d", cfg->merge_in_wg);
-  const bool merged = cfg->merge_in_wg == 1;
+  // (2: built with AE_MERGE_LAST 1 - the workgroup that finishes last merges; it needs the work buffers, whose
+  // row-scale buffer ends with the arrival counters, but no combine kernel)
+  const bool merge_last = cfg->merge_in_wg == 2;
+  if (merge_last) {
+    if (combine)
+      return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel whose last workgroup merges takes no combine kernel");
+    if (!p->partial_o || !p->partial_rs)
+      return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
+  }
+  const bool merged = cfg->merge_in_wg == 1 || merge_last;
   if (merged && combine)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel that merges in the workgroup takes no combine kernel");
-  if (merged && p->num_splits != waves)
+  if (merged && !merge_last && p->num_splits != waves)
     return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel that merges in the workgroup needs the %d splits to be "
                 "the %d waves of one workgroup", p->num_splits, waves);
   if (!merged && !combine)

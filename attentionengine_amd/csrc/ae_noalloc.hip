@@ -67,6 +67,11 @@ extern "C" int ae_decode_fwd_noalloc(ae_kernel* split, ae_kernel* combine, const
   if (p->batch <= 0 || p->heads_q <= 0 || p->num_splits <= 0 || cfg->head_dim_v <= 0 || cfg->n_rowscales < 0)
     return ae_internal_fail(AE_ERR_INVALID_ARG, "ae_decode_fwd_noalloc: bad extents (B=%d Hq=%d splits=%d DV=%d)",
                             p->batch, p->heads_q, p->num_splits, cfg->head_dim_v);
+  // a kernel whose last workgroup merges counts arrivals in counters that must read zero when it starts; the
+  // built-in buffer keeps whatever the last call left and is not cleared here
+  if (cfg->merge_in_wg == 2)
+    return ae_internal_fail(AE_ERR_INVALID_ARG, "ae_decode_fwd_noalloc: a split kernel whose last workgroup merges "
+                            "(merge_in_wg=2) needs zeroed arrival counters: launch it through ae_decode_fwd");
   // layout inside the array: partial_o fp32 [B,Hq,splits,DV], then (256-byte aligned) partial_rs fp32
   // [max(1, n_rowscales),B,Hq,splits] -- the shapes ae_decode_fwd documents for the caller's buffers
   const uint64_t rows = (uint64_t)p->batch * (uint64_t)p->heads_q * (uint64_t)p->num_splits;

@@ -46,6 +46,18 @@
 #ifndef AE_MERGE_IN_WG
 #define AE_MERGE_IN_WG 0
 #endif
+// 1: launches that share the kv axis of a (batch, kv head, head tile) out over SEVERAL workgroups merge in the
+// workgroup that finishes last instead of in a second launch: every workgroup writes its partial results with
+// device-scope stores, waits for them, then counts itself in with an atomic add on a counter of its (batch, kv head,
+// head tile); the one that reads gridDim.x - 1 is the last, sets the counter back to zero for the next launch, and
+// merges all AE_NSPLIT partial results in the order of ae_decode_combine_kernel (equal results to the last bit).  The
+// counters are 32-bit integers behind the row scales in p.partial_rs (after max(1, AE_N_ROWSCALES) * batch * heads_q *
+// num_splits floats), one per (batch, blockIdx.y); they must be zero before the first launch and are left at zero by
+// every launch.  Saves the second launch and the gap in front of it: 2 to 4 us of a 20 us call at batch 1.
+#ifndef AE_MERGE_LAST
+#define AE_MERGE_LAST 0
+#endif
+static_assert(!(AE_MERGE_IN_WG && AE_MERGE_LAST), "one way to merge");
 static_assert(!AE_MERGE_IN_WG || AE_NSPLIT == AE_NWAVES, "the workgroup merges exactly its own waves' partial results");
 static_assert(AE_D % 32 == 0, "head dim must be a multiple of 32");
 static_assert(AE_DV % 16 == 0, "value head dim must be a multiple of 16");
@@ -291,6 +303,98 @@ void ae_decode_split_kernel(const ae_attn_params p) {
     return;
   }
 #endif
+#if AE_MERGE_LAST
+  // The partial results of the tile's heads, as one buffer for device-scope accesses (sc1: stores are written
+  // through this XCD's L2, loads do not take a line the L2 may still hold from an earlier launch -- the merging
+  // workgroup may sit on another XCD.  A device-scope release / acquire fence pair instead writes back and
+  // invalidates the whole L2: measured at several microseconds a workgroup, twice the call at batch 4).
+  constexpr int kDeviceScope = 16;     // the sc1 bit of a buffer instruction's cache policy
+  const int tile_heads = group - ht * 16 < 16 ? group - ht * 16 : 16;
+  const int64_t tile_row0 = ((int64_t)b * p.heads_q + hk * group + ht * 16) * p.num_splits;
+  __amdgpu_buffer_rsrc_t po_buf = __builtin_amdgcn_make_buffer_rsrc(
+      p.partial_o + tile_row0 * AE_DV, 0, tile_heads * p.num_splits * AE_DV * 4, 0x00020000);
+  if (head_ok) {
+    const int row_in_tile = l16 * p.num_splits + split;
+#pragma unroll
+    for (int db = 0; db < AE_NDB; db++) {
+      ae_f32x4 w = {o[db * 4 + 0], o[db * 4 + 1], o[db * 4 + 2], o[db * 4 + 3]};
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(ae_u32x4, w), po_buf,
+                                             (row_in_tile * AE_DV + db * 16 + g4 * 4) * 4, 0, kDeviceScope);
+    }
+    if (g4 == 0) {
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+        __hip_atomic_store(p.partial_rs + (int64_t)i * p.batch * p.heads_q * p.num_splits + tile_row0 + row_in_tile,
+                           frs[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  {
+    // the barrier waits for every wave's stores above to be acknowledged (its workgroup-scope release is an
+    // s_waitcnt vmcnt(0), and stores count in vmcnt); then the workgroup counts itself in
+    __syncthreads();                   // (every wave is also past its last tile: the V tile regions are free)
+    __attribute__((address_space(3))) int* flag = (__attribute__((address_space(3))) int*)ae_smem;
+    if (tid == 0) {
+      int* counter = (int*)(p.partial_rs + (int64_t)(AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1) * p.batch * p.heads_q *
+                                               p.num_splits) + (blockIdx.z * gridDim.y + blockIdx.y);
+      const int seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = seen == (int)gridDim.x - 1;
+      // (nobody else touches the counter until the next launch)
+      if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *flag = last;
+    }
+    __syncthreads();
+    if (*flag == 0) return;
+    // Every other workgroup's partial results were in memory before it counted itself in.  One thread merges four
+    // neighbouring output columns of one head; its loads of the row scales (the same addresses for the 32 threads
+    // of a head) and of the first partial results go out together: one trip to memory, not one after the other.
+    for (int idx = tid; idx < tile_heads * (AE_DV / 4); idx += AE_NT) {
+      const int hl = idx / (AE_DV / 4), dv = (idx % (AE_DV / 4)) * 4;
+      const int hq2 = hk * group + ht * 16 + hl;
+      float rs[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1][AE_NSPLIT];
+#pragma unroll
+      for (int i = 0; i < AE_N_ROWSCALES; i++)
+#pragma unroll
+        for (int k = 0; k < AE_NSPLIT; k++)
+          rs[i][k] = __hip_atomic_load(p.partial_rs + (int64_t)i * p.batch * p.heads_q * p.num_splits + tile_row0 +
+                                           hl * AE_NSPLIT + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      constexpr int G = AE_NSPLIT < 16 ? AE_NSPLIT : 16;     // partial results in flight at a time
+      ae_f32x4 val[G];
+#pragma unroll
+      for (int i = 0; i < G; i++)
+        val[i] = __builtin_bit_cast(ae_f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  po_buf, ((hl * AE_NSPLIT + i) * AE_DV + dv) * 4, 0, kDeviceScope));
+      float w[AE_NSPLIT];
+      float merged[AE_N_ROWSCALES > 0 ? AE_N_ROWSCALES : 1];
+      ae_combine(rs, w, merged);
+      // (the sum runs over the splits in ascending order, as in ae_decode_combine_kernel: equal to the last bit)
+      ae_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k0 = 0; k0 < AE_NSPLIT; k0 += G) {
+        if (k0 > 0) {
+#pragma unroll
+          for (int i = 0; i < G; i++)
+            if (k0 + i < AE_NSPLIT)
+              val[i] = __builtin_bit_cast(ae_f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                        po_buf, ((hl * AE_NSPLIT + k0 + i) * AE_DV + dv) * 4, 0, kDeviceScope));
+        }
+#pragma unroll
+        for (int i = 0; i < G; i++)
+          if (k0 + i < AE_NSPLIT) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += val[i][r] * w[k0 + i];
+          }
+      }
+      ae_elem* orow = (ae_elem*)p.out + (int64_t)b * p.o_stride_b + (int64_t)hq2 * p.o_stride_h + dv;
+#pragma unroll
+      for (int r = 0; r < 4; r++) orow[r] = (ae_elem)acc[r];
+      if (dv == 0) {
+#pragma unroll
+        for (int i = 0; i < AE_N_ROWSCALES; i++)
+          if (p.rowscale_out[i]) p.rowscale_out[i][(int64_t)b * p.heads_q + hq2] = merged[i];
+      }
+    }
+  }
+#else
   if (head_ok) {
     const int64_t row = ((int64_t)b * p.heads_q + hq) * p.num_splits + split;
     float* po = p.partial_o + row * AE_DV;
@@ -305,6 +409,7 @@ void ae_decode_split_kernel(const ae_attn_params p) {
         p.partial_rs[(int64_t)i * p.batch * p.heads_q * p.num_splits + row] = frs[i];
     }
   }
+#endif
 }
 
 #include "ae_combine.h"

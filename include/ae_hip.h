@@ -52,7 +52,7 @@ using __hip_internal::uint64_t;
 extern "C" {
 #endif
 
-#define AE_ABI_VERSION 5
+#define AE_ABI_VERSION 6
 
 typedef enum ae_status {
   AE_OK = 0,
@@ -134,7 +134,9 @@ typedef struct ae_tile_cfg {
   int32_t paged;       /* MLA decode: 1 when the kernel reads KV through block_table / seqlens_k */
   int32_t merge_in_wg; /* GQA decode: 1 when the split kernel was compiled with AE_MERGE_IN_WG 1 (its one
                           workgroup per (batch, kv head, head tile) merges its waves' partial results and
-                          writes out itself: no combine kernel, no work buffers), else 0                   */
+                          writes out itself: no combine kernel, no work buffers); 2 when it was compiled with
+                          AE_MERGE_LAST 1 (the workgroup that finishes last merges: no combine kernel, work
+                          buffers with arrival counters, see ae_decode_fwd); else 0                        */
   int32_t table_rows;  /* mask_mode 2: block-mask rows one q tile may span, the AE_TT_ROWS the kernel was
                           compiled with (1, 2, 4 or 8); 0 stands for the kernels' default of 8             */
 } ae_tile_cfg;
@@ -256,8 +258,14 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
  *   splits the combine kernel was compiled for and must equal num_splits.  A split kernel compiled with
  *   AE_MERGE_IN_WG 1 is announced by cfg->merge_in_wg = 1: num_splits must then equal the waves of one
  *   workgroup, `combine` must be NULL (that workgroup merges its waves' partial results itself and writes
- *   out: one launch, no work buffers).  With cfg->merge_in_wg = 0 the combine kernel, its configuration and
- *   both work buffers are required; a launch that lacks any of them is refused, nothing runs.
+ *   out: one launch, no work buffers).  A split kernel compiled with AE_MERGE_LAST 1 is announced by
+ *   cfg->merge_in_wg = 2: `combine` must be NULL and both work buffers are required; the workgroup of a (batch,
+ *   kv head, head tile) that finishes last merges all partial results and writes out (one launch).  Its arrival
+ *   counters are 32-bit integers BEHIND the row scales in partial_rs -- after max(1, n_rowscales) * batch * heads_q *
+ *   num_splits floats, batch * ceil(Hq/Hkv / block_m) * Hkv of them -- which must be zero before the first launch
+ *   and which every launch leaves at zero; launches that share these buffers must not overlap.  With
+ *   cfg->merge_in_wg = 0 the combine kernel, its configuration and both work buffers are required; a launch that
+ *   lacks any of them is refused, nothing runs.
  */
 int ae_prefill_fwd(ae_kernel* k, const ae_attn_params* p, const ae_tile_cfg* cfg, void* stream);
 int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
@@ -318,7 +326,9 @@ int ae_prefill_bwd(ae_kernel* delta, ae_kernel* dkv, ae_kernel* dq, const ae_att
  *   fit returns AE_ERR_INVALID_ARG and launches nothing.  All calls on one GPU share that GPU's buffer:
  *   calls that may overlap in time on one GPU (different streams, different threads) race -- serialise
  *   them, or use ae_decode_fwd with separate buffers.  Nothing in the buffer has to be cleared between
- *   calls (every partial that is read has been written by the same call).
+ *   calls (every partial that is read has been written by the same call); for that reason a split kernel
+ *   whose last workgroup merges (cfg->merge_in_wg == 2, which needs arrival counters that read zero) is
+ *   refused here.
  */
 #define AE_NOALLOC_SCRATCH_BYTES (16u << 20)
 int ae_decode_fwd_noalloc(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,

@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported_and_bound():
     for n in names:
         assert hasattr(lib, n), f"{n} declared in ae_hip.h but not exported"
     assert sorted(rt.EXPORTED_SYMBOLS) == names
-    assert rt.lib().ae_abi_version() == 5
+    assert rt.lib().ae_abi_version() == 6
 
 
 def test_struct_layout_matches_the_header():
@@ -233,6 +233,14 @@ def test_decode_merge_form_is_checked_before_any_launch():
         assert rc == 1 and "merge_in_wg=7" in msg, msg
         rc, msg = run(entry, params(), cfg(merge_in_wg=1, n_rowscales=1), None)
         assert rc == 1 and "rowscale_out[0] is NULL" in msg, msg
+    # the last workgroup merges (2): no combine kernel, but both work buffers (partial results, arrival counters)
+    rc, msg = run(lib.ae_decode_fwd, params(num_splits=16, kv_per_split=32, partial_o=addr, partial_rs=addr),
+                  cfg(merge_in_wg=2), fake)
+    assert rc == 1 and "takes no combine kernel" in msg, msg
+    rc, msg = run(lib.ae_decode_fwd, params(num_splits=16, kv_per_split=32), cfg(merge_in_wg=2), None)
+    assert rc == 1 and "work buffers are NULL" in msg, msg
+    rc, msg = run(lib.ae_decode_fwd_noalloc, params(num_splits=16, kv_per_split=32), cfg(merge_in_wg=2), None)
+    assert rc == 1 and "needs zeroed arrival counters" in msg, msg
     # without the merge: both work buffers and the combine configuration are required
     rc, msg = run(lib.ae_decode_fwd, params(), cfg(), fake)
     assert rc == 1 and "work buffers are NULL" in msg, msg

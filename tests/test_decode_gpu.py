@@ -67,6 +67,72 @@ def test_gqa_decode_merged_in_the_workgroup(cuda_device, monkeypatch, B, Hq, Hkv
         assert (res["1"][1][b:b + 1].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Skv,D,dtype,kind", [
+    (1, 32, 8, 8192, 128, torch.float16, "softmax"),     # attn_script/gqa_inference.py shape: 8 workgroups a kv head
+    (2, 40, 2, 4001, 64, torch.bfloat16, "softmax"),     # two head tiles (one partly filled), ragged kv
+    (1, 16, 8, 2048, 128, torch.float16, "softmax"),     # two q heads a kv head: 14 of a tile's 16 rows are padding
+    (2, 8, 2, 3000, 128, torch.float16, "sigmoid"),      # no row scales: the partial results are summed
+])
+def test_gqa_decode_merged_by_the_last_workgroup(cuda_device, monkeypatch, B, Hq, Hkv, Skv, D, dtype, kind):
+    """Small batches spread one kv axis over several workgroups; the workgroup that counts itself in last merges
+    all partial results (one launch).  Bit for bit equal to the split launch followed by the merge kernel
+    (attn_gqa_decode_tl.py:224-266), on 300 launches that alternate between two inputs (a merge that read another
+    launch's partial results, or that ran before the last partial result was visible, would differ), and again
+    as replays of a captured HIP graph with eager work between them."""
+    print(f"case last-workgroup gqa decode B{B} Hq{Hq} Hkv{Hkv} Skv{Skv} D{D} {dtype} {kind}", flush=True)
+
+    def sig(score, custom_fwd_inputs, b, h, q_idx, kv_idx):
+        return (((score * (1 / math.sqrt(D)) - 6.0) * 0.5).tanh() + 1) * 0.5
+    score_mod, online = ((C.make_scale_score_mod(1 / math.sqrt(D)), C.OnlineSoftmax()) if kind == "softmax"
+                         else (sig, C.OnlineIdentity()))
+    inputs = [tuple(t.cuda() for t in C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, dtype, seed=s)) for s in (0, 1)]
+
+    def rowscale(mod):
+        return mod.final_rowscales["lse"].clone() if kind == "softmax" else torch.zeros(1)
+    monkeypatch.setenv("AE_DECODE_MERGE_LAST", "0")
+    two = _decode_engine(B, Hq, Hkv, Skv, D, D, dtype, score_mod, online)
+    n_split, _ = two.attention.plan_splits(B, Hq, Hkv, Skv)
+    assert n_split > two.attention.N_WAVES and two.attention._merge_mode(n_split) == 0
+    want = []
+    for q, k, v in inputs:
+        want.append((two(q, k, v).clone(), rowscale(two)))
+    assert not torch.equal(want[0][0], want[1][0])
+    monkeypatch.setenv("AE_DECODE_MERGE_LAST", "1")
+    one = _decode_engine(B, Hq, Hkv, Skv, D, D, dtype, score_mod, online)
+    assert one.attention._merge_mode(n_split) == 2
+    got = []
+    for it in range(300):
+        q, k, v = inputs[it & 1]
+        got.append((one(q, k, v), rowscale(one)))
+    torch.cuda.synchronize()
+    for it, (o, r) in enumerate(got):
+        assert torch.equal(o, want[it & 1][0]), f"launch {it}: out differs"
+        assert torch.equal(r.cpu(), want[it & 1][1].cpu()), f"launch {it}: row scale differs"
+    if kind == "softmax":
+        q, k, v = (t.cpu() for t in inputs[0])
+        ref, lse = R.softmax_attention(q, k, v, causal=False)
+        assert (want[0][0].float().cpu() - ref).abs().max().item() <= OUT_TOL
+        assert (want[0][1].cpu() - lse).abs().max().item() <= LSE_TOL
+    # under a HIP graph: the work buffers are the operator's (allocated by the first call on the stream, outside the
+    # capture), the arrival counters are back at zero after every launch
+    side = torch.cuda.Stream()
+    q, k, v = (t.clone() for t in inputs[0])
+    with torch.cuda.stream(side):
+        one(q, k, v)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out_g = one(q, k, v)
+        out_g2 = one(q, k, v)          # two launches in one graph share the buffers, one after the other
+    for rep in range(6):
+        for dst, src in zip((q, k, v), inputs[rep & 1]):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want[rep & 1][0]) and torch.equal(out_g2, want[rep & 1][0]), f"replay {rep}"
+        assert torch.equal(one(*inputs[1]), want[1][0])        # eager work between the replays
+
+
 def test_gqa_decode_full_size_properties(cuda_device):
     """BASELINE config 4 at full size (B64 Hq32 Hkv8 Skv8192 D128 fp16).  Checked against the oracle
     on two batch entries, and everywhere through linearity in V: decode(q, k, a*v1 + v2) ==

@@ -632,21 +632,63 @@ def test_decode_kernel_cache_is_keyed_by_the_merge_form(monkeypatch):
     assert n_split == op.N_WAVES
     monkeypatch.delenv("AE_DECODE_MERGE_IN_WG", raising=False)
     # the constructor compiled the merging form
-    assert set(op._variants) == {(4, False, True)}
-    merged = op._variant(n_split, False, op.merges_in_workgroup(n_split))
+    assert set(op._variants) == {(4, False, 1)}
+    merged = op._variant(n_split, False, op._merge_mode(n_split))
     assert "#define AE_MERGE_IN_WG 1" in merged[3] and merged[1].merge_in_wg == 1
     # the documented toggle: the launch without allocations keeps the merge kernel
     op.static_workspace = True
     assert not op.merges_in_workgroup(n_split)
-    plain = op._variant(n_split, False, op.merges_in_workgroup(n_split))
+    plain = op._variant(n_split, False, op._merge_mode(n_split))
     assert plain is not merged and plain[0] is not merged[0]
     assert "#define AE_MERGE_IN_WG 0" in plain[3] and plain[1].merge_in_wg == 0
     op.static_workspace = False
-    assert op._variant(n_split, False, op.merges_in_workgroup(n_split)) is merged
+    assert op._variant(n_split, False, op._merge_mode(n_split)) is merged
     # ... and the environment variable that keeps the two launches
     monkeypatch.setenv("AE_DECODE_MERGE_IN_WG", "0")
-    assert op._variant(n_split, False, op.merges_in_workgroup(n_split)) is plain
-    assert set(op._variants) == {(4, False, True), (4, False, False)}
+    assert op._variant(n_split, False, op._merge_mode(n_split)) is plain
+    assert set(op._variants) == {(4, False, 1), (4, False, 0)}
+
+
+def test_decode_splits_over_several_workgroups_merge_in_the_last_one(monkeypatch):
+    """A small batch spreads one kv axis over several workgroups; the one that finishes last merges
+    (AE_MERGE_LAST, merge_in_wg = 2) unless the launch must not keep buffers of its own (``static_workspace``)
+    or the environment asks for the two launches.  Compiled here by hipRTC, without register spills."""
+    from core.lower.lower_decode import GQADecodeOp
+    dt = torch.float16
+    B, Hq, Hkv, Skv, D = 1, 32, 8, 8192, 128
+    meta = (meta_tensor(B, Hq, 1, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt))
+    monkeypatch.delenv("AE_DECODE_MERGE_LAST", raising=False)
+    op = GQADecodeOp(meta, CustomIO({}), C.make_scale_score_mod(D ** -0.5), None, C.OnlineSoftmax(), "-inf")
+    n_split, _ = op.plan_splits(B, Hq, Hkv, Skv)
+    assert n_split > op.N_WAVES and op._merge_mode(n_split) == 2
+    assert set(op._variants) == {(n_split, True, 2)}
+    last = op._variant(n_split, True, 2)
+    assert "#define AE_MERGE_LAST 1" in last[3] and "#define AE_MERGE_IN_WG 0" in last[3] and last[1].merge_in_wg == 2
+    op.static_workspace = True
+    assert op._merge_mode(n_split) == 0
+    op.static_workspace = False
+    monkeypatch.setenv("AE_DECODE_MERGE_LAST", "0")
+    assert op._merge_mode(n_split) == 0
+    plain = op._variant(n_split, True, 0)
+    assert "#define AE_MERGE_LAST 0" in plain[3] and plain[0] is not last[0]
+
+
+def test_decode_build_that_spills_is_built_again_for_one_wave_a_simd():
+    """Value heads of 256 do not fit the 256 registers of two waves a SIMD (85 spilled registers, 2.3x the time on
+    the chip); the operator then builds the kernel for one wave a SIMD, which does not spill.  Head dims of 128
+    keep two waves."""
+    import warnings
+    from core.lower.lower_decode import GQADecodeOp
+    dt = torch.float16
+    for D, want in ((256, 1), (128, 2)):
+        B, Hq, Hkv, Skv = 64, 32, 8, 8192
+        meta = (meta_tensor(B, Hq, 1, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt), meta_tensor(B, Hkv, Skv, D, dtype=dt))
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            op = GQADecodeOp(meta, CustomIO({}), C.make_scale_score_mod(D ** -0.5), None, C.OnlineSoftmax(), "-inf")
+        (module, _, _, src), = op._variants.values()
+        assert f"#define AE_WAVES_PER_EU {want}" in src
+        assert module.kernel_info()["ae_decode_split_kernel"].get(".vgpr_spill_count", 0) == 0
 
 
 def test_numerics_keywords_of_the_constructor(monkeypatch):
