@@ -403,6 +403,11 @@ class PrefillOp:
         rowscales = [torch.empty(rs_shape, dtype=torch.float32, device=dev) for _ in range(self.n_rowscales)]
         p = rt.AttnParams()
         p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+        p.q_stride_b, p.q_stride_s, p.q_stride_h, _ = q.stride()
+        p.k_stride_b, p.k_stride_s, p.k_stride_h, _ = k.stride()
+        p.v_stride_b, p.v_stride_s, p.v_stride_h, _ = v.stride()
+        p.o_stride_b, p.o_stride_s, p.o_stride_h, _ = out.stride()
+        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = B, Hq, Hkv, Sq, Skv
         for i, r in enumerate(rowscales):
             p.rowscale_out[i] = r.data_ptr()
         keep = []
@@ -410,17 +415,12 @@ class PrefillOp:
             t = t.to(device=dev, dtype=desc.torch_dtype).contiguous()
             keep.append(t)
             p.custom[i] = t.data_ptr()
-        p.q_stride_b, p.q_stride_s, p.q_stride_h = q.stride(0), q.stride(1), q.stride(2)
-        p.k_stride_b, p.k_stride_s, p.k_stride_h = k.stride(0), k.stride(1), k.stride(2)
-        p.v_stride_b, p.v_stride_s, p.v_stride_h = v.stride(0), v.stride(1), v.stride(2)
-        p.o_stride_b, p.o_stride_s, p.o_stride_h = out.stride(0), out.stride(1), out.stride(2)
-        p.batch, p.heads_q, p.heads_kv, p.seqlen_q, p.seqlen_kv = B, Hq, Hkv, Sq, Skv
         if mode == 2:
             p.block_mask = table.data_ptr()
             p.mask_b, p.mask_h, p.mask_nq, p.mask_nkv = table.shape
             p.mask_block_m, p.mask_block_n = mbm, mbn
             keep.append(table)
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = rt.current_stream(dev)
         if n_split > 1:
             partial_o = torch.empty((B, Sq, Hq, n_split, self.DV), dtype=torch.float32, device=dev)
             partial_rs = torch.empty((max(1, self.n_rowscales), B, Sq, Hq, n_split), dtype=torch.float32, device=dev)

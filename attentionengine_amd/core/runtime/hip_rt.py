@@ -469,9 +469,32 @@ def rows_for_kernels(t):
     """``t`` as the kernels can read it: dense in the last dimension, starting on a 16-byte boundary, every
     other stride a multiple of 8 elements (rows are moved 16 bytes at a time; the C entry points refuse anything
     else).  Tensors laid out otherwise - a column slice that starts at an odd offset, say - are copied."""
-    if t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(st % 8 == 0 for st in t.stride()[:-1]):
-        return t
+    st = t.stride()
+    if st[-1] == 1 and t.data_ptr() % 16 == 0:
+        for x in st[:-1]:
+            if x % 8:
+                break
+        else:
+            return t
     return t.contiguous()
+
+
+_raw_stream = None
+
+
+def current_stream(device) -> int:
+    """The raw handle of torch's current stream on ``device`` (what ``torch.cuda.current_stream(device).cuda_stream``
+    returns, without building the Stream object: a third of the time of a small call)."""
+    global _raw_stream
+    if _raw_stream is None:
+        import torch
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        _raw_stream = raw if raw is not None else (lambda index: torch.cuda.current_stream(index).cuda_stream)
+    index = device.index
+    if index is None:
+        import torch
+        index = torch.cuda.current_device()
+    return _raw_stream(index)
 
 
 def prefill_fwd(kernel: Kernel, params: AttnParams, cfg: TileCfg, stream: int = 0):
