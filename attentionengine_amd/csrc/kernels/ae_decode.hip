@@ -412,4 +412,6 @@ void ae_decode_split_kernel(const ae_attn_params p) {
 #endif
 }
 
-#include "ae_combine.h"
+#if !(AE_MERGE_IN_WG || AE_MERGE_LAST)
+#include "ae_combine.h"      // the merge kernel of the two-launch form
+#endif

@@ -38,9 +38,15 @@ WORKLOADS = {
     "c3_sigmoid": ("c3_sigmoid", "prefill"),
     "c4_gqa_decode": ("c4_gqa_decode", "gqa_decode"),
     "c5_mla_decode": ("c5_mla_decode", "mla_decode"),
+    # not a BASELINE configuration: the decode shape of the reference's own script (attn_script/gqa_inference.py,
+    # batch 1: one launch whose last workgroup merges; the call is bound by latency, not by HBM)
+    "gqa_decode_b1": ("gqa_decode_b1", "gqa_decode"),
     # not a BASELINE configuration: the backward of c2_causal (dq, dk, dv from dout; three launches)
     "c2_causal_bwd": ("c2_softmax_causal", "prefill_bwd"),
 }
+
+
+ONLY_ON_REQUEST = {"gqa_decode_b1"}      # measured with --workload, not part of the default line's other_configs
 
 
 # HBM bytes per launch of each workload's dominant kernel, from the hardware counters FETCH_SIZE and
@@ -78,8 +84,8 @@ def _inputs(name, device):
             flops *= 2.5     # the reference's count: 4*B*H*S^2*DV + 6*B*H*S^2*D, halved (bench_utils.py:1199-1201)
         return args, {"flops": flops, "bytes": 4.0 * B * S * H * D * 2,
                       "shape": {"B": B, "H": H, "S": S, "D": D, "DV": D}, "dtype": "fp16"}
-    if name == "c4_gqa_decode":
-        B, Hq, Hkv, Skv, D = 64, 32, 8, 8192, 128
+    if name in ("c4_gqa_decode", "gqa_decode_b1"):
+        B, Hq, Hkv, Skv, D = (64 if name == "c4_gqa_decode" else 1), 32, 8, 8192, 128
         args = [rn(B, 1, Hq, D, dtype=f16), rn(B, Skv, Hkv, D, dtype=f16), rn(B, Skv, Hkv, D, dtype=f16)]
         return args, {"flops": 4.0 * B * Hq * Skv * D, "bytes": 2.0 * B * Skv * Hkv * D * 2,
                       "shape": {"B": B, "Hq": Hq, "Hkv": Hkv, "Skv": Skv, "D": D, "DV": D}, "dtype": "fp16"}
@@ -436,8 +442,8 @@ def cpu_baseline(name):
         return {"value": passes * flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
                 "sample": f"oracle/attention_ref.py on 1 of 2 batch entries (32 heads, S=4096, D=128, "
                           f"fp32), {passes} passes in {dt:.1f} s, reference flop convention"}
-    if name == "c4_gqa_decode":
-        nb, Hq, Hkv, Skv, D = 8, 32, 8, 8192, 128
+    if name in ("c4_gqa_decode", "gqa_decode_b1"):
+        nb, Hq, Hkv, Skv, D = (8 if name == "c4_gqa_decode" else 1), 32, 8, 8192, 128
         q = torch.randn(nb, 1, Hq, D, generator=g).half().float()
         k = torch.randn(nb, Skv, Hkv, D, generator=g).half().float()
         v = torch.randn(nb, Skv, Hkv, D, generator=g).half().float()
@@ -447,7 +453,8 @@ def cpu_baseline(name):
         dt = time.perf_counter() - t0
         by = 2.0 * nb * Skv * Hkv * D * 2
         return {"value": by / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-                "sample": f"oracle on 8 of 64 batch entries (fp32 compute, fp16-sized KV bytes), {dt:.2f} s"}
+                "sample": f"oracle on {nb} of {64 if name == 'c4_gqa_decode' else 1} batch entries (fp32 compute, "
+                          f"fp16-sized KV bytes), {dt:.2f} s"}
     if name == "c5_mla_decode":
         nb, H, Skv, D, DV = 8, 128, 4096, 576, 512
         q = torch.randn(nb, H, DV, generator=g).bfloat16().float()
@@ -531,7 +538,7 @@ def main():
     if not a.no_extra:
         others = {}
         for name in WORKLOADS:
-            if name == a.workload:
+            if name == a.workload or name in ONLY_ON_REQUEST:
                 continue
             r = measure(name, max(5, a.steps // 2), max(2, a.warmup // 2))
             others[name] = {"ms_per_step": r["ms_per_step"], "kernel_ms": r["kernel_ms"],
