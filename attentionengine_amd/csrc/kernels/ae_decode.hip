@@ -329,8 +329,10 @@ void ae_decode_split_kernel(const ae_attn_params p) {
     }
   }
   {
-    // the barrier waits for every wave's stores above to be acknowledged (its workgroup-scope release is an
-    // s_waitcnt vmcnt(0), and stores count in vmcnt); then the workgroup counts itself in
+    // Every wave waits until its stores above have been acknowledged (stores count in vmcnt; the barrier alone
+    // does not wait for them: a workgroup-scope release on this target orders only what the waves of one CU see),
+    // then the workgroup meets and counts itself in: no partial result is still travelling when the counter moves.
+    __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0), the other counters left alone
     __syncthreads();                   // (every wave is also past its last tile: the V tile regions are free)
     __attribute__((address_space(3))) int* flag = (__attribute__((address_space(3))) int*)ae_smem;
     if (tid == 0) {
