@@ -133,6 +133,26 @@ def test_gqa_decode_merged_by_the_last_workgroup(cuda_device, monkeypatch, B, Hq
         assert torch.equal(one(*inputs[1]), want[1][0])        # eager work between the replays
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Skv,dtype", [
+    (64, 32, 8, 777, torch.float16),       # one workgroup per (batch, kv head): merged in the workgroup
+    (2, 32, 8, 4100, torch.bfloat16),      # kv axis over several workgroups: merged by the last one
+])
+def test_gqa_decode_head_dim_256(cuda_device, B, Hq, Hkv, Skv, dtype):
+    """Head dim 256 (the kernel is built for one wave per SIMD there: at two it spills 85 registers): against the
+    oracle on every batch entry."""
+    D = 256
+    print(f"case gqa decode D256 B{B} Hq{Hq} Hkv{Hkv} Skv{Skv} {dtype}", flush=True)
+    q, k, v = C.make_inputs(B, 1, Skv, Hq, Hkv, D, D, dtype, seed=5)
+    mod = _decode_engine(B, Hq, Hkv, Skv, D, D, dtype, C.make_scale_score_mod(1 / math.sqrt(D)), C.OnlineSoftmax())
+    (module, _, _, src), = mod.attention._variants.values()
+    assert "#define AE_WAVES_PER_EU 1" in src
+    assert module.kernel_info()["ae_decode_split_kernel"].get(".vgpr_spill_count", 0) == 0
+    out = mod(q.cuda(), k.cuda(), v.cuda())
+    ref, lse = R.softmax_attention(q, k, v, causal=False)
+    assert (out.float().cpu() - ref).abs().max().item() <= OUT_TOL
+    assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
+
+
 def test_gqa_decode_full_size_properties(cuda_device):
     """BASELINE config 4 at full size (B64 Hq32 Hkv8 Skv8192 D128 fp16).  Checked against the oracle
     on two batch entries, and everywhere through linearity in V: decode(q, k, a*v1 + v2) ==
