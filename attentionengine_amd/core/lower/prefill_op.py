@@ -398,9 +398,7 @@ class PrefillOp:
         kern = module.kernel("ae_prefill_kernel")
 
         out = torch.empty((B, Sq, Hq, self.DV), dtype=self.dtype, device=dev)
-        # the merge kernel of the split-KV path writes rowscales in (batch, q position, head) order
-        rs_shape = (B, Sq, Hq) if n_split > 1 else (B, Hq, Sq)
-        rowscales = [torch.empty(rs_shape, dtype=torch.float32, device=dev) for _ in range(self.n_rowscales)]
+        rowscales = [torch.empty((B, Hq, Sq), dtype=torch.float32, device=dev) for _ in range(self.n_rowscales)]
         p = rt.AttnParams()
         p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
         p.q_stride_b, p.q_stride_s, p.q_stride_h, _ = q.stride()
@@ -431,7 +429,6 @@ class PrefillOp:
                               head_dim=self.D, head_dim_v=self.DV, elem_bytes=2,
                               n_rowscales=self.n_rowscales, mask_mode=0)
             rt.prefill_split_fwd(kern, module.kernel("ae_decode_combine_kernel"), p, cfg, ccfg, stream)
-            rowscales = [r.transpose(1, 2).contiguous() for r in rowscales]
         else:
             if self._clock_stamps():
                 n_wg = -(-Sq // self.tiles.block_m) * (-(-(B * Hq) // 8) * 8)

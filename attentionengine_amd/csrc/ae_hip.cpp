@@ -527,10 +527,10 @@ int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_par
   uint32_t block[3] = {(uint32_t)cfg->threads, 1, 1};
   rc = ae_launch(split, p, sizeof *p, grid, block, (uint32_t)cfg->lds_bytes, stream);
   if (rc) return rc;
-  // the merge kernel sees the (q position, head) pairs as the heads of a one-token decode
+  // the merge kernel sees the (q position, head) pairs as the heads of a one-token decode; seqlen_q stays, and
+  // tells it to write the merged row scales in [B, Hq, Sq] order
   ae_attn_params cp = *p;
   cp.heads_q = (int32_t)rows;
-  cp.seqlen_q = 1;
   uint32_t cgrid[3] = {(uint32_t)rows, (uint32_t)p->batch, 1};
   uint32_t cblock[3] = {(uint32_t)combine_cfg->threads, 1, 1};
   return ae_launch(combine, &cp, sizeof cp, cgrid, cblock, (uint32_t)combine_cfg->lds_bytes, stream);

@@ -55,9 +55,17 @@ void ae_decode_combine_kernel(const ae_attn_params p) {
     optr[dv] = (ae_elem)acc;
   }
   if (threadIdx.x == 0) {
+    // One-token decode: row scales [B, Hq].  Split-KV prefill (p.seqlen_q > 1: its launch hands the (q position,
+    // head) pairs over as p.heads_q = Sq * Hq "heads", h = s * Hq + head): row scales [B, Hq, Sq], the layout of
+    // the unsplit kernels.
+    int64_t at = (int64_t)b * p.heads_q + h;
+    if (p.seqlen_q > 1) {
+      const int hq = p.heads_q / p.seqlen_q;
+      at = ((int64_t)b * hq + h % hq) * p.seqlen_q + h / hq;
+    }
 #pragma unroll
     for (int i = 0; i < AE_N_ROWSCALES; i++)
-      if (p.rowscale_out[i]) p.rowscale_out[i][(int64_t)b * p.heads_q + h] = merged[i];
+      if (p.rowscale_out[i]) p.rowscale_out[i][at] = merged[i];
   }
 }
 

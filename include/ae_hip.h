@@ -278,7 +278,7 @@ int ae_decode_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
  *   num_splits runs once per (q tile, head, batch, split) on kv_per_split positions (a multiple of
  *   block_n) and writes fp32 partials ordered (batch, q position, head, split); the combine kernel then
  *   merges them with the user's combine() into `out`, which must be contiguous [B,Sq,Hq,DV], and writes
- *   the merged rowscales in (batch, q position, head) order to rowscale_out (the caller transposes).
+ *   the merged rowscales to rowscale_out as fp32 [B,Hq,Sq], the layout of ae_prefill_fwd.
  */
 int ae_prefill_split_fwd(ae_kernel* split, ae_kernel* combine, const ae_attn_params* p,
                          const ae_tile_cfg* cfg, const ae_tile_cfg* combine_cfg, void* stream);
