@@ -430,6 +430,11 @@ static int decode_fwd_impl(ae_kernel* split, ae_kernel* combine, const ae_attn_p
       return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel whose last workgroup merges takes no combine kernel");
     if (!p->partial_o || !p->partial_rs)
       return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: split-KV work buffers are NULL");
+    // (the kernel merges exactly the AE_NSPLIT partial results it was compiled for; the host cannot see that
+    // number, so it travels as it does for the merge kernel)
+    if (!combine_cfg)
+      return fail(AE_ERR_INVALID_ARG, "ae_decode_fwd: a split kernel whose last workgroup merges needs combine_cfg "
+                  "(its block_n is the number of splits the kernel was compiled for)");
   }
   const bool merged = cfg->merge_in_wg == 1 || merge_last;
   if (merged && combine)

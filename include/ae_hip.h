@@ -259,7 +259,8 @@ int ae_launch(ae_kernel* k, const void* params, size_t params_bytes,
  *   AE_MERGE_IN_WG 1 is announced by cfg->merge_in_wg = 1: num_splits must then equal the waves of one
  *   workgroup, `combine` must be NULL (that workgroup merges its waves' partial results itself and writes
  *   out: one launch, no work buffers).  A split kernel compiled with AE_MERGE_LAST 1 is announced by
- *   cfg->merge_in_wg = 2: `combine` must be NULL and both work buffers are required; the workgroup of a (batch,
+ *   cfg->merge_in_wg = 2: `combine` must be NULL, both work buffers and combine_cfg are required (block_n = the
+ *   number of splits the kernel was compiled for, which must equal num_splits); the workgroup of a (batch,
  *   kv head, head tile) that finishes last merges all partial results and writes out (one launch).  Its arrival
  *   counters are 32-bit integers BEHIND the row scales in partial_rs -- after max(1, n_rowscales) * batch * heads_q *
  *   num_splits floats, batch * ceil(Hq/Hkv / block_m) * Hkv of them -- which must be zero before the first launch

@@ -239,6 +239,9 @@ def test_decode_merge_form_is_checked_before_any_launch():
     assert rc == 1 and "takes no combine kernel" in msg, msg
     rc, msg = run(lib.ae_decode_fwd, params(num_splits=16, kv_per_split=32), cfg(merge_in_wg=2), None)
     assert rc == 1 and "work buffers are NULL" in msg, msg
+    rc, msg = run(lib.ae_decode_fwd, params(num_splits=16, kv_per_split=32, partial_o=addr, partial_rs=addr),
+                  cfg(merge_in_wg=2), None, ccfg=False)
+    assert rc == 1 and "needs combine_cfg" in msg, msg
     rc, msg = run(lib.ae_decode_fwd_noalloc, params(num_splits=16, kv_per_split=32), cfg(merge_in_wg=2), None)
     assert rc == 1 and "needs zeroed arrival counters" in msg, msg
     # without the merge: both work buffers and the combine configuration are required
