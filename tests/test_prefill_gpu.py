@@ -53,6 +53,47 @@ def test_softmax_prefill(cuda_device, B, H, S, D, dtype, causal):
     assert (mod.final_rowscales["lse"].cpu() - lse).abs().max().item() <= LSE_TOL
 
 
+@pytest.mark.parametrize("B,H,S,D,causal,splits", [
+    (2, 32, 1024, 128, True, False),      # the software-pipelined kernel, tile-class order of a causal launch
+    (1, 4, 512, 64, False, False),        # the generic kernel
+    (1, 8, 64, 128, False, True),         # few query rows against 4096 keys: split launch + merge kernel
+])
+def test_prefill_as_nodes_of_a_hip_graph(cuda_device, B, H, S, D, causal, splits):
+    """A prefill call captured into a HIP graph and replayed on changing inputs gives what the eager call gives, bit
+    for bit, on every replay (launch arguments are copied when the launch is recorded; the only buffers a call makes
+    are torch allocations, which a capture takes from its own pool), with eager work between the replays."""
+    dtype = torch.float16
+    Skv = 4096 if splits else S
+    print(f"case prefill in a graph B{B} H{H} S{S} Skv{Skv} D{D} causal={causal}", flush=True)
+    meta = (meta_tensor(B, H, S, D, dtype=dtype), meta_tensor(B, H, Skv, D, dtype=dtype),
+            meta_tensor(B, H, Skv, D, dtype=dtype))
+    mod = AttentionEngine(meta, CustomIO({}), score_mod=C.make_scale_score_mod(1 / math.sqrt(D)),
+                          mask_mod=C.causal_mask if causal else None, online_func=C.OnlineSoftmax())
+    if splits:
+        assert mod.attention.plan_splits(B, H, S, Skv)[0] > 1
+    inputs = [tuple(t.cuda() for t in C.make_inputs(B, S, Skv, H, H, D, D, dtype, seed=s)) for s in (3, 4)]
+    want = []
+    for q, k, v in inputs:
+        want.append((mod(q, k, v).clone(), mod.final_rowscales["lse"].clone()))
+    assert not torch.equal(want[0][0], want[1][0])
+    side = torch.cuda.Stream()
+    q, k, v = (t.clone() for t in inputs[0])
+    with torch.cuda.stream(side):
+        mod(q, k, v)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out_g = mod(q, k, v)
+        lse_g = mod.final_rowscales["lse"]
+    for rep in range(5):
+        for dst, src in zip((q, k, v), inputs[rep & 1]):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want[rep & 1][0]) and torch.equal(lse_g, want[rep & 1][1]), f"replay {rep}"
+        assert torch.equal(mod(*inputs[1]), want[1][0])            # eager work between the replays
+
+
 def test_softmax_headline_shape_properties(cuda_device):
     """BASELINE config 2 at full size (B2 H32 S4096 D128 fp16, causal): too big for the CPU
     oracle in a test, so it is checked through size-independent properties -- one (batch, head)
