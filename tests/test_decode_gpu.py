@@ -206,6 +206,34 @@ def _mla_engine(B, H, G, S, D, DV, dtype, scale, **kw):
                            online_func=C.OnlineSoftmax(), kv_shared=True, **kw)
 
 
+@pytest.mark.parametrize("B,S", [(2, 4096), (40, 600)])      # several splits with the merge kernel / one split
+def test_mla_decode_as_nodes_of_a_hip_graph(cuda_device, B, S):
+    """MLA decode captured into a HIP graph and replayed on changing inputs: every replay equals the eager call, bit
+    for bit, with eager work between the replays."""
+    H, D, DV, dtype = 128, 576, 512, torch.bfloat16
+    print(f"case mla decode in a graph B{B} S{S}", flush=True)
+    mod = _mla_engine(B, H, 1, S, D, DV, dtype, 1 / math.sqrt(192))
+    inputs = [tuple(t.cuda() for t in _mla_inputs(B, H, 1, S, DV, D - DV, dtype, seed=s)) for s in (11, 12)]
+    want = [(mod(*a).clone(), mod.final_rowscales["lse"].clone()) for a in inputs]
+    assert not torch.equal(want[0][0], want[1][0])
+    side = torch.cuda.Stream()
+    args = [t.clone() for t in inputs[0]]
+    with torch.cuda.stream(side):
+        mod(*args)
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out_g = mod(*args)
+        lse_g = mod.final_rowscales["lse"]
+    for rep in range(5):
+        for dst, src in zip(args, inputs[rep & 1]):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want[rep & 1][0]) and torch.equal(lse_g, want[rep & 1][1]), f"replay {rep}"
+        assert torch.equal(mod(*inputs[1]), want[1][0])
+
+
 @pytest.mark.parametrize("B,H,G,S,dtype", [
     (2, 128, 1, 512, torch.bfloat16),     # DeepSeek-V3 head layout (BASELINE config 5, short KV)
     (1, 128, 1, 4096, torch.bfloat16),    # attn_script/mla_decode.py shape, one batch entry -> many splits
